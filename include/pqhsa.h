@@ -1,0 +1,227 @@
+/*
+ * pqhsa.h — C ABI of the MI355X (gfx950) PQ-HSA single-token decode-attention kernels.
+ *
+ * Every entry point is extern "C", takes plain device pointers, sizes and a HIP stream
+ * (passed as void*), enqueues its kernels on that stream and returns without synchronising
+ * or allocating.  Return value: 0 on success, a negative PQHSA_E* code otherwise;
+ * pqhsa_last_error() gives the message of the calling thread's last failure.
+ *
+ * Fixed geometry of the path: head dim D = Dv = 128, M = 8 PQ subspaces x 16 codewords
+ * (4 bits) of 16 dims, num_lists L <= 4096, GQA group G <= 16.
+ *
+ * Device index layout, one set per stream (b, h), stream id bh = b * H + h:
+ *   codes     u32 [BH, n_cap]   nibble m of the word = code of subspace m
+ *                               (the little-endian view of the reference's [N, 4] uint8
+ *                               packing, pq_hsa/index/packing.py:6-34)
+ *   list_ids  u16 [BH, n_cap]   IVF list of each indexed key (pq_hsa/index/ivfpq.py:19-33)
+ *   norms     f32 [BH, n_cap]   key norm (pq_hsa/index/ivfpq.py:1052-1059)
+ *   coarse    f32 [BH, L, 128]  coarse centroids;  codebooks f32 [BH, 8, 16, 16]
+ *   vbar      f32 [BH, L, 128]  per-list mean value (pq_hsa/attention/kv_cache.py:688-776)
+ *   vsum      f32 [BH, L, 128], vcount f32 [BH, L]   running sums behind vbar
+ *   n_idx     i32 [B]           indexed keys per sequence (device memory)
+ * Indexed key i of a sequence is token position sink + i (insertion order); top-k indices
+ * are reported in that retrieval-local space, like the reference's
+ * (pq_hsa/attention/kv_cache.py:479-484).
+ */
+#ifndef PQHSA_H
+#define PQHSA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PQHSA_OK 0
+#define PQHSA_EINVAL (-1)   /* bad argument / unsupported shape */
+#define PQHSA_ELAUNCH (-2)  /* HIP reported a launch error */
+#define PQHSA_ENOSPC (-3)   /* workspace too small */
+
+#define PQHSA_F32 0
+#define PQHSA_BF16 1
+#define PQHSA_F16 2
+
+#define PQHSA_HEAD_DIM 128
+#define PQHSA_SUBSPACES 8
+#define PQHSA_HIST_BINS 2048
+
+/*
+ * Where the full-precision K/V rows live.  Row (b, h, pos) starts at element
+ *   contiguous (paged == 0):  b*stride_seq + h*stride_head + pos*stride_tok
+ *   paged      (paged == 1):  block_table[b*max_blocks + pos/block_size]*stride_block
+ *                             + (pos % block_size)*stride_tok + h*stride_head
+ * of k_base / v_base (strides in elements of `dtype`).  This covers both page layouts the
+ * reference reads (benchmarks/vllm_backend/paged_kv_fa.py:44-57): 5-D
+ * [2, blocks, block_size, Hkv, D] (v_base = k_base + blocks*block_size*Hkv*D) and 4-D
+ * [blocks, Hkv, block_size, 2*D] (v_base = k_base + D), and the device-side addressing of
+ * pq_paged_slot / pq_paged_row (pq_hsa/kernels/cuda/pq_fused_h20.cu:869-903).
+ */
+typedef struct pqhsa_kv_view {
+    const void *k_base;
+    const void *v_base;
+    int32_t dtype;
+    int32_t paged;
+    int64_t stride_seq;
+    int64_t stride_head;
+    int64_t stride_tok;
+    int64_t stride_block;
+    int32_t block_size;
+    int32_t max_blocks;
+    const int32_t *block_table; /* device, [B, max_blocks] */
+} pqhsa_kv_view;
+
+/* Trained index + running state of BH = B*H streams (all device pointers). */
+typedef struct pqhsa_index {
+    uint32_t *codes;
+    uint16_t *list_ids;
+    float *norms;
+    const float *coarse;
+    const float *codebooks;
+    float *vbar;
+    float *vsum;
+    float *vcount;
+    const int32_t *n_idx; /* [B] */
+    int64_t n_cap;        /* row stride of codes / list_ids / norms */
+    int32_t num_lists;
+    int32_t batch;        /* B */
+    int32_t kv_heads;     /* H */
+} pqhsa_index;
+
+/* Selection policy: k = min(max(ceil(n * fraction), 0), n) if fraction > 0
+ * (pq_hsa/attention/sparse_attention.py:1756-1783), else k = min(topk, n). */
+typedef struct pqhsa_select {
+    double fraction;
+    int32_t topk;
+    int32_t k_cap; /* row stride of topk_idx / topk_val; >= the largest k of the batch */
+} pqhsa_select;
+
+const char *pqhsa_version(void);
+const char *pqhsa_last_error(void);
+
+/*
+ * Encode key rows with a given trained index: norm, direction, nearest coarse list, residual,
+ * nearest codeword per subspace, nibble packing.  For sequence b the token positions
+ * sink + slot0[b] + j, j < count[b], of every KV head are encoded into index slots
+ * slot0[b] + j.  count_max >= max_b count[b] sizes the grid.
+ * Replaces IVFPQIndex.build_with_codebooks (pq_hsa/index/ivfpq.py:350-433) with
+ * slot0 = 0, count = n, and the encode half of IVFPQIndex.add (ivfpq.py:598-645).
+ */
+int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
+                 const int32_t *slot0, const int32_t *count, int32_t count_max, float eps,
+                 void *stream);
+
+/*
+ * Rebuild vsum / vcount / vbar from the values of all indexed keys
+ * (SparseKVCache._build_retrieval_value_summaries, pq_hsa/attention/kv_cache.py:688-728).
+ * n_max >= max_b n_idx[b].
+ */
+int pqhsa_value_summaries(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
+                          int32_t n_max, void *stream);
+
+/*
+ * One launch for the per-step index update of a decode step: encode the rows at slots
+ * slot0[b] .. slot0[b] + count[b] (as pqhsa_encode) and add their values to the list sums,
+ * counts and means (IVFPQIndex.add + SparseKVCache._append_retrieval_value_summaries,
+ * pq_hsa/index/ivfpq.py:598-645, pq_hsa/attention/kv_cache.py:730-764).  The caller bumps
+ * n_idx afterwards.
+ */
+int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
+                        const int32_t *slot0, const int32_t *count, int32_t count_max,
+                        float eps, void *stream);
+
+/*
+ * Query -> lookup tables for the G query rows of every stream:
+ *   qnorm       f32 [BH, Gp]          |q|, clamped at eps
+ *   lut         f32 [BH, 8, 16, Gp]   <q_hat_m, codebook[m, c]>
+ *   list_scores f32 [BH, L, Gp]       <q_hat, coarse[l]>
+ * Gp = G rounded up to a power of two (pqhsa_padded_groups); padding rows are zero.
+ * q is [B, H*G, 128] of q_dtype, query head h*G + g belongs to KV head h.
+ * Replaces _project_query + ProductQuantizer.compute_lut + _coarse_score_bias
+ * (pq_hsa/index/ivfpq.py:1061-1070, 1179-1190; pq_hsa/index/pq.py:190-217) and the
+ * reference binding pq_lut_prep (pq_hsa/kernels/cuda/pq_fused_h20.cu:2974-3051).
+ */
+int32_t pqhsa_padded_groups(int32_t G);
+int pqhsa_lut_build(const void *q, int32_t q_dtype, const pqhsa_index *index, int32_t G,
+                    float eps, float *qnorm, float *lut, float *list_scores, void *stream);
+
+/*
+ * Fused LUT scan: approximate logit of every indexed key for every query row,
+ *   logit = ((((sum_m lut[m, code_m]) + list_scores[list]) * qnorm) * knorm) * scale
+ * with the adds in subspace order (pq_hsa/kernels/lut_scan.py:92-114,
+ * pq_hsa/index/ivfpq.py:1084-1118, pq_hsa/attention/sparse_attention.py:646).
+ * logits is f32 [BH, G, logit_stride].  n_max >= max_b n_idx[b].
+ */
+int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max, const float *qnorm,
+                   const float *lut, const float *list_scores, float scale, float *logits,
+                   int64_t logit_stride, void *stream);
+
+/*
+ * Exact top-k of each row of a logit matrix [rows, stride] by radix selection on the fp32
+ * bit pattern (no sort); ties at the k boundary go to the lowest index; the k winners are
+ * written in ascending index order with their logits.  n[r] and k[r] are per-row device
+ * arrays.  Replaces torch.topk in the reference path
+ * (pq_hsa/attention/sparse_attention.py:661-666) and the binding pq_topk_radix
+ * (pq_hsa/kernels/cuda/pq_fused_h20.cu:3624-3688).
+ */
+size_t pqhsa_topk_workspace_bytes(int32_t rows, int64_t n_max);
+int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t rows, const int32_t *n,
+                     const int32_t *k, int64_t n_max, int32_t *topk_idx, float *topk_val,
+                     int32_t k_cap, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The whole single-token decode attention of one layer, for every sequence of the batch:
+ * LUT build -> scan + histogram -> threshold -> scan + select + per-list mass -> exact
+ * attention over sink, local window and the selected keys read in place from `kv`, merged
+ * with the per-list background (list mass x list mean value) in one softmax.
+ *   q, out     [B, H*G, 128] of q_dtype
+ *   seq_lens   i32 [B] device: tokens currently in the cache of each sequence
+ *   topk_idx   i32 [BH, G, k_cap], topk_val f32 same shape, topk_cnt i32 [BH, G]: the
+ *              selected keys (retrieval-local, ascending) — optional outputs, may be NULL
+ * Replaces IVFPQSparseAttention.forward_many for mode "hybrid", value mode "centroid",
+ * top-k source "all_pq", exact rerank (pq_hsa/attention/sparse_attention.py:245-335,
+ * 759-1013), the batched GQA forward (benchmarks/e2e_pq_param_sweep.py:5026-5747) and the
+ * bindings pq_lut_prep / pq_scan_select / pq_merge_only / pq_exact_attend_paged
+ * (pq_hsa/kernels/cuda/pq_fused_h20.cu:3826-3839).
+ */
+size_t pqhsa_decode_workspace_bytes(int32_t B, int32_t H, int32_t G, int64_t n_cap,
+                                    int32_t num_lists, int32_t k_cap);
+int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                      const pqhsa_index *index, int32_t G, const int32_t *seq_lens,
+                      int32_t sink, int32_t n_max, int32_t full_max,
+                      const pqhsa_select *select, float scale, float eps, int32_t *topk_idx,
+                      float *topk_val, int32_t *topk_cnt, void *workspace,
+                      size_t workspace_bytes, void *stream);
+
+/*
+ * Hybrid exact attention alone, given the selection and the per-list masses:
+ *   list_mass f32 [BH, G, L] = sum over the list's indexed keys of exp(logit - row_max),
+ *   row_max f32 [BH, G] (the maximum approximate logit of the row).
+ * Mirrors the reference binding pq_exact_attend_paged
+ * (pq_hsa/kernels/cuda/pq_fused_h20.cu:905-1084, 3187-3205).
+ */
+size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G);
+int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *out,
+                              const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t G,
+                              const int32_t *seq_lens, int32_t sink, int32_t full_max,
+                              const int32_t *topk_idx, const float *topk_val,
+                              const int32_t *topk_cnt, int32_t k_cap, const float *list_mass,
+                              const float *row_max, float scale, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
+/*
+ * Paged-KV readers (benchmarks/vllm_backend/paged_kv_fa.py:95-156).  Both copy rows of
+ * sequence `seq` out of the paged cache into contiguous [H, count, 128] K and V tensors of
+ * the cache dtype: a token range [start, start + count), or per-head token positions
+ * positions[H, count] (i64, device).
+ */
+int pqhsa_paged_gather_range(const pqhsa_kv_view *kv, int32_t H, int32_t seq, int64_t start,
+                             int64_t count, void *out_k, void *out_v, void *stream);
+int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq,
+                          const int64_t *positions, int64_t count, void *out_k, void *out_v,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PQHSA_H */

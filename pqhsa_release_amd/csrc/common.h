@@ -1,0 +1,214 @@
+// Shared host/device helpers of the PQ-HSA gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/pqhsa.h"
+
+namespace pqhsa {
+
+constexpr int kD = PQHSA_HEAD_DIM;      // head dim of keys and values
+constexpr int kM = PQHSA_SUBSPACES;     // PQ subspaces
+constexpr int kSub = kD / kM;           // dims per subspace
+constexpr int kCodes = 16;              // codewords per subspace (4 bits)
+constexpr int kHistBits = 11;
+constexpr int kHistBins = 1 << kHistBits;
+constexpr int kWave = 64;
+
+// ---- host-side error plumbing -------------------------------------------------------
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+#define PQHSA_REQUIRE(cond, ...)            \
+    do {                                    \
+        if (!(cond)) {                      \
+            ::pqhsa::set_error(__VA_ARGS__); \
+            return PQHSA_EINVAL;            \
+        }                                   \
+    } while (0)
+
+inline int padded_groups(int G) {
+    int p = 1;
+    while (p < G) p <<= 1;
+    return p;
+}
+
+// ---- order-preserving float <-> uint32 keys --------------------------------------------
+// Larger float = larger key; -0 is folded onto +0 so that equal values have equal keys.
+__host__ __device__ inline uint32_t order_key(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if (u == 0x80000000u) u = 0u;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__host__ __device__ inline float key_to_float(uint32_t k) {
+    uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __builtin_bit_cast(float, u);
+}
+
+// ---- K/V row addressing -------------------------------------------------------------
+struct KvView {
+    const char *k_base;
+    const char *v_base;
+    int64_t stride_seq, stride_head, stride_tok, stride_block;
+    const int32_t *block_table;
+    int32_t block_size, max_blocks, paged, esize;
+};
+
+inline KvView make_view(const pqhsa_kv_view *kv) {
+    KvView v;
+    v.k_base = static_cast<const char *>(kv->k_base);
+    v.v_base = static_cast<const char *>(kv->v_base);
+    v.stride_seq = kv->stride_seq;
+    v.stride_head = kv->stride_head;
+    v.stride_tok = kv->stride_tok;
+    v.stride_block = kv->stride_block;
+    v.block_table = kv->block_table;
+    v.block_size = kv->block_size;
+    v.max_blocks = kv->max_blocks;
+    v.paged = kv->paged;
+    v.esize = kv->dtype == PQHSA_F32 ? 4 : 2;
+    return v;
+}
+
+int validate_view(const pqhsa_kv_view *kv);
+
+// element offset of row (b, h, pos)
+__device__ inline int64_t row_offset(const KvView &v, int b, int h, int64_t pos) {
+    if (v.paged) {
+        int64_t blk = pos / v.block_size;
+        int64_t row = pos - blk * v.block_size;
+        int64_t phys = v.block_table[(int64_t)b * v.max_blocks + blk];
+        return phys * v.stride_block + row * v.stride_tok + (int64_t)h * v.stride_head;
+    }
+    return (int64_t)b * v.stride_seq + (int64_t)h * v.stride_head + pos * v.stride_tok;
+}
+
+// ---- typed 8-element row slices ---------------------------------------------------------
+// Load elements [8*j, 8*j + 8) of a 128-element row as floats.
+template <int DT>
+__device__ inline void load8(const char *row, int j, float (&f)[8]);
+
+template <>
+__device__ inline void load8<PQHSA_F32>(const char *row, int j, float (&f)[8]) {
+    const float4 *p = reinterpret_cast<const float4 *>(row) + 2 * j;
+    float4 a = p[0], b = p[1];
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+    f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+template <>
+__device__ inline void load8<PQHSA_BF16>(const char *row, int j, float (&f)[8]) {
+    uint4 r = reinterpret_cast<const uint4 *>(row)[j];
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+        f[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+    }
+}
+
+template <>
+__device__ inline void load8<PQHSA_F16>(const char *row, int j, float (&f)[8]) {
+    uint4 r = reinterpret_cast<const uint4 *>(row)[j];
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        __half2 h = __builtin_bit_cast(__half2, w[i]);
+        float2 t = __half22float2(h);
+        f[2 * i] = t.x;
+        f[2 * i + 1] = t.y;
+    }
+}
+
+template <int DT>
+__device__ inline float load1(const char *row, int d);
+template <>
+__device__ inline float load1<PQHSA_F32>(const char *row, int d) {
+    return reinterpret_cast<const float *>(row)[d];
+}
+template <>
+__device__ inline float load1<PQHSA_BF16>(const char *row, int d) {
+    uint32_t w = reinterpret_cast<const uint16_t *>(row)[d];
+    return __builtin_bit_cast(float, w << 16);
+}
+template <>
+__device__ inline float load1<PQHSA_F16>(const char *row, int d) {
+    return __half2float(reinterpret_cast<const __half *>(row)[d]);
+}
+
+template <int DT>
+__device__ inline void store1(char *row, int d, float x);
+template <>
+__device__ inline void store1<PQHSA_F32>(char *row, int d, float x) {
+    reinterpret_cast<float *>(row)[d] = x;
+}
+template <>
+__device__ inline void store1<PQHSA_BF16>(char *row, int d, float x) {
+    // round to nearest even, like torch's float -> bfloat16 conversion
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    uint16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r = 0x7fc0;
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r = (uint16_t)(u >> 16);
+    }
+    reinterpret_cast<uint16_t *>(row)[d] = r;
+}
+template <>
+__device__ inline void store1<PQHSA_F16>(char *row, int d, float x) {
+    reinterpret_cast<__half *>(row)[d] = __float2half_rn(x);
+}
+
+// Dispatch a callable templated on the element type.
+#define PQHSA_DISPATCH_DTYPE(dt, ...)                                  \
+    switch (dt) {                                                      \
+        case PQHSA_F32: { constexpr int DT = PQHSA_F32; __VA_ARGS__; } break;   \
+        case PQHSA_BF16: { constexpr int DT = PQHSA_BF16; __VA_ARGS__; } break; \
+        case PQHSA_F16: { constexpr int DT = PQHSA_F16; __VA_ARGS__; } break;   \
+        default: ::pqhsa::set_error("unsupported dtype %d", (int)(dt)); return PQHSA_EINVAL; \
+    }
+
+// ---- wave64 reductions -------------------------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = (uint32_t)__shfl_xor((int)v, off, kWave);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+__device__ inline int wave_sum_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// k = min(max(ceil(n * fraction), 0), n), or min(topk, n) when no fraction is given
+__host__ __device__ inline int resolve_k(int n, double fraction, int topk) {
+    int k;
+    if (fraction > 0.0) {
+        k = (int)ceil((double)n * fraction);
+    } else {
+        k = topk;
+    }
+    if (k < 0) k = 0;
+    if (k > n) k = n;
+    return k;
+}
+
+}  // namespace pqhsa

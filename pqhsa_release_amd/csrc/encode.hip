@@ -1,0 +1,398 @@
+// Index maintenance kernels: encode key rows with a trained index (bulk build and per-step
+// append), per-list value sums / means, and the paged-KV row gathers.
+//
+// Every distance is a left-to-right chain  t = a[i] - b[i]; acc = fma(t, t, acc)  and every
+// argmin keeps the first strict minimum, so list ids and codes are bit-identical to the scalar
+// CPU oracle whichever of the two encode kernels produced them.
+#include "common.h"
+
+namespace pqhsa {
+
+constexpr int kEncThreads = 256;
+constexpr int kCoarseChunk = 32;
+
+struct EncodeArgs {
+    KvView kv;
+    int H, L, sink;
+    const int32_t *slot0;  // [B]
+    const int32_t *count;  // [B]
+    const float *coarse;   // [BH, L, 128]
+    const float *codebooks;
+    float eps;
+    uint32_t *codes;
+    uint16_t *list_ids;
+    float *norms;
+    int64_t n_cap;
+    float *vsum, *vcount, *vbar;
+    const int32_t *n_idx;
+};
+
+// One thread per key row; coarse centroids pass through LDS in chunks shared by the block.
+template <int DT>
+__global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) {
+    __shared__ __align__(16) float cs[kCoarseChunk][kD];
+    __shared__ __align__(16) float cb_s[kM * kCodes * kSub];
+    const int tid = threadIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / a.H, h = bh % a.H;
+    const int j = blockIdx.x * kEncThreads + tid;
+    const int cnt = a.count[b];
+    if ((int)(blockIdx.x * kEncThreads) >= cnt) return;
+    const bool valid = j < cnt;
+    const int slot = a.slot0[b] + j;
+    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+
+    for (int i = tid; i < kM * kCodes * kSub; i += kEncThreads) cb_s[i] = a.codebooks[(size_t)bh * kM * kCodes * kSub + i];
+
+    float x[kD];
+    float nrm = 1.0f;
+    if (valid) {
+        const char *row = a.kv.k_base + row_offset(a.kv, b, h, (int64_t)a.sink + slot) * esz;
+#pragma unroll
+        for (int c8 = 0; c8 < kD / 8; ++c8) {
+            float f[8];
+            load8<DT>(row, c8, f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[c8 * 8 + e] = f[e];
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(x[d], x[d], ss);
+        nrm = sqrtf(ss);
+        if (nrm < a.eps) nrm = a.eps;
+#pragma unroll
+        for (int d = 0; d < kD; ++d) x[d] = x[d] / nrm;
+    } else {
+#pragma unroll
+        for (int d = 0; d < kD; ++d) x[d] = 0.0f;
+    }
+
+    int best = 0;
+    float bestd = INFINITY;
+    const float *cbase = a.coarse + (size_t)bh * a.L * kD;
+    for (int l0 = 0; l0 < a.L; l0 += kCoarseChunk) {
+        const int nl = min(kCoarseChunk, a.L - l0);
+        __syncthreads();
+        for (int i = tid; i < nl * kD / 4; i += kEncThreads)
+            reinterpret_cast<float4 *>(&cs[0][0])[i] = reinterpret_cast<const float4 *>(cbase + (size_t)l0 * kD)[i];
+        __syncthreads();
+        if (valid) {
+            for (int l = 0; l < nl; ++l) {
+                float d2 = 0.0f;
+#pragma unroll
+                for (int d4 = 0; d4 < kD / 4; ++d4) {
+                    const float4 c = reinterpret_cast<const float4 *>(&cs[l][0])[d4];
+                    float t;
+                    t = x[4 * d4] - c.x; d2 = __builtin_fmaf(t, t, d2);
+                    t = x[4 * d4 + 1] - c.y; d2 = __builtin_fmaf(t, t, d2);
+                    t = x[4 * d4 + 2] - c.z; d2 = __builtin_fmaf(t, t, d2);
+                    t = x[4 * d4 + 3] - c.w; d2 = __builtin_fmaf(t, t, d2);
+                }
+                if (d2 < bestd) { bestd = d2; best = l0 + l; }
+            }
+        }
+    }
+    if (!valid) return;
+
+    const float *cbest = cbase + (size_t)best * kD;
+#pragma unroll
+    for (int d4 = 0; d4 < kD / 4; ++d4) {
+        const float4 c = reinterpret_cast<const float4 *>(cbest)[d4];
+        x[4 * d4] -= c.x; x[4 * d4 + 1] -= c.y; x[4 * d4 + 2] -= c.z; x[4 * d4 + 3] -= c.w;
+    }
+    uint32_t word = 0;
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+        int bc = 0;
+        float bd = INFINITY;
+        for (int c = 0; c < kCodes; ++c) {
+            const float *w = &cb_s[(m * kCodes + c) * kSub];
+            float d2 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < kSub; ++e) {
+                const float t = x[m * kSub + e] - w[e];
+                d2 = __builtin_fmaf(t, t, d2);
+            }
+            if (d2 < bd) { bd = d2; bc = c; }
+        }
+        word |= (uint32_t)bc << (4 * m);
+    }
+    const size_t o = (size_t)bh * a.n_cap + slot;
+    a.codes[o] = word;
+    a.list_ids[o] = (uint16_t)best;
+    a.norms[o] = nrm;
+}
+
+__device__ inline unsigned long long wave_min_u64(unsigned long long v, int width) {
+    for (int off = width / 2; off > 0; off >>= 1) {
+        const unsigned int lo = (unsigned int)__shfl_xor((int)(v & 0xffffffffull), off, width);
+        const unsigned int hi = (unsigned int)__shfl_xor((int)(v >> 32), off, width);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        v = o < v ? o : v;
+    }
+    return v;
+}
+
+// One workgroup per key row: the latency-bound form used for the per-step append.
+template <int DT>
+__global__ __launch_bounds__(kEncThreads) void encode_row_kernel(EncodeArgs a) {
+    __shared__ float xs[kD];
+    __shared__ float nrm_s;
+    __shared__ unsigned long long best_s[kEncThreads / kWave];
+    __shared__ int code_s[kM];
+    const int tid = threadIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / a.H, h = bh % a.H;
+    const int j = blockIdx.x;
+    if (j >= a.count[b]) return;
+    const int slot = a.slot0[b] + j;
+    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+    const char *row = a.kv.k_base + row_offset(a.kv, b, h, (int64_t)a.sink + slot) * esz;
+    if (tid < kD) xs[tid] = load1<DT>(row, tid);
+    __syncthreads();
+    if (tid == 0) {
+        float ss = 0.0f;
+        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(xs[d], xs[d], ss);
+        float n = sqrtf(ss);
+        nrm_s = n < a.eps ? a.eps : n;
+    }
+    __syncthreads();
+    if (tid < kD) xs[tid] = xs[tid] / nrm_s;
+    __syncthreads();
+
+    const float *cbase = a.coarse + (size_t)bh * a.L * kD;
+    unsigned long long best = ~0ull;
+    for (int l = tid; l < a.L; l += kEncThreads) {
+        const float4 *c4 = reinterpret_cast<const float4 *>(cbase + (size_t)l * kD);
+        float d2 = 0.0f;
+#pragma unroll 8
+        for (int d4 = 0; d4 < kD / 4; ++d4) {
+            const float4 c = c4[d4];
+            float t;
+            t = xs[4 * d4] - c.x; d2 = __builtin_fmaf(t, t, d2);
+            t = xs[4 * d4 + 1] - c.y; d2 = __builtin_fmaf(t, t, d2);
+            t = xs[4 * d4 + 2] - c.z; d2 = __builtin_fmaf(t, t, d2);
+            t = xs[4 * d4 + 3] - c.w; d2 = __builtin_fmaf(t, t, d2);
+        }
+        // d2 >= 0, so its bit pattern orders like the value; the list id breaks ties low
+        const unsigned long long key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)l;
+        best = key < best ? key : best;
+    }
+    best = wave_min_u64(best, kWave);
+    if ((tid & (kWave - 1)) == 0) best_s[tid / kWave] = best;
+    __syncthreads();
+    best = best_s[0];
+#pragma unroll
+    for (int w = 1; w < kEncThreads / kWave; ++w) best = best_s[w] < best ? best_s[w] : best;
+    const int list = (int)(best & 0xffffffffull);
+    __syncthreads();
+    if (tid < kD) xs[tid] = xs[tid] - cbase[(size_t)list * kD + tid];
+    __syncthreads();
+    if (tid < kM * kCodes) {
+        const int m = tid / kCodes, c = tid % kCodes;
+        const float *w = a.codebooks + ((size_t)bh * kM * kCodes + tid) * kSub;
+        float d2 = 0.0f;
+#pragma unroll
+        for (int e = 0; e < kSub; ++e) {
+            const float t = xs[m * kSub + e] - w[e];
+            d2 = __builtin_fmaf(t, t, d2);
+        }
+        unsigned long long key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)c;
+        key = wave_min_u64(key, kCodes);
+        if (c == 0) code_s[m] = (int)(key & 0xffffffffull);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int m = 0; m < kM; ++m) word |= (uint32_t)code_s[m] << (4 * m);
+        const size_t o = (size_t)bh * a.n_cap + slot;
+        a.codes[o] = word;
+        a.list_ids[o] = (uint16_t)list;
+        a.norms[o] = nrm_s;
+    }
+}
+
+// Add the values of freshly encoded rows to their lists, in insertion order, then refresh the
+// touched list means.  One workgroup per stream, one thread per value channel.
+template <int DT>
+__global__ __launch_bounds__(kD) void value_append_kernel(EncodeArgs a) {
+    const int d = threadIdx.x;
+    const int bh = blockIdx.x;
+    const int b = bh / a.H, h = bh % a.H;
+    const int cnt = a.count[b];
+    const int s0 = a.slot0[b];
+    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+    float *vsum = a.vsum + (size_t)bh * a.L * kD;
+    float *vcount = a.vcount + (size_t)bh * a.L;
+    float *vbar = a.vbar + (size_t)bh * a.L * kD;
+    for (int j = 0; j < cnt; ++j) {
+        const int l = a.list_ids[(size_t)bh * a.n_cap + s0 + j];
+        const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + s0 + j) * esz;
+        vsum[(size_t)l * kD + d] += load1<DT>(row, d);
+        __syncthreads();
+        if (d == 0) vcount[l] += 1.0f;
+        __syncthreads();
+        vbar[(size_t)l * kD + d] = vsum[(size_t)l * kD + d] / vcount[l];
+    }
+}
+
+// Rebuild per-list value sums / counts / means.  One workgroup per (stream, 8 lists); every
+// workgroup walks the list ids in insertion order and accumulates the rows of its lists.
+constexpr int kListsPerWg = 8;
+
+template <int DT>
+__global__ __launch_bounds__(kD) void value_summaries_kernel(EncodeArgs a) {
+    __shared__ float acc[kListsPerWg][kD];
+    __shared__ float cnt_s[kListsPerWg];
+    const int d = threadIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / a.H, h = bh % a.H;
+    const int l0 = blockIdx.x * kListsPerWg;
+    const int n = a.n_idx[b];
+    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+#pragma unroll
+    for (int l = 0; l < kListsPerWg; ++l) acc[l][d] = 0.0f;
+    if (d < kListsPerWg) cnt_s[d] = 0.0f;
+    __syncthreads();
+    __shared__ int rel[kD];
+    const uint16_t *lids = a.list_ids + (size_t)bh * a.n_cap;
+    for (int i0 = 0; i0 < n; i0 += kD) {
+        __syncthreads();
+        rel[d] = (i0 + d < n) ? (int)lids[i0 + d] - l0 : -1;
+        __syncthreads();
+        const int lim = min(kD, n - i0);
+        for (int t = 0; t < lim; ++t) {
+            const int l = rel[t];
+            if (l < 0 || l >= kListsPerWg) continue;
+            const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + i0 + t) * esz;
+            acc[l][d] += load1<DT>(row, d);
+            if (d == 0) cnt_s[l] += 1.0f;
+        }
+    }
+    __syncthreads();
+    for (int l = 0; l < kListsPerWg; ++l) {
+        if (l0 + l >= a.L) break;
+        const size_t o = ((size_t)bh * a.L + l0 + l) * kD + d;
+        const float c = cnt_s[l];
+        a.vsum[o] = acc[l][d];
+        a.vbar[o] = c > 0.0f ? acc[l][d] / c : 0.0f;
+        if (d == 0) a.vcount[(size_t)bh * a.L + l0 + l] = c;
+    }
+}
+
+// ---- paged readers ----------------------------------------------------------------------
+// positions == NULL: token range [start, start + count); else positions[h, i].
+__global__ __launch_bounds__(256) void paged_gather_kernel(KvView kv, int seq, int64_t start, int64_t count,
+                                                           const int64_t *positions, char *out_k, char *out_v) {
+    const int lanes = kD * kv.esize / 16;  // 16-byte lanes per row
+    const int rows_per_block = 256 / lanes;
+    const int h = blockIdx.y;
+    const int64_t i = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / lanes;
+    const int lane = threadIdx.x % lanes;
+    if (i >= count) return;
+    const int64_t pos = positions ? positions[(int64_t)h * count + i] : start + i;
+    const int64_t off = row_offset(kv, seq, h, pos) * kv.esize;
+    const int64_t dst = ((int64_t)h * count + i) * kD * kv.esize;
+    reinterpret_cast<uint4 *>(out_k + dst)[lane] = reinterpret_cast<const uint4 *>(kv.k_base + off)[lane];
+    reinterpret_cast<uint4 *>(out_v + dst)[lane] = reinterpret_cast<const uint4 *>(kv.v_base + off)[lane];
+}
+
+static int fill_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *index, int sink, const int32_t *slot0,
+                     const int32_t *count, float eps) {
+    PQHSA_REQUIRE(index != nullptr, "index is NULL");
+    int rc = validate_view(kv);
+    if (rc) return rc;
+    PQHSA_REQUIRE(index->codes && index->list_ids && index->norms && index->coarse && index->codebooks,
+                  "index has NULL arrays");
+    PQHSA_REQUIRE(index->num_lists >= 1 && index->num_lists <= 65536, "num_lists=%d", index->num_lists);
+    a.kv = make_view(kv);
+    a.H = index->kv_heads; a.L = index->num_lists; a.sink = sink; a.slot0 = slot0; a.count = count;
+    a.coarse = index->coarse; a.codebooks = index->codebooks; a.eps = eps;
+    a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.n_cap = index->n_cap;
+    a.vsum = index->vsum; a.vcount = index->vcount; a.vbar = index->vbar; a.n_idx = index->n_idx;
+    return PQHSA_OK;
+}
+
+static int launch_encode(const EncodeArgs &a, int dtype, int BH, int count_max, hipStream_t stream) {
+    if (BH == 0 || count_max <= 0) return PQHSA_OK;
+    if (count_max >= 64) {
+        dim3 grid((count_max + kEncThreads - 1) / kEncThreads, BH);
+        PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(encode_bulk_kernel<DT>, grid, dim3(kEncThreads), 0, stream, a));
+    } else {
+        dim3 grid(count_max, BH);
+        PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(encode_row_kernel<DT>, grid, dim3(kEncThreads), 0, stream, a));
+    }
+    return check_launch("encode");
+}
+
+}  // namespace pqhsa
+
+using namespace pqhsa;
+
+extern "C" int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink, const int32_t *slot0,
+                            const int32_t *count, int32_t count_max, float eps, void *stream) {
+    EncodeArgs a = {};
+    int rc = fill_args(a, kv, index, sink, slot0, count, eps);
+    if (rc) return rc;
+    PQHSA_REQUIRE(slot0 && count, "encode: NULL slot0/count");
+    return launch_encode(a, kv->dtype, index->batch * index->kv_heads, count_max, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
+                                   const int32_t *slot0, const int32_t *count, int32_t count_max, float eps,
+                                   void *stream_v) {
+    EncodeArgs a = {};
+    int rc = fill_args(a, kv, index, sink, slot0, count, eps);
+    if (rc) return rc;
+    PQHSA_REQUIRE(slot0 && count, "encode_append: NULL slot0/count");
+    PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar, "encode_append: index has no value summaries");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const int BH = index->batch * index->kv_heads;
+    rc = launch_encode(a, kv->dtype, BH, count_max, stream);
+    if (rc || BH == 0 || count_max <= 0) return rc;
+    PQHSA_DISPATCH_DTYPE(kv->dtype, hipLaunchKernelGGL(value_append_kernel<DT>, dim3(BH), dim3(kD), 0, stream, a));
+    return check_launch("value_append");
+}
+
+extern "C" int pqhsa_value_summaries(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink, int32_t n_max,
+                                     void *stream) {
+    EncodeArgs a = {};
+    int rc = fill_args(a, kv, index, sink, nullptr, nullptr, 0.0f);
+    if (rc) return rc;
+    PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar && index->n_idx, "value_summaries: NULL arrays");
+    (void)n_max;
+    const int BH = index->batch * index->kv_heads;
+    if (BH == 0) return PQHSA_OK;
+    dim3 grid((index->num_lists + kListsPerWg - 1) / kListsPerWg, BH);
+    PQHSA_DISPATCH_DTYPE(kv->dtype, hipLaunchKernelGGL(value_summaries_kernel<DT>, grid, dim3(kD), 0,
+                                                       static_cast<hipStream_t>(stream), a));
+    return check_launch("value_summaries");
+}
+
+static int paged_gather(const pqhsa_kv_view *kv, int H, int seq, int64_t start, int64_t count,
+                        const int64_t *positions, void *out_k, void *out_v, void *stream) {
+    int rc = validate_view(kv);
+    if (rc) return rc;
+    PQHSA_REQUIRE(out_k && out_v, "paged_gather: NULL output");
+    PQHSA_REQUIRE(H >= 1 && seq >= 0 && count >= 0 && start >= 0, "paged_gather: bad H/seq/start/count");
+    if (count == 0) return PQHSA_OK;
+    KvView v = make_view(kv);
+    const int lanes = kD * v.esize / 16;
+    const int rows_per_block = 256 / lanes;
+    dim3 grid((unsigned)((count + rows_per_block - 1) / rows_per_block), H);
+    hipLaunchKernelGGL(paged_gather_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), v, seq, start,
+                       count, positions, static_cast<char *>(out_k), static_cast<char *>(out_v));
+    return check_launch("paged_gather");
+}
+
+extern "C" int pqhsa_paged_gather_range(const pqhsa_kv_view *kv, int32_t H, int32_t seq, int64_t start, int64_t count,
+                                        void *out_k, void *out_v, void *stream) {
+    return paged_gather(kv, H, seq, start, count, nullptr, out_k, out_v, stream);
+}
+
+extern "C" int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq, const int64_t *positions,
+                                     int64_t count, void *out_k, void *out_v, void *stream) {
+    PQHSA_REQUIRE(positions != nullptr, "paged_gather_at: NULL positions");
+    return paged_gather(kv, H, seq, 0, count, positions, out_k, out_v, stream);
+}

@@ -1,0 +1,118 @@
+// Kernel 1: per-(sequence, KV head) query -> lookup tables, staged in LDS.
+//
+// One workgroup column per stream bh; block x == 0 builds the 8 x 16 PQ table of every query
+// row of the GQA group, blocks x >= 1 each take 64 coarse lists and compute the
+// query-to-IVF-centroid dot products.  All reductions are left-to-right fused multiply-add
+// chains so the results are bit-identical to the scalar CPU oracle.
+#include "common.h"
+
+namespace pqhsa {
+
+constexpr int kLutThreads = 256;
+constexpr int kListsPerBlock = 64;
+constexpr int kMaxG = 16;
+
+template <int DT>
+__global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
+    const char *__restrict__ q, int H, int G, int Gp, const float *__restrict__ coarse,
+    const float *__restrict__ codebooks, int L, float eps, float *__restrict__ qnorm,
+    float *__restrict__ lut, float *__restrict__ list_scores, uint32_t *__restrict__ zero_base,
+    size_t zero_words) {
+    __shared__ float qh[kMaxG][kD];
+    __shared__ float qn[kMaxG];
+    __shared__ float cs[kListsPerBlock][kD + 1];
+
+    const int tid = threadIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / H, h = bh % H;
+
+    // scratch that the later kernels of a decode step accumulate into starts at zero
+    if (zero_words) {
+        const size_t nthreads = (size_t)gridDim.x * gridDim.y * kLutThreads;
+        const size_t me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kLutThreads + tid;
+        for (size_t i = me; i < zero_words; i += nthreads) zero_base[i] = 0u;
+    }
+
+    // query rows of this stream: q[b, h*G + g, :]
+    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+    const char *qrow0 = q + ((size_t)b * H * G + (size_t)h * G) * kD * esz;
+    for (int i = tid; i < G * kD; i += kLutThreads) {
+        int g = i / kD, d = i % kD;
+        qh[g][d] = load1<DT>(qrow0 + (size_t)g * kD * esz, d);
+    }
+    __syncthreads();
+    if (tid < G) {
+        float ss = 0.0f;
+        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(qh[tid][d], qh[tid][d], ss);
+        float n = sqrtf(ss);
+        qn[tid] = n < eps ? eps : n;
+    }
+    __syncthreads();
+    for (int i = tid; i < G * kD; i += kLutThreads) {
+        int g = i / kD, d = i % kD;
+        qh[g][d] = qh[g][d] / qn[g];
+    }
+    __syncthreads();
+
+    if (blockIdx.x == 0) {
+        if (tid < Gp) qnorm[(size_t)bh * Gp + tid] = tid < G ? qn[tid] : 0.0f;
+        const float *cb = codebooks + (size_t)bh * kM * kCodes * kSub;
+        float *out = lut + (size_t)bh * kM * kCodes * Gp;
+        for (int e = tid; e < kM * kCodes * Gp; e += kLutThreads) {
+            int g = e % Gp;
+            int mc = e / Gp;  // m * 16 + c
+            float acc = 0.0f;
+            if (g < G) {
+                int m = mc / kCodes;
+                const float *w = cb + (size_t)mc * kSub;
+#pragma unroll
+                for (int j = 0; j < kSub; ++j) acc = __builtin_fmaf(qh[g][m * kSub + j], w[j], acc);
+            }
+            out[e] = acc;
+        }
+        return;
+    }
+
+    const int l0 = (blockIdx.x - 1) * kListsPerBlock;
+    const float *cbase = coarse + ((size_t)bh * L + l0) * kD;
+    const int nl = min(kListsPerBlock, L - l0);
+    for (int i = tid; i < nl * kD; i += kLutThreads) cs[i / kD][i % kD] = cbase[i];
+    __syncthreads();
+    const int lane = tid % kListsPerBlock;
+    const int wave = tid / kListsPerBlock;
+    float *out = list_scores + ((size_t)bh * L + l0) * Gp;
+    for (int g = wave; g < Gp; g += kLutThreads / kListsPerBlock) {
+        if (lane >= nl) continue;
+        float acc = 0.0f;
+        if (g < G) {
+#pragma unroll 8
+            for (int d = 0; d < kD; ++d) acc = __builtin_fmaf(qh[g][d], cs[lane][d], acc);
+        }
+        out[(size_t)lane * Gp + g] = acc;
+    }
+}
+
+int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps,
+                     float *qnorm, float *lut, float *list_scores, uint32_t *zero_base,
+                     size_t zero_words, hipStream_t stream) {
+    PQHSA_REQUIRE(q && index && qnorm && lut && list_scores, "lut_build: NULL argument");
+    PQHSA_REQUIRE(G >= 1 && G <= kMaxG, "lut_build: G=%d outside [1, %d]", G, kMaxG);
+    PQHSA_REQUIRE(index->num_lists >= 1 && index->num_lists <= 4096, "lut_build: num_lists=%d", index->num_lists);
+    const int BH = index->batch * index->kv_heads;
+    if (BH == 0) return PQHSA_OK;
+    const int Gp = padded_groups(G);
+    dim3 grid(1 + (index->num_lists + kListsPerBlock - 1) / kListsPerBlock, BH);
+    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(lut_build_kernel<DT>, grid, dim3(kLutThreads), 0, stream,
+                                                     static_cast<const char *>(q), index->kv_heads, G, Gp,
+                                                     index->coarse, index->codebooks, index->num_lists, eps,
+                                                     qnorm, lut, list_scores, zero_base, zero_words));
+    return check_launch("lut_build");
+}
+
+}  // namespace pqhsa
+
+extern "C" int pqhsa_lut_build(const void *q, int32_t q_dtype, const pqhsa_index *index, int32_t G,
+                               float eps, float *qnorm, float *lut, float *list_scores, void *stream) {
+    return pqhsa::launch_lut_build(q, q_dtype, index, G, eps, qnorm, lut, list_scores, nullptr, 0,
+                                   static_cast<hipStream_t>(stream));
+}

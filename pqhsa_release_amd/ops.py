@@ -1,0 +1,346 @@
+"""Torch-facing wrappers of the C ABI: tensors in, tensors out, kernels on the current stream.
+
+PyTorch only provides device memory and the stream here; every computation below is one of
+the HIP kernels behind ``libpqhsa.so``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import Index, KvView, Select
+
+HEAD_DIM = 128
+SUBSPACES = 8
+CODES = 16
+SUBDIM = HEAD_DIM // SUBSPACES
+EPS = 1e-12
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _lib.F32
+    if dtype == torch.bfloat16:
+        return _lib.BF16
+    if dtype == torch.float16:
+        return _lib.F16
+    raise ValueError(f"unsupported dtype {dtype}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _need_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("PQ-HSA kernels need device tensors; there is no CPU path")
+
+
+def padded_groups(groups: int) -> int:
+    p = 1
+    while p < groups:
+        p <<= 1
+    return p
+
+
+def resolve_topk(n: int, fraction: float | None, topk: int) -> int:
+    """k = min(max(ceil(n * fraction), 0), n) or min(topk, n)."""
+    if fraction is not None and fraction > 0:
+        k = int(math.ceil(n * fraction))
+    else:
+        k = int(topk)
+    return min(max(k, 0), n)
+
+
+# --------------------------------------------------------------------------- K/V views
+@dataclass
+class KvSource:
+    """A ``pqhsa_kv_view`` plus the tensors it points into (kept alive)."""
+
+    view: KvView
+    keep: tuple
+    dtype: torch.dtype
+    batch: int
+    kv_heads: int
+
+    def ref(self):
+        return ctypes.byref(self.view)
+
+
+def kv_contiguous(keys: torch.Tensor, values: torch.Tensor) -> KvSource:
+    """keys/values ``[B, H, cap, 128]`` with unit stride in the last dim and equal strides."""
+    _need_cuda(keys, values)
+    if keys.ndim != 4 or values.ndim != 4 or keys.shape[-1] != HEAD_DIM or values.shape[-1] != HEAD_DIM:
+        raise ValueError(f"keys/values must be [B, H, S, {HEAD_DIM}]")
+    if keys.stride() != values.stride() or keys.stride(-1) != 1 or keys.dtype != values.dtype:
+        raise ValueError("keys and values must share dtype and strides, last dim contiguous")
+    v = KvView()
+    v.k_base, v.v_base = keys.data_ptr(), values.data_ptr()
+    v.dtype, v.paged = dtype_code(keys.dtype), 0
+    v.stride_seq, v.stride_head, v.stride_tok, v.stride_block = keys.stride(0), keys.stride(1), keys.stride(2), 0
+    v.block_size, v.max_blocks, v.block_table = 0, 0, None
+    return KvSource(v, (keys, values), keys.dtype, keys.shape[0], keys.shape[1])
+
+
+def kv_paged(kv_cache: torch.Tensor, block_table: torch.Tensor) -> KvSource:
+    """Paged cache in either layout: 5-D ``[2, blocks, bs, H, D]`` or 4-D ``[blocks, H, bs, 2*D]``."""
+    _need_cuda(kv_cache, block_table)
+    if block_table.dtype != torch.int32 or block_table.ndim != 2 or not block_table.is_contiguous():
+        raise ValueError("block_table must be a contiguous int32 [B, max_blocks] tensor")
+    v = KvView()
+    esz = kv_cache.element_size()
+    if kv_cache.dim() == 5:
+        if kv_cache.shape[0] != 2 or kv_cache.shape[-1] != HEAD_DIM or kv_cache.stride(-1) != 1:
+            raise ValueError(f"unsupported 5-D kv_cache shape {tuple(kv_cache.shape)}")
+        v.k_base = kv_cache.data_ptr()
+        v.v_base = kv_cache.data_ptr() + kv_cache.stride(0) * esz
+        v.stride_block, v.stride_tok, v.stride_head = kv_cache.stride(1), kv_cache.stride(2), kv_cache.stride(3)
+        v.block_size, heads = kv_cache.shape[2], kv_cache.shape[3]
+    elif kv_cache.dim() == 4:
+        if kv_cache.shape[-1] != 2 * HEAD_DIM or kv_cache.stride(-1) != 1:
+            raise ValueError(f"unsupported 4-D kv_cache shape {tuple(kv_cache.shape)}")
+        v.k_base = kv_cache.data_ptr()
+        v.v_base = kv_cache.data_ptr() + HEAD_DIM * esz
+        v.stride_block, v.stride_head, v.stride_tok = kv_cache.stride(0), kv_cache.stride(1), kv_cache.stride(2)
+        v.block_size, heads = kv_cache.shape[2], kv_cache.shape[1]
+    else:
+        raise ValueError(f"unsupported FLASH_ATTN kv_cache shape {tuple(kv_cache.shape)}")
+    v.dtype, v.paged, v.stride_seq = dtype_code(kv_cache.dtype), 1, 0
+    v.max_blocks, v.block_table = block_table.shape[1], block_table.data_ptr()
+    return KvSource(v, (kv_cache, block_table), kv_cache.dtype, block_table.shape[0], heads)
+
+
+# --------------------------------------------------------------------------- device index
+class DeviceIndex:
+    """Device-resident IVF-PQ index of B x H streams (structure of arrays, spare capacity)."""
+
+    def __init__(self, batch: int, kv_heads: int, num_lists: int, n_cap: int, device) -> None:
+        n_cap = max(8, (int(n_cap) + 7) // 8 * 8)
+        bh = batch * kv_heads
+        self.batch, self.kv_heads, self.num_lists, self.n_cap = batch, kv_heads, int(num_lists), n_cap
+        self.device = torch.device(device)
+        dev = self.device
+        self.codes = torch.zeros(bh, n_cap, dtype=torch.int32, device=dev)       # bit pattern of u32
+        self.list_ids = torch.zeros(bh, n_cap, dtype=torch.int16, device=dev)    # bit pattern of u16
+        self.norms = torch.zeros(bh, n_cap, dtype=torch.float32, device=dev)
+        self.coarse = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
+        self.codebooks = torch.zeros(bh, SUBSPACES, CODES, SUBDIM, dtype=torch.float32, device=dev)
+        self.vbar = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
+        self.vsum = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
+        self.vcount = torch.zeros(bh, num_lists, dtype=torch.float32, device=dev)
+        self.n_idx = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.n_host = [0] * batch          # host mirror of n_idx
+        self._struct = None
+
+    @property
+    def n_max(self) -> int:
+        return max(self.n_host) if self.n_host else 0
+
+    def set_counts(self, counts) -> None:
+        self.n_host = [int(c) for c in counts]
+        if max(self.n_host, default=0) > self.n_cap:
+            raise ValueError("index capacity exceeded")
+        self.n_idx.copy_(torch.tensor(self.n_host, dtype=torch.int32), non_blocking=False)
+
+    def struct(self) -> Index:
+        if self._struct is None:
+            s = Index()
+            s.codes, s.list_ids, s.norms = self.codes.data_ptr(), self.list_ids.data_ptr(), self.norms.data_ptr()
+            s.coarse, s.codebooks = self.coarse.data_ptr(), self.codebooks.data_ptr()
+            s.vbar, s.vsum, s.vcount = self.vbar.data_ptr(), self.vsum.data_ptr(), self.vcount.data_ptr()
+            s.n_idx, s.n_cap = self.n_idx.data_ptr(), self.n_cap
+            s.num_lists, s.batch, s.kv_heads = self.num_lists, self.batch, self.kv_heads
+            self._struct = s
+        return self._struct
+
+    def ref(self):
+        return ctypes.byref(self.struct())
+
+    def list_ids_long(self) -> torch.Tensor:
+        """List ids as int64 (the stored int16 tensor holds uint16 bit patterns)."""
+        return self.list_ids.to(torch.int64) & 0xFFFF
+
+    def packed_bytes(self) -> torch.Tensor:
+        """The reference's ``[N, 4]`` uint8 packing is the little-endian view of the code words."""
+        return self.codes.view(torch.uint8).reshape(self.codes.shape[0], self.n_cap, 4)
+
+
+def _i32(values, device) -> torch.Tensor:
+    return torch.tensor([int(v) for v in values], dtype=torch.int32, device=device)
+
+
+# --------------------------------------------------------------------------- index maintenance
+def encode(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: float = EPS) -> None:
+    """Encode ``count[b]`` key rows per sequence starting at index slot ``slot0[b]``."""
+    lib = _lib.load()
+    s0, c = _i32(slot0, index.device), _i32(count, index.device)
+    rc = lib.pqhsa_encode(kv.ref(), index.ref(), int(sink), s0.data_ptr(), c.data_ptr(), int(max(count)), eps,
+                          _stream())
+    _lib.check(rc, "pqhsa_encode")
+
+
+def value_summaries(kv: KvSource, index: DeviceIndex, sink: int) -> None:
+    lib = _lib.load()
+    rc = lib.pqhsa_value_summaries(kv.ref(), index.ref(), int(sink), int(index.n_max), _stream())
+    _lib.check(rc, "pqhsa_value_summaries")
+
+
+def encode_append(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: float = EPS,
+                  slot0_dev: torch.Tensor | None = None, count_dev: torch.Tensor | None = None,
+                  count_max: int | None = None) -> None:
+    lib = _lib.load()
+    s0 = slot0_dev if slot0_dev is not None else _i32(slot0, index.device)
+    c = count_dev if count_dev is not None else _i32(count, index.device)
+    cmax = int(count_max if count_max is not None else max(count))
+    rc = lib.pqhsa_encode_append(kv.ref(), index.ref(), int(sink), s0.data_ptr(), c.data_ptr(), cmax, eps, _stream())
+    _lib.check(rc, "pqhsa_encode_append")
+
+
+# --------------------------------------------------------------------------- scoring
+def lut_build(q: torch.Tensor, index: DeviceIndex, groups: int, *, eps: float = EPS):
+    """q ``[B, H*G, 128]`` -> qnorm ``[BH, Gp]``, lut ``[BH, 8, 16, Gp]``, list_scores ``[BH, L, Gp]``."""
+    _need_cuda(q)
+    lib = _lib.load()
+    bh, gp = index.batch * index.kv_heads, padded_groups(groups)
+    if tuple(q.shape) != (index.batch, index.kv_heads * groups, HEAD_DIM) or not q.is_contiguous():
+        raise ValueError(f"q must be contiguous [B, H*G, {HEAD_DIM}], got {tuple(q.shape)}")
+    qnorm = torch.empty(bh, gp, dtype=torch.float32, device=q.device)
+    lut = torch.empty(bh, SUBSPACES, CODES, gp, dtype=torch.float32, device=q.device)
+    ls = torch.empty(bh, index.num_lists, gp, dtype=torch.float32, device=q.device)
+    rc = lib.pqhsa_lut_build(q.data_ptr(), dtype_code(q.dtype), index.ref(), groups, eps, qnorm.data_ptr(),
+                             lut.data_ptr(), ls.data_ptr(), _stream())
+    _lib.check(rc, "pqhsa_lut_build")
+    return qnorm, lut, ls
+
+
+def lut_scan(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scale: float) -> torch.Tensor:
+    """Approximate logits ``[BH, G, n_cap]`` (columns >= n_idx are not written)."""
+    lib = _lib.load()
+    bh = index.batch * index.kv_heads
+    logits = torch.zeros(bh, groups, index.n_cap, dtype=torch.float32, device=index.device)
+    rc = lib.pqhsa_lut_scan(index.ref(), groups, int(index.n_max), qnorm.data_ptr(), lut.data_ptr(),
+                            list_scores.data_ptr(), float(scale), logits.data_ptr(), index.n_cap, _stream())
+    _lib.check(rc, "pqhsa_lut_scan")
+    return logits
+
+
+def topk_radix(logits: torch.Tensor, n, k):
+    """Exact top-k of each row of ``logits [rows, stride]``; ``n``/``k`` per row.  Returns
+    (indices int32 [rows, k_cap], values f32 [rows, k_cap]) in ascending index order."""
+    _need_cuda(logits)
+    lib = _lib.load()
+    if logits.ndim != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise ValueError("logits must be a float32 [rows, stride] matrix")
+    rows = logits.shape[0]
+    n_t, k_t = _i32(n, logits.device), _i32(k, logits.device)
+    n_max, k_cap = int(max(n, default=0)), max(int(max(k, default=0)), 1)
+    ws_bytes = lib.pqhsa_topk_workspace_bytes(rows, n_max)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=logits.device)
+    idx = torch.full((rows, k_cap), -1, dtype=torch.int32, device=logits.device)
+    val = torch.zeros(rows, k_cap, dtype=torch.float32, device=logits.device)
+    rc = lib.pqhsa_topk_radix(logits.data_ptr(), logits.stride(0), rows, n_t.data_ptr(), k_t.data_ptr(), n_max,
+                              idx.data_ptr(), val.data_ptr(), k_cap, ws.data_ptr(), ws_bytes, _stream())
+    _lib.check(rc, "pqhsa_topk_radix")
+    return idx, val
+
+
+# --------------------------------------------------------------------------- decode step
+class DecodeWorkspace:
+    """Scratch memory of ``pqhsa_decode_step`` for a fixed (B, H, G, n_cap, L, k_cap)."""
+
+    def __init__(self, index: DeviceIndex, groups: int, k_cap: int) -> None:
+        lib = _lib.load()
+        self.k_cap = max(int(k_cap), 1)
+        self.groups = groups
+        self.bytes = lib.pqhsa_decode_workspace_bytes(index.batch, index.kv_heads, groups, index.n_cap,
+                                                      index.num_lists, self.k_cap)
+        self.buf = torch.empty(self.bytes, dtype=torch.uint8, device=index.device)
+        rows = index.batch * index.kv_heads * groups
+        self.topk_idx = torch.full((rows, self.k_cap), -1, dtype=torch.int32, device=index.device)
+        self.topk_val = torch.zeros(rows, self.k_cap, dtype=torch.float32, device=index.device)
+        self.topk_cnt = torch.zeros(rows, dtype=torch.int32, device=index.device)
+
+
+def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
+                seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
+                scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None) -> torch.Tensor:
+    """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``."""
+    _need_cuda(q, out, seq_lens)
+    lib = _lib.load()
+    if tuple(q.shape) != (index.batch, index.kv_heads * groups, HEAD_DIM) or not q.is_contiguous():
+        raise ValueError(f"q must be contiguous [B, H*G, {HEAD_DIM}], got {tuple(q.shape)}")
+    if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise ValueError("out must match q in shape and dtype")
+    if seq_lens.dtype != torch.int32 or seq_lens.numel() != index.batch:
+        raise ValueError("seq_lens must be int32 [B]")
+    sel = Select()
+    sel.fraction = float(fraction) if fraction else 0.0
+    sel.topk = int(topk)
+    sel.k_cap = workspace.k_cap
+    n_max = index.n_max if n_max is None else int(n_max)
+    rc = lib.pqhsa_decode_step(q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups,
+                               seq_lens.data_ptr(), int(sink), n_max, int(full_max), ctypes.byref(sel), float(scale),
+                               eps, workspace.topk_idx.data_ptr(), workspace.topk_val.data_ptr(),
+                               workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(), workspace.bytes, _stream())
+    _lib.check(rc, "pqhsa_decode_step")
+    return out
+
+
+def hybrid_attend_paged(q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int, full_max: int,
+                        topk_idx, topk_val, topk_cnt, list_mass, row_max, scale: float) -> torch.Tensor:
+    """Exact hybrid attention given a selection and per-list masses (``list_mass [BH, G, L]``
+    relative to ``row_max [BH, G]``)."""
+    _need_cuda(q, out, topk_idx, topk_val, topk_cnt, list_mass, row_max)
+    lib = _lib.load()
+    ws_bytes = lib.pqhsa_attend_workspace_bytes(index.batch, index.kv_heads, groups)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    rc = lib.pqhsa_hybrid_attend_paged(q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(),
+                                       groups, seq_lens.data_ptr(), int(sink), int(full_max), topk_idx.data_ptr(),
+                                       topk_val.data_ptr(), topk_cnt.data_ptr(), topk_idx.shape[-1],
+                                       list_mass.data_ptr(), row_max.data_ptr(), float(scale), ws.data_ptr(),
+                                       ws_bytes, _stream())
+    _lib.check(rc, "pqhsa_hybrid_attend_paged")
+    return out
+
+
+# --------------------------------------------------------------------------- paged readers
+def paged_gather_range(kv: KvSource, seq: int, start: int, end: int):
+    """Token range [start, end) of sequence ``seq`` -> K, V ``[H, n, 128]``."""
+    lib = _lib.load()
+    n = max(int(end) - int(start), 0)
+    dev = kv.keep[0].device
+    out_k = torch.empty(kv.kv_heads, n, HEAD_DIM, dtype=kv.dtype, device=dev)
+    out_v = torch.empty_like(out_k)
+    if n:
+        rc = lib.pqhsa_paged_gather_range(kv.ref(), kv.kv_heads, int(seq), int(start), n, out_k.data_ptr(),
+                                          out_v.data_ptr(), _stream())
+        _lib.check(rc, "pqhsa_paged_gather_range")
+    return out_k, out_v
+
+
+def paged_gather_at(kv: KvSource, seq: int, positions: torch.Tensor):
+    """positions int64 ``[H, ...]`` -> K, V shaped like ``positions`` + ``[128]``."""
+    lib = _lib.load()
+    _need_cuda(positions)
+    if positions.shape[0] != kv.kv_heads:
+        raise ValueError("positions must have the KV head as leading dimension")
+    flat = positions.reshape(kv.kv_heads, -1).to(torch.int64).contiguous()
+    n = flat.shape[1]
+    out_k = torch.empty(kv.kv_heads, n, HEAD_DIM, dtype=kv.dtype, device=positions.device)
+    out_v = torch.empty_like(out_k)
+    if n:
+        rc = lib.pqhsa_paged_gather_at(kv.ref(), kv.kv_heads, int(seq), flat.data_ptr(), n, out_k.data_ptr(),
+                                       out_v.data_ptr(), _stream())
+        _lib.check(rc, "pqhsa_paged_gather_at")
+    shape = (*positions.shape, HEAD_DIM)
+    return out_k.reshape(shape), out_v.reshape(shape)

@@ -1,0 +1,236 @@
+"""GPU parity tests: every HIP kernel, through the C ABI, against the fixed-order CPU oracle.
+
+Integer results (packed codes, list ids, top-k index sets) and fp32 table/score values are
+compared bit-exactly; attention outputs within 1e-4 (fp32 K/V) or 2e-3 max-abs (bf16 K/V).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fixed
+from tests.gpu_util import DIM, SCALE, Problem, u16, u32
+
+pytestmark = pytest.mark.gpu
+
+ops = pytest.importorskip("pqhsa_release_amd.ops")
+
+
+def _cuda():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return "cuda"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("paged", [None, "5d", "4d"])
+def test_encode_bulk_and_row_kernels_match_oracle_bitwise(dtype, paged):
+    dev = _cuda()
+    p = Problem(lens=[900, 517], heads=2, lists=48, dtype=dtype, seed=3)
+    idx = p.device_index(dev, upload_codes=False)
+    if paged:
+        cache, table = p.paged_kv(paged)
+        kv = ops.kv_paged(cache, table)
+    else:
+        kv = ops.kv_contiguous(*p.dense_kv())
+    counts = [p.n(b) for b in range(p.B)]
+    # bulk kernel for all but the last 5 rows, one-row kernel for the rest
+    ops.encode(kv, idx, p.sink, [0, 0], [c - 5 for c in counts])
+    ops.encode(kv, idx, p.sink, [c - 5 for c in counts], [5, 5])
+    torch.cuda.synchronize()
+    for (b, h), ix in p.index.items():
+        bh, n = b * p.H + h, p.n(b)
+        assert np.array_equal(u32(idx.codes[bh, :n]), ix["codes"]), (b, h)
+        assert np.array_equal(u16(idx.list_ids[bh, :n]), ix["list_ids"]), (b, h)
+        assert np.array_equal(idx.norms[bh, :n].cpu().numpy(), ix["norms"]), (b, h)
+    # the reference's [N, 4] uint8 packing is the byte view of the words
+    packed = idx.packed_bytes()[0, : p.n(0)].cpu().numpy()
+    w = p.index[0, 0]["codes"]
+    assert np.array_equal(packed[:, 1] >> 4, (w >> 12) & 15) and np.array_equal(packed[:, 0] & 15, w & 15)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_value_summaries_and_append_match_oracle(dtype):
+    dev = _cuda()
+    p = Problem(lens=[700], heads=2, lists=32, dtype=dtype, seed=5)
+    idx = p.device_index(dev)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    idx.vbar.zero_()
+    n = p.n(0)
+    # build summaries over the first n - 3 keys, then append 3 (one launch)
+    idx.set_counts([n - 3])
+    ops.value_summaries(kv, idx, p.sink)
+    ops.encode_append(kv, idx, p.sink, [n - 3], [3])
+    idx.set_counts([n])
+    torch.cuda.synchronize()
+    for h in range(p.H):
+        ix = p.index[0, h]
+        vals = p.values[0, h][p.sink : p.sink + n].numpy()
+        sums, counts, vbar = fixed.value_summaries(vals[: n - 3], ix["list_ids"][: n - 3], p.L)
+        for j in range(n - 3, n):
+            fixed.value_append(vals[j], int(ix["list_ids"][j]), sums, counts, vbar)
+        # untouched lists keep the mean of the build; touched ones were recomputed
+        np.testing.assert_array_equal(idx.vcount[h].cpu().numpy(), counts)
+        np.testing.assert_allclose(idx.vsum[h].cpu().numpy(), sums, rtol=0, atol=1e-5)
+        np.testing.assert_allclose(idx.vbar[h].cpu().numpy(), vbar, rtol=0, atol=1e-6)
+        assert np.array_equal(u32(idx.codes[h, n - 3 : n]), ix["codes"][n - 3 :])
+        assert np.array_equal(u16(idx.list_ids[h, n - 3 : n]), ix["list_ids"][n - 3 :])
+
+
+@pytest.mark.parametrize("groups", [1, 3, 4, 7])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_lut_build_and_scan_match_oracle_bitwise(groups, dtype):
+    dev = _cuda()
+    p = Problem(lens=[1500, 1111], heads=2, groups=groups, lists=40, dtype=dtype, seed=7)
+    idx = p.device_index(dev)
+    q = p.q_tensor()
+    qnorm, lut, ls = ops.lut_build(q, idx, groups)
+    logits = ops.lut_scan(idx, groups, qnorm, lut, ls, SCALE)
+    torch.cuda.synchronize()
+    for (b, h), ix in p.index.items():
+        bh, n = b * p.H + h, p.n(b)
+        oq, olut, ols = fixed.lut_build(p.queries[b, h].numpy(), ix["coarse"], ix["codebooks"])
+        assert np.array_equal(qnorm[bh, :groups].cpu().numpy(), oq)
+        assert np.array_equal(lut[bh, :, :, :groups].permute(2, 0, 1).cpu().numpy(), olut)
+        assert np.array_equal(ls[bh, :, :groups].T.cpu().numpy(), ols)
+        assert (lut[bh, :, :, groups:] == 0).all() and (ls[bh, :, groups:] == 0).all()
+        want = fixed.scan(ix["codes"], ix["list_ids"], ix["norms"], olut, ols, oq, SCALE)
+        got = logits[bh, :, :n].cpu().numpy()
+        assert np.array_equal(got, want), (b, h, np.abs(got - want).max())
+
+
+def test_topk_radix_on_logit_matrix_with_ties():
+    dev = _cuda()
+    rng = np.random.default_rng(11)
+    rows, stride = 9, 5000
+    logits = rng.standard_normal((rows, stride)).astype(np.float32)
+    logits[1, :] = 0.5                                    # all equal: pure lowest-index rule
+    logits[2, 100:400] = logits[2].max() + 1              # wide tie at the top
+    logits[3, ::7] = np.sort(logits[3])[::-1][40]         # ties straddling the k boundary
+    logits[4] = np.abs(logits[4]) * -1                    # all negative
+    logits[5, :10] = [0.0, -0.0, 0.0, -0.0, 1.0, -0.0, 0.0, 2.0, -0.0, 0.0]
+    logits[5, 10:] = -1.0
+    n = [5000, 4097, 5000, 4999, 1, 12, 2500, 5000, 64]
+    k = [100, 37, 150, 41, 1, 6, 2500, 0, 63]
+    idx, val = ops.topk_radix(torch.from_numpy(logits).to(dev), n, k)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    for r in range(rows):
+        want_idx, _ = fixed.topk(logits[r, : n[r]], k[r])
+        got = idx[r, : k[r]]
+        assert np.array_equal(got, np.sort(want_idx)), r      # ascending index order, exact set
+        assert np.array_equal(val[r, : k[r]], logits[r, got]), r
+
+
+@pytest.mark.parametrize("case", [
+    dict(lens=[2048], heads=1, groups=1, lists=64, dtype=torch.float32, fraction=0.02, kv="dense"),
+    dict(lens=[3000, 1800], heads=2, groups=4, lists=64, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
+    dict(lens=[2500, 1900, 700], heads=2, groups=4, lists=32, dtype=torch.bfloat16, fraction=0.05, kv="4d"),
+    dict(lens=[2200], heads=2, groups=7, lists=48, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
+    dict(lens=[1500], heads=1, groups=2, lists=16, dtype=torch.float16, fraction=0.1, kv="dense"),
+])
+def test_decode_step_topk_bitexact_and_output_close(case):
+    dev = _cuda()
+    p = Problem(lens=case["lens"], heads=case["heads"], groups=case["groups"], lists=case["lists"],
+                dtype=case["dtype"], seed=13)
+    idx = p.device_index(dev)
+    if case["kv"] == "dense":
+        kv = ops.kv_contiguous(*p.dense_kv())
+    else:
+        kv = ops.kv_paged(*p.paged_kv(case["kv"]))
+    k_cap = ops.resolve_topk(p.n_max, case["fraction"], 0)
+    ws = ops.DecodeWorkspace(idx, p.G, k_cap)
+    # 16-bit K/V are read in place; the query/output pair is tried both in fp32 (the stated
+    # 2e-3 max-abs bound applies as is) and in the cache dtype (the output is then rounded to
+    # 8 or 11 significant bits, which alone costs up to 2^-9 relative)
+    q_dtypes = [torch.float32] if case["dtype"] == torch.float32 else [torch.float32, case["dtype"]]
+    for q_dtype in q_dtypes:
+        q = p.q_tensor().to(q_dtype)
+        out = torch.empty_like(q)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
+                        fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws)
+        torch.cuda.synchronize()
+        tol = 1e-4 if case["dtype"] == torch.float32 else 2e-3
+        rel = 0.0 if q_dtype == torch.float32 else (2.0 ** -8 if q_dtype == torch.bfloat16 else 2.0 ** -11)
+        cnt = ws.topk_cnt.cpu().numpy().reshape(p.B, p.H, p.G)
+        tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        tval = ws.topk_val.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        worst = 0.0
+        for (b, h) in p.index:
+            want_out, want_idx, logits = p.oracle_step(b, h, case["fraction"])
+            k = want_idx.shape[1]
+            for g in range(p.G):
+                assert cnt[b, h, g] == k
+                got = tidx[b, h, g, :k]
+                assert np.array_equal(got, np.sort(want_idx[g])), (b, h, g)          # bit-exact set
+                assert np.array_equal(tval[b, h, g, :k], logits[g, got]), (b, h, g)  # and their logits
+            err = np.abs(o[b, h] - want_out)
+            assert (err <= tol + rel * np.abs(want_out)).all(), (b, h, q_dtype, err.max())
+            worst = max(worst, float(err.max()))
+        print(f"decode_step {case['dtype']} q={q_dtype}: max abs err {worst:.3e}")
+
+
+def test_decode_step_all_selected_equals_dense_attention():
+    dev = _cuda()
+    p = Problem(lens=[600], heads=1, groups=2, lists=16, seed=17)
+    idx = p.device_index(dev)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    q = p.q_tensor()
+    out = torch.empty_like(q)
+    ws = ops.DecodeWorkspace(idx, p.G, p.n_max)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=1.0,
+                    topk=0, scale=SCALE, workspace=ws)
+    k64, v64, q64 = p.keys[0, 0].double(), p.values[0, 0].double(), p.queries[0, 0].double()
+    dense = torch.softmax((q64 @ k64.T) * SCALE, dim=-1) @ v64
+    np.testing.assert_allclose(out[0].cpu().double().numpy(), dense.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_decode_step_degenerate_shapes():
+    dev = _cuda()
+    # no indexed keys at all (context shorter than sink + local): plain exact attention
+    p = Problem(lens=[40], heads=1, groups=2, lists=8, seed=19)
+    assert p.n(0) == 0
+    idx = ops.DeviceIndex(1, 1, 8, 8, dev)
+    idx.set_counts([0])
+    kv = ops.kv_contiguous(*p.dense_kv())
+    q = p.q_tensor()
+    out = torch.full_like(q, float("nan"))
+    ws = ops.DecodeWorkspace(idx, p.G, 1)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=40, fraction=0.02, topk=0,
+                    scale=SCALE, workspace=ws)
+    k64, v64, q64 = p.keys[0, 0].double(), p.values[0, 0].double(), p.queries[0, 0].double()
+    dense = torch.softmax((q64 @ k64.T) * SCALE, dim=-1) @ v64
+    np.testing.assert_allclose(out[0].cpu().double().numpy(), dense.numpy(), rtol=1e-4, atol=1e-5)
+    assert (ws.topk_cnt == 0).all()
+
+
+@pytest.mark.parametrize("layout", ["5d", "4d"])
+def test_paged_readers_match_contiguous_tensor(layout):
+    dev = _cuda()
+    p = Problem(lens=[333, 190], heads=3, lists=8, dtype=torch.bfloat16, seed=23)
+    cache, table = p.paged_kv(layout)
+    kv = ops.kv_paged(cache, table)
+    for b in range(p.B):
+        want_k = torch.stack([p.keys[b, h] for h in range(p.H)]).to(torch.bfloat16)
+        want_v = torch.stack([p.values[b, h] for h in range(p.H)]).to(torch.bfloat16)
+        k, v = ops.paged_gather_range(kv, b, 0, p.lens[b])
+        assert torch.equal(k.cpu(), want_k) and torch.equal(v.cpu(), want_v)
+        k, v = ops.paged_gather_range(kv, b, 37, 150)
+        assert torch.equal(k.cpu(), want_k[:, 37:150]) and torch.equal(v.cpu(), want_v[:, 37:150])
+        pos = torch.randint(0, p.lens[b], (p.H, 2, 11), generator=torch.Generator().manual_seed(b))
+        k, v = ops.paged_gather_at(kv, b, pos.to(dev))
+        for h in range(p.H):
+            assert torch.equal(k[h].cpu(), want_k[h][pos[h]]) and torch.equal(v[h].cpu(), want_v[h][pos[h]])
+
+
+def test_missing_or_bad_arguments_fail_loudly():
+    dev = _cuda()
+    p = Problem(lens=[300], heads=1, lists=8, seed=29)
+    idx = p.device_index(dev)
+    with pytest.raises(ValueError):
+        ops.lut_build(torch.zeros(1, 1, 64, device=dev), idx, 1)            # wrong head dim
+    with pytest.raises(ValueError):
+        ops.kv_contiguous(torch.zeros(1, 1, 8, 128), torch.zeros(1, 1, 8, 128))   # CPU tensors
+    with pytest.raises(ValueError):
+        ops.lut_build(torch.zeros(1, 17, 128, device=dev), idx, 17)         # G too large
