@@ -1,0 +1,298 @@
+#!/usr/bin/env python3
+"""PQ-HSA decode-attention benchmark: one step = one layer's single-token decode attention
+over one batch of synthetic sequences resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2]
+
+Prints ONE JSON line: decode-attention microseconds per layer on the headline configuration
+(Llama-3-8B-shape layer, 131 072-token context, batch 4, bf16 paged K/V), the HBM roofline of
+the dominant kernel from HIP-event timings taken on the launch stream, and the torch-CPU
+restatement of the reference path timed on this box's host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MODEL_LAYERS = 32  # Llama-3-8B depth, for the tokens/s figure
+
+CONFIGS = {
+    # name: (description, batch, kv_heads, groups, ctx or (lo, hi), dtype, paged, shuffled blocks)
+    0: ("cfg0: single KV head, single query, ctx 8192, fp32", 1, 1, 1, 8192, torch.float32, False, False),
+    1: ("cfg1: Llama-3-8B-shape layer, batch 1, ctx 32768, bf16 paged (block 16)", 1, 8, 4, 32768,
+        torch.bfloat16, True, True),
+    2: ("cfg2: Llama-3-8B-shape layer, batch 4, ctx 131072, bf16 paged (block 16)", 4, 8, 4, 131072,
+        torch.bfloat16, True, True),
+    3: ("cfg3: ragged batch 16, ctx U[16K,64K], bf16 paged, shuffled blocks", 16, 8, 4, (16384, 65536),
+        torch.bfloat16, True, True),
+    4: ("cfg4: GQA-7 layer, batch 1, ctx 262144, bf16 paged", 1, 4, 7, 262144, torch.bfloat16, True, True),
+}
+SINK, LOCAL, FRACTION, LISTS, BLOCK = 4, 64, 0.02, 512, 16
+KERNELS = ["lut_build", "scan_hist", "thresh", "scan_emit", "select_final", "attend_partial", "attend_reduce"]
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_stream(ctx, groups, seed, device, dtype):
+    """Seeded keys/values/queries of one (sequence, KV head), drawn on the device generator."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    dim = 128
+    centres = torch.randn(512, dim, generator=gen, device=device)
+    member = torch.randint(0, 512, (ctx,), generator=gen, device=device)
+    keys = centres[member] + 0.3 * torch.randn(ctx, dim, generator=gen, device=device)
+    scale = torch.exp(0.5 * torch.randn(dim, generator=gen, device=device))
+    outliers = torch.randperm(dim, generator=gen, device=device)[:4]
+    scale[outliers] *= 8.0
+    keys = keys * scale
+    values = torch.randn(ctx, dim, generator=gen, device=device)
+    needle = torch.randint(8, max(9, ctx - 128), (groups,), generator=gen, device=device)
+    queries = keys[needle] + 0.2 * torch.randn(groups, dim, generator=gen, device=device)
+    return keys.to(dtype), values.to(dtype), queries.to(dtype)
+
+
+class Layer:
+    """One layer's resident state: K/V (paged or dense), trained + encoded index, queries."""
+
+    def __init__(self, cfg_id, seed0, device):
+        from pqhsa_release_amd import ops
+        from pqhsa_release_amd.index.train import train_ivfpq
+
+        desc, B, H, G, ctx, dtype, paged, shuffled = CONFIGS[cfg_id]
+        self.B, self.H, self.G, self.dtype = B, H, G, dtype
+        gen = torch.Generator().manual_seed(seed0)
+        if isinstance(ctx, tuple):
+            self.lens = [int(x) for x in torch.randint(ctx[0], ctx[1] + 1, (B,), generator=gen)]
+        else:
+            self.lens = [ctx] * B
+        self.n = [max(SINK, ln - LOCAL) - SINK for ln in self.lens]
+        n_max = max(self.n)
+        self.index = ops.DeviceIndex(B, H, LISTS, n_max + 256, device)
+        if paged:
+            blocks_per = [(ln + BLOCK - 1) // BLOCK for ln in self.lens]
+            total = sum(blocks_per)
+            order = torch.randperm(total, generator=gen) if shuffled else torch.arange(total)
+            table = torch.zeros(B, max(blocks_per), dtype=torch.int32)
+            at = 0
+            for b, nb in enumerate(blocks_per):
+                table[b, :nb] = order[at : at + nb].to(torch.int32)
+                at += nb
+            self.block_table = table.to(device)
+            self.cache = torch.zeros(2, total, BLOCK, H, 128, dtype=dtype, device=device)
+            self.kv = ops.kv_paged(self.cache, self.block_table)
+        else:
+            self.keys = torch.zeros(B, H, max(self.lens), 128, dtype=dtype, device=device)
+            self.values = torch.zeros_like(self.keys)
+            self.kv = ops.kv_contiguous(self.keys, self.values)
+        q = torch.empty(B, H * G, 128, dtype=dtype, device=device)
+        for b, ln in enumerate(self.lens):
+            pos = torch.arange(ln, device=device)
+            for h in range(H):
+                k, v, qq = make_stream(ln, G, seed0 + 1000 * b + h, device, dtype)
+                if paged:
+                    blk = self.block_table[b, pos // BLOCK].long()
+                    self.cache[0, blk, pos % BLOCK, h] = k
+                    self.cache[1, blk, pos % BLOCK, h] = v
+                else:
+                    self.keys[b, h, :ln] = k
+                    self.values[b, h, :ln] = v
+                q[b, h * G : (h + 1) * G] = qq
+                coarse, books = train_ivfpq(k[SINK : SINK + self.n[b]], num_lists=LISTS, coarse_iter=1, pq_iter=2,
+                                            seed=0)
+                self.index.coarse[b * H + h, : coarse.shape[0]] = coarse
+                self.index.codebooks[b * H + h] = books
+                del k, v
+        self.q = q
+        self.out = torch.empty_like(q)
+        self.index.set_counts(self.n)
+        ops.encode(self.kv, self.index, SINK, [0] * B, self.n)
+        ops.value_summaries(self.kv, self.index, SINK)
+        self.seq_lens = torch.tensor(self.lens, dtype=torch.int32, device=device)
+        k_cap = ops.resolve_topk(n_max, FRACTION, 0)
+        self.ws = ops.DecodeWorkspace(self.index, G, k_cap)
+        self.call = ops.DecodeCall(self.q, self.out, self.kv, self.index, G, self.seq_lens, sink=SINK,
+                                   full_max=SINK + LOCAL, fraction=FRACTION, topk=0, scale=1.0 / math.sqrt(128),
+                                   workspace=self.ws)
+        torch.cuda.synchronize()
+
+    def algorithmic_bytes(self):
+        """Bytes each kernel must touch per launch (10 B per indexed key-head, tables, selected and
+        full K/V rows, list means)."""
+        e = 4 if self.dtype == torch.float32 else 2
+        scan = sum(self.H * n * 10 for n in self.n)
+        tables = self.B * self.H * (LISTS * 128 + 8 * 16 * 16) * 4
+        exact = sum(self.H * self.G * math.ceil(n * FRACTION) * 2 * 128 * e for n in self.n)
+        full = sum(self.H * (min(SINK, ln) + ln - (SINK + n)) * 2 * 128 * e for ln, n in zip(self.lens, self.n))
+        bg = self.B * self.H * LISTS * 128 * 4
+        return {"scan": scan, "tables": tables, "exact": exact, "full": full, "bg": bg,
+                "total": scan + tables + exact + full + bg}
+
+
+def cpu_baseline(layer, seconds=12.0):
+    """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
+    the same inputs and trained index, and scale to the whole layer."""
+    from oracle import torch_ref as tr
+    from pqhsa_release_amd import ops
+
+    b = h = 0
+    bh, n, ln, G = 0, layer.n[0], layer.lens[0], layer.G
+    kk, vv = ops.paged_gather_range(layer.kv, b, 0, ln) if layer.kv.view.paged else (layer.keys[b], layer.values[b])
+    keys, values = kk[h].float().cpu(), vv[h].float().cpu()
+    idx = layer.index
+    ref = tr.RefIndex(idx.coarse[bh].cpu(), idx.codebooks[bh].cpu(), idx.list_ids_long()[bh, :n].cpu(),
+                      idx.packed_bytes()[bh, :n].cpu().clone(), idx.norms[bh, :n].cpu())
+    vbar = idx.vbar[bh].cpu()
+    q = layer.q[b, h * G : (h + 1) * G].float().cpu()
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    args = dict(sink_end=SINK, retrieval_end=SINK + n, index=ref, vbar=vbar, fraction=FRACTION,
+                scale=1.0 / math.sqrt(128))
+    out = tr.hybrid_forward_many(q, keys, values, **args)
+    t0, reps = time.perf_counter(), 0
+    while True:
+        tr.hybrid_forward_many(q, keys, values, **args)
+        reps += 1
+        if time.perf_counter() - t0 > seconds and reps >= 3:
+            break
+    per_stream = (time.perf_counter() - t0) / reps
+    got = layer.out[b, h * G : (h + 1) * G].float().cpu()
+    err = float((got - out).abs().max())
+    streams = sum(1 for _ in range(layer.B * layer.H))
+    scale_factor = sum(layer.n) * layer.H / max(n, 1)  # streams weighted by their indexed length
+    return {
+        "value": per_stream * scale_factor * 1e6,
+        "unit": "us/layer",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"torch-CPU restatement of forward_many on 1 of {streams} (sequence, KV head) streams "
+                  f"(n={n}, G={G}), {reps} reps, scaled by indexed keys to the whole layer",
+        "max_abs_diff_vs_gpu": err,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--layers", type=int, default=3, help="distinct resident layers rotated through (defeats cache reuse)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (every sequence and KV head of the layer is on it); "
+                 "--gpus must be 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the PQ-HSA kernels have no CPU path")
+
+    from pqhsa_release_amd import _lib
+
+    lib = _lib.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    t_setup = time.perf_counter()
+    layers = [Layer(args.config, 100 + 7919 * i, device) for i in range(max(1, args.layers))]
+    log(f"setup {time.perf_counter() - t_setup:.1f}s: {CONFIGS[args.config][0]}, {len(layers)} resident layers")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run_steps(count, offset=0):
+        for i in range(count):
+            layers[(i + offset) % len(layers)].call.run(stream)
+
+    run_steps(args.warmup)
+    torch.cuda.synchronize()
+    # timed region: exactly --steps steps, with the per-kernel event log recording on the stream
+    _lib.check(lib.pqhsa_profile_enable(args.steps), "pqhsa_profile_enable")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(args.steps)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kms = (ctypes.c_float * len(KERNELS))()
+    seen = ctypes.c_int32(0)
+    _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
+    ms_per_step = (t1 - t0) * 1000.0 / args.steps
+    # the same steps without the event log, to show what the log costs
+    run_steps(args.warmup)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    run_steps(args.steps)
+    torch.cuda.synchronize()
+    ms_plain = (time.perf_counter() - t2) * 1000.0 / args.steps
+
+    layer = layers[0]
+    ab = layer.algorithmic_bytes()
+    kus = {name: float(kms[i]) * 1000.0 for i, name in enumerate(KERNELS)}
+    algo = {"lut_build": ab["tables"], "scan_hist": ab["scan"], "scan_emit": ab["scan"], "thresh": 0,
+            "select_final": 0, "attend_partial": ab["exact"] + ab["full"], "attend_reduce": ab["bg"]}
+    kernels = {}
+    for name in KERNELS:
+        us = kus[name]
+        kernels[name] = {"us": round(us, 3), "algo_MB": round(algo[name] / 1e6, 3),
+                         "GBps": round(algo[name] / 1e3 / us, 1) if us > 0 else None}
+    dominant = max(KERNELS, key=lambda k: kus[k])
+    dom_bytes = algo[dominant]
+    roofline = {
+        "kernel": dominant,
+        "bound": "hbm",
+        "achieved": round(dom_bytes / 1e3 / kus[dominant], 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(dom_bytes / 1e3 / kus[dominant] / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "algorithmic_bytes": dom_bytes,
+        "launch_us": round(kus[dominant], 3),
+    }
+    scan_us = kus["scan_hist"] + kus["scan_emit"]
+    result = {
+        "metric": "decode attn us/layer at 128K ctx (8 KV heads); LUT-scan HBM GB/s vs peak",
+        "value": round(ms_per_step * 1000.0, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": CONFIGS[args.config][0], "batch": layer.B, "kv_heads": layer.H,
+                   "gqa_group": layer.G, "context": layer.lens if len(set(layer.lens)) > 1 else layer.lens[0],
+                   "num_lists": LISTS, "top_fraction": FRACTION, "sink": SINK, "local_window": LOCAL,
+                   "kv_dtype": str(layer.dtype).replace("torch.", ""), "resident_layers": len(layers)},
+        "roofline": roofline,
+        "tokens_per_s": round(layer.B / (MODEL_LAYERS * ms_per_step / 1000.0), 1),
+        "step_bytes_MB": round(ab["total"] / 1e6, 2),
+        "step_roofline_frac": round(ab["total"] / 1e3 / (ms_per_step * 1000.0) / HBM_PEAK_GBPS, 4),
+        "lut_scan": {"us_two_passes": round(scan_us, 3), "algo_MB": round(ab["scan"] / 1e6, 3),
+                     "GBps": round(ab["scan"] / 1e3 / scan_us, 1) if scan_us > 0 else None,
+                     "frac_of_peak": round(ab["scan"] / 1e3 / scan_us / HBM_PEAK_GBPS, 4) if scan_us > 0 else None},
+        "kernels": kernels,
+        "kernel_sum_us": round(sum(kus.values()), 3),
+        "ms_per_step_without_event_log": round(ms_plain, 6),
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(layer, args.cpu_seconds)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

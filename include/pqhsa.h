@@ -221,6 +221,19 @@ int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq,
                           const int64_t *positions, int64_t count, void *out_k, void *out_v,
                           void *stream);
 
+/*
+ * Per-kernel timing of pqhsa_decode_step with HIP events recorded on the caller's stream and
+ * read back only at collect time (the sync-free event log of the reference,
+ * benchmarks/cuda_event_log.py:49-88).  pqhsa_profile_enable creates events for up to
+ * max_steps decode steps; pqhsa_profile_collect synchronises the recorded events, writes the
+ * average milliseconds of the 7 kernels (lut_build, scan_hist, thresh, scan_emit,
+ * select_final, attend_partial, attend_reduce) and the number of steps seen, and turns
+ * profiling off.  Not thread-safe; meant for benchmarks.
+ */
+#define PQHSA_PROFILE_KERNELS 7
+int pqhsa_profile_enable(int32_t max_steps);
+int pqhsa_profile_collect(float *kernel_ms, int32_t *steps);
+
 #ifdef __cplusplus
 }
 #endif

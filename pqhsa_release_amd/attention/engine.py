@@ -1,0 +1,334 @@
+"""Device-side state of PQ-HSA decode attention for a batch of sequences.
+
+``PQHSAEngine`` owns what the reference spreads over ``SparseKVCache`` + ``IVFPQIndex`` +
+``IVFPQSparseAttention`` for every (sequence, KV head) stream
+(pq_hsa/attention/kv_cache.py:68-314, 1160-1201; pq_hsa/index/ivfpq.py:275-433, 598-707;
+pq_hsa/attention/sparse_attention.py:219-335): the sink / retrieval / local region
+bookkeeping, the trained index and its per-step updates, and the forward call.  All
+arithmetic runs in the HIP kernels behind ``pqhsa_release_amd.ops``; torch supplies memory
+and the few small tensor updates of the (off-hot-path) codebook refresh.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import ops
+from ..config import IVFPQConfig, SparseAttentionConfig, validate_for_kernels
+from ..index.train import train_ivfpq
+
+D = ops.HEAD_DIM
+
+
+class PQHSAEngine:
+    def __init__(self, index_config: IVFPQConfig, attention_config: SparseAttentionConfig, *, batch: int,
+                 kv_heads: int, device, growth_margin: int = 4096) -> None:
+        validate_for_kernels(index_config, attention_config)
+        self.index_config, self.attention_config = index_config, attention_config
+        self.B, self.H = int(batch), int(kv_heads)
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("PQ-HSA decode attention needs a GPU: the MI355X kernels have no CPU path")
+        self.growth_margin = int(growth_margin)
+        self.sink, self.local = attention_config.sink_tokens, attention_config.local_window
+        self.kv: ops.KvSource | None = None
+        self.keys_buf = self.values_buf = None      # dense storage owned by the engine (optional)
+        self.index: ops.DeviceIndex | None = None
+        self.lens = [0] * self.B                    # tokens in the cache
+        self.indexed_len = [0] * self.B             # tokens visible to the index bookkeeping
+        self.pending = [0] * self.B                 # appended since the last index update
+        self.deferred_pending = False
+        self.seq_lens = torch.zeros(self.B, dtype=torch.int32, device=self.device)
+        self._ws: dict[int, ops.DecodeWorkspace] = {}
+        self.index_adds = self.index_rebuilds = self.online_codebook_updates = self.deferred_index_updates = 0
+
+    # ------------------------------------------------------------------ regions
+    def _sink_end(self, b: int) -> int:
+        return min(self.sink, self.lens[b])
+
+    def _retrieval_end(self, b: int) -> int:
+        s = self._sink_end(b)
+        idx_len = min(self.indexed_len[b], self.lens[b])
+        return max(s, idx_len - self.local) if self.local > 0 else max(s, idx_len)
+
+    def n(self, b: int) -> int:
+        """Indexed (retrieval-region) keys of sequence b."""
+        return self._retrieval_end(b) - self._sink_end(b)
+
+    def full_count(self, b: int) -> int:
+        return self._sink_end(b) + self.lens[b] - self._retrieval_end(b)
+
+    # ------------------------------------------------------------------ storage
+    def bind_dense(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Use caller-provided ``[B, H, cap, 128]`` tensors as the K/V store."""
+        self.kv = ops.kv_contiguous(keys, values)
+        self.keys_buf, self.values_buf = keys, values
+
+    def bind_paged(self, kv_cache: torch.Tensor, block_table: torch.Tensor) -> None:
+        """Read K/V rows in place from a paged cache; the engine keeps no copy of its own."""
+        self.kv = ops.kv_paged(kv_cache, block_table)
+        self.keys_buf = self.values_buf = None
+
+    def adopt(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Copy ``[B, H, S, 128]`` K/V into an engine-owned buffer with spare capacity."""
+        b, h, s, _ = keys.shape
+        cap = s + self.growth_margin
+        kb = torch.empty(b, h, cap, D, dtype=keys.dtype, device=self.device)
+        vb = torch.empty_like(kb)
+        kb[:, :, :s].copy_(keys)
+        vb[:, :, :s].copy_(values)
+        self.bind_dense(kb, vb)
+
+    def _grow_dense(self, need: int) -> None:
+        cap = self.keys_buf.shape[2]
+        if need <= cap:
+            return
+        new_cap = need + self.growth_margin
+        kb = torch.empty(self.B, self.H, new_cap, D, dtype=self.keys_buf.dtype, device=self.device)
+        vb = torch.empty_like(kb)
+        kb[:, :, :cap].copy_(self.keys_buf)
+        vb[:, :, :cap].copy_(self.values_buf)
+        self.bind_dense(kb, vb)
+
+    def write_rows(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Store one new ``[B, H, 128]`` K/V row per sequence at its current length (dense store)."""
+        if self.keys_buf is None:
+            return  # paged: the owner of the cache has already written the row
+        self._grow_dense(max(self.lens) + 1)
+        if len(set(self.lens)) == 1:
+            self.keys_buf[:, :, self.lens[0]].copy_(keys)
+            self.values_buf[:, :, self.lens[0]].copy_(values)
+        else:
+            for b, ln in enumerate(self.lens):
+                self.keys_buf[b, :, ln].copy_(keys[b])
+                self.values_buf[b, :, ln].copy_(values[b])
+
+    # ------------------------------------------------------------------ index
+    def _effective_lists(self) -> int:
+        smallest = min((self.n(b) for b in range(self.B) if self.n(b) > 0), default=1)
+        return max(1, min(self.index_config.num_lists, smallest))
+
+    def _alloc_index(self, n_need: int, num_lists: int) -> None:
+        old = self.index
+        self.index = ops.DeviceIndex(self.B, self.H, num_lists, n_need + self.growth_margin, self.device)
+        self._ws.clear()
+        if old is not None and old.num_lists == num_lists:
+            keep = min(old.n_cap, self.index.n_cap)
+            for name in ("codes", "list_ids", "norms"):
+                getattr(self.index, name)[:, :keep].copy_(getattr(old, name)[:, :keep])
+            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+                getattr(self.index, name).copy_(getattr(old, name))
+
+    def _retrieval_keys(self, b: int, h: int, start: int, count: int) -> torch.Tensor:
+        s = self._sink_end(b)
+        if self.keys_buf is not None:
+            return self.keys_buf[b, h, s + start : s + start + count]
+        k, _ = ops.paged_gather_range(self.kv, b, s + start, s + start + count)
+        return k[h]
+
+    def build(self, lens, *, coarse: torch.Tensor | None = None, codebooks: torch.Tensor | None = None) -> None:
+        """(Re)build the index over the retrieval region of every sequence.  Without
+        ``coarse``/``codebooks`` (``[BH, L, 128]`` / ``[BH, 8, 16, 16]`` or one set shared by all
+        streams) each stream trains its own (IVFPQIndex.build); with them this is
+        ``build_with_codebooks``."""
+        if self.kv is None:
+            raise RuntimeError("bind K/V storage before building the index")
+        self.lens = [int(x) for x in lens]
+        self.indexed_len = list(self.lens)
+        self.pending = [0] * self.B
+        self.deferred_pending = False
+        counts = [self.n(b) for b in range(self.B)]
+        lists = self._effective_lists() if coarse is None else int(coarse.shape[-2])
+        self.index = None
+        self._alloc_index(max(counts), lists)
+        ic = self.index_config
+        if coarse is None:
+            paged_cache = {}
+            for b in range(self.B):
+                if counts[b] == 0:
+                    continue
+                if self.keys_buf is None:
+                    s = self._sink_end(b)
+                    paged_cache[b], _ = ops.paged_gather_range(self.kv, b, s, s + counts[b])
+                for h in range(self.H):
+                    rows = (self.keys_buf[b, h, self._sink_end(b) : self._sink_end(b) + counts[b]]
+                            if self.keys_buf is not None else paged_cache[b][h])
+                    c, cb = train_ivfpq(rows, num_lists=lists, coarse_iter=ic.coarse_max_iter,
+                                        pq_iter=ic.pq_max_iter, seed=ic.seed, eps=ic.eps)
+                    self.index.coarse[b * self.H + h, : c.shape[0]].copy_(c)
+                    self.index.codebooks[b * self.H + h].copy_(cb)
+                paged_cache.pop(b, None)
+        else:
+            self.index.coarse.copy_(coarse.to(self.device, torch.float32).expand_as(self.index.coarse))
+            self.index.codebooks.copy_(codebooks.to(self.device, torch.float32).expand_as(self.index.codebooks))
+        self.index.set_counts(counts)
+        if max(counts) > 0:
+            ops.encode(self.kv, self.index, self.sink, [0] * self.B, counts, eps=ic.eps)
+            ops.value_summaries(self.kv, self.index, self.sink)
+        self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
+        self.index_rebuilds += 1
+
+    def _ensure_capacity(self, n_need: int) -> None:
+        if n_need > self.index.n_cap:
+            counts = list(self.index.n_host)
+            self._alloc_index(n_need, self.index.num_lists)
+            self.index.set_counts(counts)
+
+    def advance(self, count: int = 1) -> None:
+        """Bookkeeping after ``count`` tokens were appended to every sequence
+        (SparseKVCache.append, pq_hsa/attention/kv_cache.py:195-226)."""
+        ac = self.attention_config
+        for b in range(self.B):
+            self.lens[b] += count
+            self.pending[b] += count
+        self.seq_lens += count
+        if max(self.pending) >= ac.index_update_interval:
+            if ac.index_update_strategy == "deferred":
+                if not self.deferred_pending:
+                    self.deferred_index_updates += 1
+                self.deferred_pending = True
+            else:
+                self._refresh_index_now()
+
+    def apply_pending_index_update(self) -> bool:
+        if not self.deferred_pending:
+            return False
+        self._refresh_index_now()
+        self.deferred_pending = False
+        return True
+
+    def _refresh_index_now(self) -> None:
+        """SparseKVCache._refresh_index_now (pq_hsa/attention/kv_cache.py:276-314)."""
+        strategy = self.attention_config.index_update_strategy
+        if strategy == "rebuild" or self.index is None or self.index.n_max == 0:
+            self.build(self.lens)
+            return
+        old = [self.n(b) for b in range(self.B)]
+        self.indexed_len = list(self.lens)
+        self.pending = [0] * self.B
+        new = [self.n(b) for b in range(self.B)]
+        added = [n1 - n0 for n0, n1 in zip(old, new)]
+        if max(added) <= 0:
+            return
+        self._ensure_capacity(max(new))
+        if strategy in {"online", "deferred"}:
+            self._online_refresh(old, added)
+            self.online_codebook_updates += 1
+        else:
+            ops.encode_append(self.kv, self.index, self.sink, old, added, eps=self.index_config.eps)
+            self.index_adds += 1
+        self.index.set_counts(new)
+
+    def _online_refresh(self, old, added) -> None:
+        """EMA move of the coarse centroids and PQ codewords towards the newly indexed keys, then
+        re-encode every indexed key (IVFPQIndex.online_refresh, pq_hsa/index/ivfpq.py:647-707;
+        ProductQuantizer.update_codebooks_ema, pq_hsa/index/pq.py:117-173).  The assignments come
+        from the HIP encode kernel; the small per-list means are torch ops on the device."""
+        ic, idx = self.index_config, self.index
+        lr = ic.online_codebook_lr
+        ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # lists of the new rows
+        for b in range(self.B):
+            if added[b] <= 0:
+                continue
+            for h in range(self.H):
+                bh = b * self.H + h
+                rows = self._retrieval_keys(b, h, old[b], added[b]).float()
+                dirs = rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
+                lids = idx.list_ids_long()[bh, old[b] : old[b] + added[b]]
+                _ema_rows(idx.coarse[bh], dirs, lids, lr, ic.eps)
+        ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # re-assign with moved lists
+        for b in range(self.B):
+            if added[b] <= 0:
+                continue
+            for h in range(self.H):
+                bh = b * self.H + h
+                rows = self._retrieval_keys(b, h, old[b], added[b]).float()
+                dirs = rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
+                sl = slice(old[b], old[b] + added[b])
+                lids = idx.list_ids_long()[bh, sl]
+                resid = (dirs - idx.coarse[bh][lids]).reshape(-1, ops.SUBSPACES, ops.SUBDIM)
+                words = idx.codes[bh, sl].to(torch.int64) & 0xFFFFFFFF
+                for m in range(ops.SUBSPACES):
+                    _ema_rows(idx.codebooks[bh, m], resid[:, m], (words >> (4 * m)) & 15, lr, ic.eps)
+        new = [o + a for o, a in zip(old, added)]
+        idx.set_counts(new)
+        ops.encode(self.kv, idx, self.sink, [0] * self.B, new, eps=ic.eps)
+        ops.value_summaries(self.kv, idx, self.sink)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, q: torch.Tensor, groups: int, out: torch.Tensor | None = None) -> torch.Tensor:
+        """q ``[B, H*groups, 128]`` -> context of the same shape and dtype."""
+        if self.index is None:
+            raise RuntimeError("build_cache must be called before forward")
+        ac = self.attention_config
+        if q.dtype != self.kv.dtype and q.dtype != torch.float32:
+            q = q.float()
+        q = q.contiguous()
+        if out is None:
+            out = torch.empty_like(q)
+        ws = self._ws.get(groups)
+        k_cap = ops.resolve_topk(self.index.n_cap, ac.retrieval_top_fraction, ac.retrieval_topk)
+        if ws is None or ws.k_cap < k_cap:
+            ws = self._ws[groups] = ops.DecodeWorkspace(self.index, groups, k_cap)
+        scale = (1.0 / math.sqrt(D)) if ac.scale is None else float(ac.scale)
+        full_max = max(self.full_count(b) for b in range(self.B))
+        ops.decode_step(q, out, self.kv, self.index, groups, self.seq_lens, sink=self.sink, full_max=full_max,
+                        fraction=ac.retrieval_top_fraction, topk=ac.retrieval_topk, scale=scale, workspace=ws,
+                        eps=self.index_config.eps)
+        return out
+
+    def last_topk(self, groups: int):
+        """(indices, logits, counts) of the most recent forward for ``groups`` rows per KV head."""
+        ws = self._ws[groups]
+        return ws.topk_idx, ws.topk_val, ws.topk_cnt
+
+    # ------------------------------------------------------------------ checkpoint
+    def state_dict(self) -> dict[str, object]:
+        idx = self.index
+        state: dict[str, object] = {
+            "lens": list(self.lens), "indexed_len": list(self.indexed_len), "pending": list(self.pending),
+            "deferred_pending": self.deferred_pending, "batch": self.B, "kv_heads": self.H,
+        }
+        if idx is not None:
+            state["index"] = {name: getattr(idx, name).detach().clone() for name in
+                              ("codes", "list_ids", "norms", "coarse", "codebooks", "vbar", "vsum", "vcount")}
+            state["index_counts"] = list(idx.n_host)
+            state["num_lists"] = idx.num_lists
+        if self.keys_buf is not None:
+            top = max(self.lens)
+            state["keys"] = self.keys_buf[:, :, :top].detach().clone()
+            state["values"] = self.values_buf[:, :, :top].detach().clone()
+        return state
+
+    def load_state_dict(self, state: dict[str, object]) -> None:
+        if int(state["batch"]) != self.B or int(state["kv_heads"]) != self.H:
+            raise ValueError("state does not match the engine's batch / KV heads")
+        self.lens = [int(x) for x in state["lens"]]
+        self.indexed_len = [int(x) for x in state["indexed_len"]]
+        self.pending = [int(x) for x in state["pending"]]
+        self.deferred_pending = bool(state["deferred_pending"])
+        if "keys" in state:
+            self.adopt(state["keys"].to(self.device), state["values"].to(self.device))
+        if "index" in state:
+            tensors = state["index"]
+            self.index = None
+            self._alloc_index(max(int(c) for c in state["index_counts"]), int(state["num_lists"]))
+            keep = min(self.index.n_cap, tensors["codes"].shape[1])
+            for name in ("codes", "list_ids", "norms"):
+                getattr(self.index, name)[:, :keep].copy_(tensors[name][:, :keep])
+            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+                getattr(self.index, name).copy_(tensors[name])
+            self.index.set_counts(state["index_counts"])
+        self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
+
+
+def _ema_rows(table: torch.Tensor, vectors: torch.Tensor, assign: torch.Tensor, lr: float, eps: float) -> None:
+    """table[j] <- (1 - lr) * table[j] + lr * mean(vectors assigned to j), for non-empty j."""
+    sums = torch.zeros_like(table)
+    sums.index_add_(0, assign, vectors.to(table.dtype))
+    counts = torch.bincount(assign, minlength=table.shape[0]).to(table.dtype)
+    filled = counts > 0
+    means = sums[filled] / counts[filled].unsqueeze(1).clamp_min(eps)
+    table[filled] = (1.0 - lr) * table[filled] + lr * means

@@ -1,6 +1,7 @@
 // Error plumbing, version string and argument validation shared by the C-ABI entry points.
 #include <cstdarg>
 #include <cstdio>
+#include <vector>
 
 #include "common.h"
 
@@ -45,7 +46,67 @@ int validate_view(const pqhsa_kv_view *kv) {
     return PQHSA_OK;
 }
 
+// ---- optional per-kernel event log of pqhsa_decode_step -------------------------------
+// Events are created up front and only recorded on the caller's stream while decode steps
+// run; nothing synchronises until pqhsa_profile_collect.
+static std::vector<hipEvent_t> g_events;
+static int g_prof_steps = 0, g_prof_step = 0;
+static bool g_prof_on = false;
+
+void profile_mark(int slot, hipStream_t stream) {
+    if (!g_prof_on || g_prof_step >= g_prof_steps) return;
+    (void)hipEventRecord(g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot], stream);
+    if (slot == kProfKernels) ++g_prof_step;
+}
+
 }  // namespace pqhsa
+
+extern "C" int pqhsa_profile_enable(int32_t max_steps) {
+    using namespace pqhsa;
+    PQHSA_REQUIRE(max_steps > 0 && max_steps <= 100000, "profile_enable: max_steps=%d", max_steps);
+    for (hipEvent_t e : g_events) (void)hipEventDestroy(e);
+    g_events.assign((size_t)max_steps * (kProfKernels + 1), nullptr);
+    for (auto &e : g_events) {
+        if (hipEventCreate(&e) != hipSuccess) {
+            set_error("profile_enable: hipEventCreate failed");
+            return PQHSA_ELAUNCH;
+        }
+    }
+    g_prof_steps = max_steps;
+    g_prof_step = 0;
+    g_prof_on = true;
+    return PQHSA_OK;
+}
+
+extern "C" int pqhsa_profile_collect(float *kernel_ms, int32_t *steps) {
+    using namespace pqhsa;
+    PQHSA_REQUIRE(kernel_ms && steps, "profile_collect: NULL argument");
+    g_prof_on = false;
+    const int n = g_prof_step;
+    *steps = n;
+    for (int k = 0; k < kProfKernels; ++k) kernel_ms[k] = 0.0f;
+    for (int s = 0; s < n; ++s) {
+        hipEvent_t *ev = &g_events[(size_t)s * (kProfKernels + 1)];
+        if (hipEventSynchronize(ev[kProfKernels]) != hipSuccess) {
+            set_error("profile_collect: event synchronize failed");
+            return PQHSA_ELAUNCH;
+        }
+        for (int k = 0; k < kProfKernels; ++k) {
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, ev[k], ev[k + 1]) != hipSuccess) {
+                set_error("profile_collect: elapsed time failed");
+                return PQHSA_ELAUNCH;
+            }
+            kernel_ms[k] += ms;
+        }
+    }
+    if (n > 0)
+        for (int k = 0; k < kProfKernels; ++k) kernel_ms[k] /= (float)n;
+    for (hipEvent_t e : g_events) (void)hipEventDestroy(e);
+    g_events.clear();
+    g_prof_steps = g_prof_step = 0;
+    return PQHSA_OK;
+}
 
 extern "C" const char *pqhsa_version(void) { return "pqhsa-mi355x 0.1 (gfx950)"; }
 

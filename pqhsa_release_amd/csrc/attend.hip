@@ -326,9 +326,11 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
 #undef PQHSA_ATT
     int rc = check_launch("attend_partial");
     if (rc) return rc;
+    if (a.subtract_selected == 0) profile_mark(kProfReduce, stream);
     const size_t lds2 = (size_t)a.L * sizeof(float);
     PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kAttThreads), lds2,
                                                      stream, a));
+    if (a.subtract_selected == 0) profile_mark(kProfKernels, stream);
     return check_launch("attend_reduce");
 }
 

@@ -21,6 +21,9 @@ constexpr int kWave = 64;
 // ---- host-side error plumbing -------------------------------------------------------
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+// Records the next profiling event on `stream` when profiling is enabled (no-op otherwise).
+void profile_mark(int slot, hipStream_t stream);
+enum { kProfLut = 0, kProfHist, kProfThresh, kProfEmit, kProfSelect, kProfAttend, kProfReduce, kProfKernels };
 
 #define PQHSA_REQUIRE(cond, ...)            \
     do {                                    \

@@ -116,8 +116,10 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     if (!topk_val) topk_val = c.topk_val;
     if (!topk_cnt) topk_cnt = c.topk_cnt;
 
+    profile_mark(kProfLut, stream);
     rc = launch_lut_build(q, q_dtype, index, G, eps, c.qnorm, c.lut, c.ls, c.hist, c.zero_words, stream);
     if (rc) return rc;
+    profile_mark(kProfHist, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.hist, c.rowmax, c.emit_count,
                             c.thr_bin, c.thr_above, c.k_row, c.row_max_f, c.pairs, c.mass_partial, c.tile_keys,
                             topk_idx, topk_val, topk_cnt, stream);

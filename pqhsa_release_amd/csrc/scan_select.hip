@@ -667,9 +667,11 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.hist = hist; a.rowmax = rowmax;
     int rc = launch_scan(a, kHist, kIndex, GP, streams, n_max, stream);
     if (rc) return rc;
+    profile_mark(kProfThresh, stream);
     rc = launch_thresh(hist, rowmax, index->n_idx, index->kv_heads * GP, GP, G, select->fraction, select->topk,
                        nullptr, thr_bin, thr_above, k_row, row_max_f, streams * GP, stream);
     if (rc) return rc;
+    profile_mark(kProfEmit, stream);
     a.tile_keys = emit_tile_keys;
     a.tiles = (int)((index->n_cap + emit_tile_keys - 1) / emit_tile_keys);
     a.thr_bin = thr_bin; a.row_max_f = row_max_f; a.emit_count = emit_count;
@@ -677,6 +679,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.mass_partial = mass_partial; a.stage_cap = stage_cap_for(GP);
     rc = launch_scan(a, kEmit, kIndex, GP, streams, n_max, stream);
     if (rc) return rc;
+    profile_mark(kProfSelect, stream);
     SelectArgs s = {};
     s.pairs = static_cast<const uint2 *>(pairs); s.emit_cap = index->n_cap; s.emit_count = emit_count;
     s.thr_bin = thr_bin; s.thr_above = thr_above; s.k_row = k_row; s.n_arr = index->n_idx;
@@ -684,7 +687,9 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = topk_cnt; s.k_cap = select->k_cap;
     s.mass_extra = mass_partial; s.mass_slots = a.tiles + 1; s.mass_slot = a.tiles; s.L = index->num_lists;
     s.row_max_f = row_max_f; s.list_ids = index->list_ids; s.n_cap = index->n_cap;
-    return launch_select_final(s, streams, n_max, stream);
+    rc = launch_select_final(s, streams, n_max, stream);
+    profile_mark(kProfAttend, stream);
+    return rc;
 }
 
 }  // namespace pqhsa

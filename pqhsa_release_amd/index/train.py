@@ -1,0 +1,87 @@
+"""Index training (coarse k-means + per-subspace PQ k-means) with torch ops on the keys' device.
+
+Training happens once after prefill and is not part of the decode hot path; it produces the
+``coarse [L, D]`` / ``codebooks [M, 16, D/M]`` tensors that the HIP encode and scan kernels
+consume.  The procedure mirrors the reference's (pq_hsa/index/kmeans.py:134-227 seeded Lloyd
+iterations with empty-cluster reseeding; pq_hsa/index/ivfpq.py:275-348 coarse k-means on key
+directions, then PQ on the residuals with seed + 10000 + subspace; pq_hsa/index/pq.py:47-95).
+"""
+
+from __future__ import annotations
+
+import torch
+
+
+def _nearest(vectors: torch.Tensor, centroids: torch.Tensor, chunk: int = 32768) -> torch.Tensor:
+    cf = centroids.float()
+    half_sq = (cf * cf).sum(dim=1)
+    out = torch.empty(vectors.shape[0], dtype=torch.long, device=vectors.device)
+    for s in range(0, vectors.shape[0], chunk):
+        v = vectors[s : s + chunk].float()
+        out[s : s + chunk] = (half_sq.unsqueeze(0) - 2.0 * (v @ cf.t())).argmin(dim=1)
+    return out
+
+
+def kmeans_l2(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed: int = 0, eps: float = 1e-12,
+              initial_centroids: torch.Tensor | None = None):
+    """Lloyd iterations from a seeded random subset; returns ``(centroids, assignments)``."""
+    if vectors.ndim != 2:
+        raise ValueError(f"vectors must be [N, D], got {tuple(vectors.shape)}")
+    n, dim = vectors.shape
+    if n == 0:
+        raise ValueError("cannot train k-means with zero vectors")
+    if num_clusters <= 0:
+        raise ValueError("num_clusters must be positive")
+    gen = torch.Generator(device=vectors.device)
+    gen.manual_seed(int(seed))
+    if initial_centroids is not None:
+        if tuple(initial_centroids.shape) != (num_clusters, dim):
+            raise ValueError(f"initial_centroids must have shape ({num_clusters}, {dim})")
+        centroids = initial_centroids.to(device=vectors.device, dtype=vectors.dtype).clone()
+    elif n >= num_clusters:
+        centroids = vectors[torch.randperm(n, generator=gen, device=vectors.device)[:num_clusters]].clone()
+    else:
+        extra = torch.randint(0, n, (num_clusters - n,), generator=gen, device=vectors.device)
+        centroids = torch.cat([vectors, vectors[extra]], dim=0).clone()
+    assign = torch.zeros(n, dtype=torch.long, device=vectors.device)
+    for _ in range(max_iter):
+        nxt = _nearest(vectors, centroids)
+        same = torch.equal(assign, nxt)
+        assign = nxt
+        if same:
+            break
+        sums = torch.zeros(num_clusters, dim, dtype=torch.float32, device=vectors.device)
+        sums.index_add_(0, assign, vectors.float())
+        counts = torch.bincount(assign, minlength=num_clusters).float()
+        filled = counts > 0
+        sums[filled] /= counts[filled].unsqueeze(1).clamp_min(eps)
+        empty = ~filled
+        if bool(empty.any()):
+            pick = torch.randint(0, n, (int(empty.sum().item()),), generator=gen, device=vectors.device)
+            sums[empty] = vectors[pick].float()
+        centroids = sums.to(vectors.dtype)
+    return centroids, _nearest(vectors, centroids)
+
+
+def train_ivfpq(keys: torch.Tensor, *, num_lists: int, num_subspaces: int = 8, num_codes: int = 16,
+                coarse_iter: int = 1, pq_iter: int = 2, seed: int = 0, eps: float = 1e-12):
+    """Train one stream's index on its retrieval-region keys ``[N, D]`` (direction-normalised,
+    residual PQ).  Returns fp32 ``(coarse [L', D], codebooks [M, num_codes, D/M])`` with
+    ``L' = min(num_lists, N)``."""
+    if keys.ndim != 2 or keys.shape[0] == 0:
+        raise ValueError("cannot build IVF-PQ index with zero keys")
+    if keys.shape[1] % num_subspaces != 0:
+        raise ValueError(f"dim={keys.shape[1]} must be divisible by num_subspaces={num_subspaces}")
+    k32 = keys.float()
+    norms = torch.linalg.vector_norm(k32, dim=-1).clamp_min(eps)
+    dirs = k32 / norms.unsqueeze(-1)
+    lists = min(int(num_lists), dirs.shape[0])
+    coarse, assign = kmeans_l2(dirs, lists, max_iter=coarse_iter, seed=seed, eps=eps)
+    resid = dirs - coarse[assign]
+    sub = keys.shape[1] // num_subspaces
+    chunks = resid.reshape(resid.shape[0], num_subspaces, sub)
+    books = []
+    for m in range(num_subspaces):
+        c, _ = kmeans_l2(chunks[:, m].contiguous(), num_codes, max_iter=pq_iter, seed=seed + 10_000 + m, eps=eps)
+        books.append(c)
+    return coarse.float().contiguous(), torch.stack(books, dim=0).float().contiguous()

@@ -296,6 +296,43 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     return out
 
 
+class DecodeCall:
+    """A decode step with every argument resolved once: ``run()`` is one C call.
+
+    For steady-state loops whose tensors do not move (the serving loop, the bench): the
+    ctypes arguments are built at construction, so the per-step host cost is the foreign
+    call itself.  ``n_max``/``full_max`` may be updated between steps.
+    """
+
+    def __init__(self, q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int,
+                 full_max: int, fraction: float | None, topk: int, scale: float, workspace: DecodeWorkspace,
+                 eps: float = EPS, n_max: int | None = None) -> None:
+        _need_cuda(q, out, seq_lens)
+        if tuple(q.shape) != (index.batch, index.kv_heads * groups, HEAD_DIM) or not q.is_contiguous():
+            raise ValueError(f"q must be contiguous [B, H*G, {HEAD_DIM}], got {tuple(q.shape)}")
+        if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+            raise ValueError("out must match q in shape and dtype")
+        self._fn = _lib.load().pqhsa_decode_step
+        self._sel = Select()
+        self._sel.fraction = float(fraction) if fraction else 0.0
+        self._sel.topk = int(topk)
+        self._sel.k_cap = workspace.k_cap
+        self._keep = (q, out, kv, index, seq_lens, workspace)
+        self.n_max = index.n_max if n_max is None else int(n_max)
+        self.full_max = int(full_max)
+        self._head = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups,
+                      seq_lens.data_ptr(), int(sink))
+        self._tail = (ctypes.byref(self._sel), float(scale), eps, workspace.topk_idx.data_ptr(),
+                      workspace.topk_val.data_ptr(), workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(),
+                      workspace.bytes)
+        self.out = out
+
+    def run(self, stream: int | None = None) -> None:
+        rc = self._fn(*self._head, self.n_max, self.full_max, *self._tail, _stream() if stream is None else stream)
+        if rc:
+            _lib.check(rc, "pqhsa_decode_step")
+
+
 def hybrid_attend_paged(q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int, full_max: int,
                         topk_idx, topk_val, topk_cnt, list_mass, row_max, scale: float) -> torch.Tensor:
     """Exact hybrid attention given a selection and per-list masses (``list_mass [BH, G, L]``

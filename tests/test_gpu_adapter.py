@@ -1,0 +1,327 @@
+"""GPU tests of the drop-in boundary: adapters, sidecar and the vLLM decode hook, end to end
+through the C ABI, against vectors recorded from the real reference (tests/golden/*.npz) and
+against the fixed-order oracle run on the engine's own trained index."""
+
+import math
+import os
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fixed
+from oracle import torch_ref as tr
+from tests.gpu_util import u16, u32
+
+pytestmark = pytest.mark.gpu
+
+DIM = 128
+SCALE = 1.0 / math.sqrt(DIM)
+
+
+def _cuda():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return torch.device("cuda")
+
+
+def _cfgs(lists, fraction, *, sink=4, local=64, strategy="incremental", interval=1):
+    from pqhsa_release_amd.config import IVFPQConfig, SparseAttentionConfig
+
+    ic = IVFPQConfig(num_lists=lists, nprobe=8, num_subspaces=8, num_bits=4, residual=True, coarse_max_iter=1,
+                     pq_max_iter=2, kernel_backend="mi355x", direction_normalize=True, seed=0)
+    ac = SparseAttentionConfig(sink_tokens=sink, local_window=local, retrieval_top_fraction=fraction,
+                               exact_rerank=True, mode="hybrid", hybrid_value_mode="centroid",
+                               index_update_interval=interval, index_update_strategy=strategy,
+                               collect_attention_details=False)
+    return ic, ac
+
+
+def _load(golden_dir, name):
+    fx = np.load(os.path.join(golden_dir, f"{name}.npz"))
+    m = dict(zip(["ctx", "heads", "groups", "lists", "steps", "sink", "local"], (int(x) for x in fx["meta"])))
+    m["fraction"] = float(fx["fraction"][0])
+    return fx, m
+
+
+def _words(packed_np):
+    return tr.packed_to_words(torch.from_numpy(packed_np)).numpy().astype(np.uint32)
+
+
+def _index_of(engine, bh, n):
+    """Download one stream's index in the oracle's format."""
+    idx = engine.index
+    return {"coarse": idx.coarse[bh].cpu().numpy(), "codebooks": idx.codebooks[bh].cpu().numpy(),
+            "codes": u32(idx.codes[bh, :n]), "list_ids": u16(idx.list_ids[bh, :n]),
+            "norms": idx.norms[bh, :n].cpu().numpy(), "vbar": idx.vbar[bh].cpu().numpy()}
+
+
+def _margin_ok(logits, got_idx, ref_idx):
+    for g in range(logits.shape[0]):
+        a, b = set(got_idx[g].tolist()), set(ref_idx[g].tolist())
+        if a == b:
+            continue
+        kth = np.sort(logits[g])[::-1][len(ref_idx[g]) - 1]
+        for i in a ^ b:
+            assert abs(logits[g, i] - kth) <= 1e-5 * max(abs(kth), 1e-3), (g, i)
+
+
+@pytest.mark.parametrize("name", ["ref_fp32_h1", "ref_bf16_gqa"])
+def test_engine_reproduces_reference_vectors_with_the_reference_index(golden_dir, name):
+    """The reference's trained index goes in (build_with_codebooks); packed codes, list ids, norms,
+    top-k sets and attention outputs must come out as the reference recorded them, before and
+    after per-step incremental appends."""
+    dev = _cuda()
+    from pqhsa_release_amd.attention import PQHSAEngine
+
+    fx, m = _load(golden_dir, name)
+    H, G, ctx, steps = m["heads"], m["groups"], m["ctx"], m["steps"]
+    bf16 = name.endswith("gqa")
+    kv_dtype = torch.bfloat16 if bf16 else torch.float32
+    ic, ac = _cfgs(m["lists"], m["fraction"], sink=m["sink"], local=m["local"])
+    keys = torch.from_numpy(fx["keys"]).to(dev, kv_dtype)[None]          # [1, H, ctx+steps, D]
+    values = torch.from_numpy(fx["values"]).to(dev, kv_dtype)[None]
+    eng = PQHSAEngine(ic, ac, batch=1, kv_heads=H, device=dev)
+    eng.adopt(keys[:, :, :ctx], values[:, :, :ctx])
+    eng.build([ctx], coarse=torch.from_numpy(fx["coarse"]), codebooks=torch.from_numpy(fx["codebooks"]))
+    tol = 2e-3 if bf16 else 1e-4
+
+    def check(tag, step):
+        n = fx[f"{tag}_list_ids"].shape[1]
+        assert eng.n(0) == n
+        q = torch.from_numpy(fx["queries"][:, step]).reshape(1, H * G, DIM).to(dev)   # fp32 queries
+        out = eng.forward(q, G)
+        torch.cuda.synchronize()
+        tidx, tval, tcnt = eng.last_topk(G)
+        for h in range(H):
+            ref_lists, ref_words = fx[f"{tag}_list_ids"][h], _words(fx[f"{tag}_packed"][h])
+            lists, codes = u16(eng.index.list_ids[h, :n]), u32(eng.index.codes[h, :n])
+            # integer parity with the reference (these fixtures hold no argmin near-tie: the
+            # fixed-order oracle reproduces them exactly too, tests/test_oracle_golden.py)
+            assert np.array_equal(lists, ref_lists) and np.array_equal(codes, ref_words)
+            np.testing.assert_allclose(eng.index.norms[h, :n].cpu().numpy(), fx[f"{tag}_norms"][h], rtol=1e-6)
+            np.testing.assert_allclose(eng.index.vbar[h].cpu().numpy(), fx[f"{tag}_vbar"][h], atol=1e-5)
+            k = fx[f"{tag}_topk_idx"].shape[2]
+            got = tidx.reshape(H, G, -1)[h, :, :k].cpu().numpy()
+            assert (tcnt.reshape(H, G)[h] == k).all()
+            _margin_ok(fx[f"{tag}_scores"][h] * np.float32(SCALE), got, fx[f"{tag}_topk_idx"][h])
+        err = (out[0].float().cpu().numpy() - fx[f"{tag}_output"]).__abs__().max()
+        assert err <= tol, (tag, err)
+        return err
+
+    e0 = check("build", 0)
+    for s in range(steps):
+        pos = ctx + s
+        eng.write_rows(keys[:, :, pos], values[:, :, pos])
+        eng.advance(1)
+    e1 = check("append", steps)
+    print(f"{name}: max |out - reference| build {e0:.2e}, after {steps} appends {e1:.2e}")
+
+
+def _problem(dev, *, batch=1, heads=2, groups=4, ctx=1500, extra=40, dtype=torch.bfloat16, seed=5):
+    from pqhsa_release_amd.synth import make_layer
+
+    k, v, _ = make_layer(ctx + extra, batch=batch, kv_heads=heads, groups=1, seed0=seed, dtype=dtype)
+    gen = torch.Generator().manual_seed(seed + 1)
+    q = k[:, :, 100:100 + (extra + 1) * groups].float() + 0.2 * torch.randn(batch, heads, (extra + 1) * groups, DIM,
+                                                                              generator=gen)
+    q = q.reshape(batch, heads, extra + 1, groups, DIM).to(dtype)
+    return k.to(dev), v.to(dev), q.to(dev)
+
+
+def _oracle_check(eng, keys, values, q_step, groups, length, fraction, tol):
+    """Run the fixed-order oracle on the engine's own index and compare top-k (exact) and output."""
+    tidx, _, tcnt = eng.last_topk(groups)
+    worst = 0.0
+    outs = []
+    for b in range(eng.B):
+        for h in range(eng.H):
+            bh, n = b * eng.H + h, eng.n(b)
+            ix = _index_of(eng, bh, n)
+            want_out, want_idx, _ = fixed.decode_step(q_step[b, h].float().cpu().numpy(),
+                                                      keys[b, h, :length].float().cpu().numpy(),
+                                                      values[b, h, :length].float().cpu().numpy(), ix,
+                                                      sink=eng.sink, local=length - eng.sink - n,
+                                                      fraction=fraction, scale=SCALE)
+            k = want_idx.shape[1]
+            got = tidx.reshape(eng.B, eng.H, groups, -1)[b, h, :, :k].cpu().numpy()
+            for g in range(groups):
+                assert np.array_equal(got[g], np.sort(want_idx[g])), (b, h, g)
+            outs.append(want_out)
+    return np.stack(outs).reshape(eng.B, eng.H * groups, DIM), worst
+
+
+def test_gqa_adapter_decode_steps_match_oracle_on_its_own_index():
+    dev = _cuda()
+    from pqhsa_release_amd.attention import GQAIVFPQDecodeAttentionAdapter
+
+    ctx, extra, H, G = 1500, 12, 2, 4
+    keys, values, q = _problem(dev, heads=H, groups=G, ctx=ctx, extra=extra)
+    ic, ac = _cfgs(64, 0.02)
+    ad = GQAIVFPQDecodeAttentionAdapter(ic, ac, num_query_heads=H * G, num_key_value_heads=H)
+    assert ad.build_cache(keys[:, :, :ctx], values[:, :, :ctx]) is ad
+    assert ad.leading_shape == (1, H) and len(ad.streams) == H
+    out = ad.forward(q[:, :, 0].reshape(1, H * G, DIM).float())
+    assert out.context.shape == (1, H * G, DIM) and len(out.per_query) == G
+    want, _ = _oracle_check(ad.engine, keys, values, q[:, :, 0], G, ctx, 0.02, 2e-3)
+    assert np.abs(out.context.cpu().numpy() - want).max() <= 2e-3
+    # decode_step appends, then attends (the new row is in the local window)
+    for s in range(1, extra + 1):
+        pos = ctx + s - 1
+        res = ad.decode_step(q[:, :, s].reshape(1, H * G, 1, DIM).float(), keys[:, :, pos], values[:, :, pos : pos + 1])
+        assert res.context.shape == (1, H * G, 1, DIM)
+    assert ad.engine.n(0) == ctx + extra - 64 - 4 and ad.engine.index_adds == extra
+    want, _ = _oracle_check(ad.engine, keys, values, q[:, :, extra], G, ctx + extra, 0.02, 2e-3)
+    assert np.abs(res.context[:, :, 0].cpu().numpy() - want).max() <= 2e-3
+    # appended keys were encoded exactly as a fresh encode of the same rows would
+    n = ad.engine.n(0)
+    for h in range(H):
+        ix = _index_of(ad.engine, h, n)
+        norms, lists, codes = fixed.encode(keys[0, h, 4 : 4 + n].float().cpu().numpy(), ix["coarse"], ix["codebooks"])
+        assert np.array_equal(lists, ix["list_ids"]) and np.array_equal(codes, ix["codes"])
+        assert np.array_equal(norms, ix["norms"])
+    # bf16 queries in, bf16 context out
+    res16 = ad.forward(q[:, :, extra].reshape(1, H * G, DIM))
+    assert res16.context.dtype == torch.bfloat16
+    assert np.abs(res16.context.float().cpu().numpy() - want).max() <= 2e-3 + 2.0 ** -8 * np.abs(want).max()
+
+
+def test_plain_adapter_multi_query_and_state_round_trip():
+    dev = _cuda()
+    from pqhsa_release_amd.attention import IVFPQDecodeAttentionAdapter
+
+    ctx, H, Q = 900, 2, 3
+    keys, values, q = _problem(dev, batch=2, heads=H, groups=Q, ctx=ctx, extra=0, dtype=torch.float32, seed=9)
+    ic, ac = _cfgs(32, 0.05)
+    ad = IVFPQDecodeAttentionAdapter(ic, ac).build_cache(keys, values)
+    queries = q[:, :, 0]                                            # [B, H, Q, D]
+    res = ad.forward(queries)
+    assert res.context.shape == (2, H, Q, DIM) and len(res.per_query) == Q
+    assert res.per_query[0].per_stream[0].exact_retrieval_count == math.ceil((ctx - 68) * 0.05)
+    want, _ = _oracle_check(ad.engine, keys, values, queries, Q, ctx, 0.05, 1e-4)
+    assert np.abs(res.context.reshape(2, H * Q, DIM).cpu().numpy() - want).max() <= 1e-4
+    single = ad.forward(queries[:, :, 0])                           # [B, H, D] -> [B, H, D]
+    assert single.context.shape == (2, H, DIM)
+    np.testing.assert_allclose(single.context.cpu().numpy(), res.context[:, :, 0].cpu().numpy(), atol=1e-5)
+    state = ad.state_dict()
+    clone = IVFPQDecodeAttentionAdapter.from_state_dict(state)
+    again = clone.forward(queries)
+    assert torch.equal(again.context, res.context)
+    assert clone.leading_shape == (2, H)
+
+
+def test_all_tokens_selected_equals_dense_attention_through_the_adapter():
+    dev = _cuda()
+    from pqhsa_release_amd.attention import IVFPQDecodeAttentionAdapter
+
+    keys, values, q = _problem(dev, heads=1, groups=1, ctx=400, extra=0, dtype=torch.float32, seed=21)
+    ic, ac = _cfgs(8, 1.0, sink=2, local=5)
+    ad = IVFPQDecodeAttentionAdapter(ic, ac).build_cache(keys, values)
+    got = ad.forward(q[:, :, 0, 0]).context[0, 0].double().cpu()
+    k64, v64, q64 = keys[0, 0].double().cpu(), values[0, 0].double().cpu(), q[0, 0, 0, 0].double().cpu()
+    dense = torch.softmax((k64 @ q64) * SCALE, dim=0) @ v64
+    np.testing.assert_allclose(got.numpy(), dense.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_deferred_strategy_flush_updates_codebooks_and_reencodes():
+    dev = _cuda()
+    from pqhsa_release_amd.attention import GQAIVFPQDecodeAttentionAdapter
+
+    ctx, extra, H, G = 1200, 20, 2, 2
+    keys, values, q = _problem(dev, heads=H, groups=G, ctx=ctx, extra=extra, seed=31)
+    ic, ac = _cfgs(32, 0.02, strategy="deferred", interval=8)
+    ad = GQAIVFPQDecodeAttentionAdapter(ic, ac, num_query_heads=H * G, num_key_value_heads=H)
+    ad.build_cache(keys[:, :, :ctx], values[:, :, :ctx])
+    n0 = ad.engine.n(0)
+    coarse0 = ad.engine.index.coarse.clone()
+    for s in range(extra):
+        ad.append(keys[:, :, ctx + s], values[:, :, ctx + s])
+    # deferred: nothing indexed yet, the pending rows stay exact in the local region
+    assert ad.engine.n(0) == n0 and ad.engine.full_count(0) == 4 + 64 + extra and ad.engine.deferred_pending
+    out = ad.forward(q[:, :, extra].reshape(1, H * G, DIM).float()).context
+    want, _ = _oracle_check(ad.engine, keys, values, q[:, :, extra], G, ctx + extra, 0.02, 2e-3)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3
+    assert ad.apply_pending_index_update() == H and ad.apply_pending_index_update() == 0
+    assert ad.engine.n(0) == n0 + extra and not torch.equal(coarse0, ad.engine.index.coarse)
+    out = ad.forward(q[:, :, extra].reshape(1, H * G, DIM).float()).context
+    want, _ = _oracle_check(ad.engine, keys, values, q[:, :, extra], G, ctx + extra, 0.02, 2e-3)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3
+    # after the flush every stored code is the encoding under the moved codebooks
+    n = ad.engine.n(0)
+    ix = _index_of(ad.engine, 1, n)
+    _, lists, codes = fixed.encode(keys[0, 1, 4 : 4 + n].float().cpu().numpy(), ix["coarse"], ix["codebooks"])
+    assert np.array_equal(lists, ix["list_ids"]) and np.array_equal(codes, ix["codes"])
+
+
+@pytest.mark.parametrize("layout", ["5d", "4d"])
+def test_vllm_hook_single_token_decode_over_a_paged_cache(layout, monkeypatch):
+    dev = _cuda()
+    from pqhsa_release_amd.vllm_backend import pq_hsa_decode_runtime as rt
+    from pqhsa_release_amd.vllm_backend import pq_hsa_flashattn_wrap as wrap
+
+    for k in list(os.environ):
+        if k.startswith("PQ_HSA_"):
+            monkeypatch.delenv(k)
+    for k, v in {"PQ_HSA_ENABLE": "1", "PQ_HSA_NUM_LISTS": "64", "PQ_HSA_TOP_FRAC": "0.02", "PQ_HSA_LOCAL": "64",
+                 "PQ_HSA_UPD_INTERVAL": "4", "PQ_HSA_FLUSH_INTERVAL": "4"}.items():
+        monkeypatch.setenv(k, v)
+    rt.reset_pq_hsa_runtime_stats()
+    rt.reset_pq_hsa_layer_state()
+    ctx, steps, H, G, bs = 1300, 9, 2, 4, 16
+    keys, values, q = _problem(dev, heads=H, groups=G, ctx=ctx, extra=steps, seed=41)
+    blocks = (ctx + steps + bs - 1) // bs
+    table = torch.randperm(blocks + 4, generator=torch.Generator().manual_seed(1))[:blocks].to(torch.int32).to(dev)[None]
+    if layout == "5d":
+        cache = torch.zeros(2, blocks + 4, bs, H, DIM, dtype=torch.bfloat16, device=dev)
+        kc, vc = cache[0], cache[1]
+    else:
+        cache = torch.zeros(blocks + 4, H, bs, 2 * DIM, dtype=torch.bfloat16, device=dev)
+        kc, vc = tr.split_kv_cache(cache)
+    pos = torch.arange(ctx, device=dev)
+    kc[table[0, pos // bs].long(), pos % bs] = keys[0, :, :ctx].transpose(0, 1)
+    vc[table[0, pos // bs].long(), pos % bs] = values[0, :, :ctx].transpose(0, 1)
+
+    class Impl:
+        scale, num_heads, num_kv_heads, kv_cache_dtype = SCALE, H * G, H, "auto"
+
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, **extra):
+            output.fill_(-7.0)
+            return output
+
+    wrap.wrap_forward(Impl)
+    impl, layer = Impl(), types.SimpleNamespace(layer_name="layers.0.attn")
+    try:
+        for s in range(steps + 1):
+            length = ctx + s
+            slot = int(table[0, (length - 1) // bs]) * bs + (length - 1) % bs
+            md = types.SimpleNamespace(max_query_len=1, num_actual_tokens=1, use_cascade=False, max_seq_len=length,
+                                       seq_lens=torch.tensor([length], dtype=torch.int32, device=dev),
+                                       block_table=table, slot_mapping=torch.tensor([slot], device=dev))
+            k_new = keys[0, :, length - 1][None]                     # [1, H, D] this step's row
+            v_new = values[0, :, length - 1][None]
+            if layout == "4d":                                        # vLLM >= 0.10 writes the page itself
+                kc[slot // bs, slot % bs] = k_new[0]
+                vc[slot // bs, slot % bs] = v_new[0]
+            out = torch.zeros(1, H * G, DIM, dtype=torch.bfloat16, device=dev)
+            query = q[0, :, s].reshape(1, H * G, DIM)
+            res = impl.forward(layer, query, k_new, v_new, cache, md, output=out)
+            assert res is out and float(out.float().abs().max()) != 7.0
+            eng = rt.state_for(impl, layer)["sidecar"].adapter.engine
+            if s > 0 and s % 4 == 0:
+                continue      # the hook flushed right after this forward: the index has moved on
+            want, _ = _oracle_check(eng, keys, values, q[:, :, s], G, length, 0.02, 2e-3)
+            err = np.abs(out.float().cpu().numpy() - want)
+            assert (err <= 2e-3 + 2.0 ** -8 * np.abs(want)).all(), (s, err.max())
+        assert rt.STATS["pq_build_calls"] == 1 and rt.STATS["pq_append_calls"] == steps
+        assert rt.STATS["pq_flush_calls"] == steps // 4 and rt.STATS["sidecar"] == "GQASidecar"
+        assert eng.keys_buf is None                                   # exact rows are read from the pages in place
+        assert eng.n(0) == ctx + 8 - 64 - 4                           # two deferred flushes of 4 rows each
+        # a prefill-shaped call goes to the wrapped original
+        md.max_query_len = 5
+        out = torch.zeros(1, H * G, DIM, dtype=torch.bfloat16, device=dev)
+        impl.forward(layer, query, k_new, v_new, cache, md, output=out)
+        assert float(out[0, 0, 0]) == -7.0
+    finally:
+        wrap.unwrap_forward(Impl)
+        rt.reset_pq_hsa_layer_state()

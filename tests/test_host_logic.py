@@ -1,0 +1,287 @@
+"""CPU tests of the host-side mirror of the reference interface: packing helpers, configuration
+records, adapter error behaviour, the vLLM decode hook's gating / state machine / STATS (with
+fake impl, metadata and sidecar objects, as the reference's own hook tests need a real vLLM)."""
+
+import os
+import types
+
+import pytest
+import torch
+
+import pqhsa_release_amd as pkg
+from pqhsa_release_amd.attention import GQAIVFPQDecodeAttentionAdapter, IVFPQDecodeAttentionAdapter
+from pqhsa_release_amd.config import IVFPQConfig, SparseAttentionConfig, validate_for_kernels
+from pqhsa_release_amd.vllm_backend import pq_hsa_decode_runtime as rt
+from pqhsa_release_amd.vllm_backend import pq_hsa_flashattn_wrap as wrap
+from pqhsa_release_amd.vllm_plugin import plugin
+from pqhsa_release_amd.vllm_plugin.config import PQHSAConfig
+
+
+def paper_cfgs():
+    ic = IVFPQConfig(num_lists=64, num_subspaces=8, num_bits=4, coarse_max_iter=1, pq_max_iter=2,
+                     direction_normalize=True, kernel_backend="mi355x")
+    ac = SparseAttentionConfig(sink_tokens=4, local_window=64, retrieval_top_fraction=0.02, mode="hybrid",
+                               hybrid_value_mode="centroid", collect_attention_details=False)
+    return ic, ac
+
+
+def test_packing_helpers_follow_reference_layout():
+    codes = torch.tensor([[0, 1, 2, 3], [15, 14, 13, 12]])
+    packed = pkg.pack_4bit_codes(codes)
+    assert packed.dtype == torch.uint8 and packed.tolist() == [[0x10, 0x32], [0xEF, 0xCD]]
+    assert torch.equal(pkg.unpack_4bit_codes(packed, 4), codes)
+    odd = torch.tensor([[1, 2, 3], [4, 5, 6]])
+    p = pkg.pack_4bit_codes(odd)
+    assert p.shape == (2, 2) and torch.all((p[:, -1] >> 4) == 0)
+    assert torch.equal(pkg.unpack_4bit_codes(p, 3), odd)
+    with pytest.raises(ValueError, match=r"\[0, 15\]"):
+        pkg.pack_4bit_codes(torch.tensor([[0, 16]]))
+    with pytest.raises(ValueError):
+        pkg.unpack_4bit_codes(packed, 7)
+
+
+def test_config_defaults_match_reference_and_validation_is_loud():
+    assert IVFPQConfig().num_lists == 256 and IVFPQConfig().num_bits == 8 and IVFPQConfig().eps == 1e-12
+    ac = SparseAttentionConfig()
+    assert (ac.mode, ac.hybrid_value_mode, ac.index_update_strategy, ac.retrieval_topk) == \
+        ("sparse", "denominator", "incremental", 100)
+    ic, ac = paper_cfgs()
+    validate_for_kernels(ic, ac)
+    for bad in (dict(num_bits=8), dict(num_subspaces=16), dict(direction_normalize=False), dict(rotation="random_orthogonal")):
+        with pytest.raises(ValueError):
+            validate_for_kernels(IVFPQConfig(**{**{n: getattr(ic, n) for n in ic.__slots__}, **bad}), ac)
+    for bad in (dict(mode="sparse"), dict(hybrid_value_mode="full"), dict(exact_rerank=False), dict(retrieval_top_p=0.9),
+                dict(retrieval_top_fraction=1.5), dict(index_update_strategy="sometimes"), dict(kv_storage="cpu")):
+        with pytest.raises(ValueError):
+            validate_for_kernels(ic, SparseAttentionConfig(**{**{n: getattr(ac, n) for n in ac.__slots__}, **bad}))
+
+
+def test_adapters_raise_like_the_reference_before_build_and_on_bad_shapes():
+    ic, ac = paper_cfgs()
+    ad = IVFPQDecodeAttentionAdapter(ic, ac)
+    with pytest.raises(RuntimeError):
+        ad.forward(torch.zeros(1, 2, 128))
+    with pytest.raises(RuntimeError):
+        ad.leading_shape
+    with pytest.raises(ValueError):
+        ad.build_cache(torch.zeros(2, 100, 128), torch.zeros(2, 100, 128))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ad.build_cache(torch.zeros(1, 2, 300, 128), torch.zeros(1, 2, 300, 128))      # CPU tensors
+    with pytest.raises(ValueError):
+        ad.decode_step(torch.zeros(1, 2, 128))                                         # append_kv without K/V
+    with pytest.raises(ValueError, match="divisible"):
+        GQAIVFPQDecodeAttentionAdapter(ic, ac, num_query_heads=7, num_key_value_heads=2)
+    g = GQAIVFPQDecodeAttentionAdapter(ic, ac, num_query_heads=8, num_key_value_heads=2)
+    assert g.num_key_value_groups == 4
+    with pytest.raises(ValueError, match="KV heads"):
+        g.build_cache(torch.zeros(1, 3, 300, 128), torch.zeros(1, 3, 300, 128))
+
+
+def meta(seq_len=500, reqs=1, qlen=1, tokens=1, cascade=False):
+    return types.SimpleNamespace(max_query_len=qlen, num_actual_tokens=tokens, use_cascade=cascade,
+                                 seq_lens=torch.full((reqs,), seq_len, dtype=torch.int32), max_seq_len=seq_len,
+                                 block_table=torch.zeros(reqs, 64, dtype=torch.int32),
+                                 slot_mapping=torch.zeros(tokens, dtype=torch.int64))
+
+
+@pytest.fixture
+def clean_runtime(monkeypatch):
+    for k in list(os.environ):
+        if k.startswith("PQ_HSA_"):
+            monkeypatch.delenv(k)
+    rt.reset_pq_hsa_runtime_stats()
+    rt.reset_pq_hsa_layer_state()
+    yield
+    rt.reset_pq_hsa_runtime_stats()
+    rt.reset_pq_hsa_layer_state()
+
+
+def test_should_pq_decode_gate_and_reject_reasons(clean_runtime, monkeypatch):
+    assert rt.min_pq_seq() == 4 + 128 + 16
+    assert rt.should_pq_decode(meta())
+    assert not rt.should_pq_decode(None)
+    assert not rt.should_pq_decode(meta(cascade=True))
+    assert not rt.should_pq_decode(meta(qlen=2))
+    assert not rt.should_pq_decode(meta(tokens=2))
+    assert not rt.should_pq_decode(meta(reqs=2))
+    assert not rt.should_pq_decode(meta(seq_len=100))
+    assert rt.STATS["reject"] == {"no_metadata": 1, "cascade": 1, "max_query_len!=1": 1, "num_actual_tokens!=1": 1,
+                                  "num_reqs!=1": 1, "seq_too_short": 1}
+    monkeypatch.setenv("PQ_HSA_BATCH", "1")
+    assert rt.should_pq_decode(meta(reqs=3, tokens=3))
+    assert not rt.should_pq_decode(meta(reqs=3, tokens=2))
+    monkeypatch.setenv("PQ_HSA_LOCAL", "64")
+    assert rt.min_pq_seq() == 84
+
+
+class FakeSidecar:
+    built = 0
+
+    def __init__(self, icfg, acfg, *, num_query_heads, num_kv_heads):
+        self.icfg, self.acfg, self.hq, self.hkv = icfg, acfg, num_query_heads, num_kv_heads
+        self.length, self.appended, self.flushed, self.fail = 0, 0, 0, False
+        self._ckpt = None
+
+    batched_heads_active = True
+    cuda_graph_active = False
+
+    @property
+    def prefix_checkpoint_length(self):
+        return self._ckpt
+
+    def build_cache(self, keys, values):
+        FakeSidecar.built += 1
+        self.length = keys.shape[2]
+        return self
+
+    def set_paged_kv_context(self, kv_cache, attn_metadata, seq_idx=0):
+        self.paged = (kv_cache, seq_idx)
+
+    def append(self, k, v):
+        assert k.shape == (1, self.hkv, 128)
+        self.appended += 1
+        self.length += 1
+
+    def forward(self, q):
+        if self.fail:
+            raise RuntimeError("boom")
+        return torch.full((1, self.hq, 128), float(self.length))
+
+    def apply_pending_index_update(self):
+        self.flushed += 1
+        return 1
+
+    def checkpoint_prefix(self):
+        self._ckpt = self.length
+
+    def restore_prefix(self, k, v, *, kv_cache=None, attn_metadata=None, seq_idx=0):
+        self.length = self._ckpt
+        return True
+
+
+@pytest.fixture
+def fake_stack(clean_runtime, monkeypatch):
+    FakeSidecar.built = 0
+    monkeypatch.setattr(rt, "sidecar_cls", lambda: FakeSidecar)
+    monkeypatch.setattr(rt, "gather_flashattn_kv",
+                        lambda kv, md, i=0: (torch.zeros(1, 2, int(md.max_seq_len), 128),
+                                             torch.zeros(1, 2, int(md.max_seq_len), 128), int(md.max_seq_len)))
+    impl = types.SimpleNamespace(scale=0.088, num_heads=8, num_kv_heads=2, kv_cache_dtype="auto")
+    layer = types.SimpleNamespace(layer_name="model.layers.0.self_attn.attn")
+    kv_cache = torch.zeros(64, 2, 16, 256)         # 4-D layout: nothing to write in the hook
+    return impl, layer, kv_cache
+
+
+def step(impl, layer, kv_cache, seq_len, dense_value=-1.0):
+    q, k, v = torch.zeros(1, 8, 128), torch.zeros(1, 2, 128), torch.zeros(1, 2, 128)
+    out = torch.zeros(1, 8, 128)
+    res = rt.pq_or_dense_forward(impl, layer, q, k, v, kv_cache, meta(seq_len), out,
+                                 lambda: torch.full((1, 8, 128), dense_value))
+    return res
+
+
+def test_hook_state_machine_build_append_flush_rebuild(fake_stack, monkeypatch):
+    impl, layer, kv_cache = fake_stack
+    # disabled: dense path, nothing built
+    assert float(step(impl, layer, kv_cache, 500)[0, 0, 0]) == -1.0
+    assert rt.STATS["dense_fa_calls"] == 1 and FakeSidecar.built == 0
+    monkeypatch.setenv("PQ_HSA_ENABLE", "1")
+    monkeypatch.setenv("PQ_HSA_FLUSH_INTERVAL", "2")
+    assert float(step(impl, layer, kv_cache, 500)[0, 0, 0]) == 500.0              # first step builds
+    sc = rt.state_for(impl, layer)["sidecar"]
+    assert isinstance(sc, FakeSidecar) and sc.acfg.scale == pytest.approx(0.088) and sc.acfg.mode == "hybrid"
+    assert sc.icfg.num_lists == 512 and sc.acfg.index_update_strategy == "deferred"
+    assert rt.STATS["pq_build_calls"] == 1 and rt.STATS["prefix_persist_misses"] == 1
+    assert rt.STATS["prefix_miss_reasons"] == {"no_adapter": 1}
+    assert float(step(impl, layer, kv_cache, 501)[0, 0, 0]) == 501.0              # sequential: append
+    assert float(step(impl, layer, kv_cache, 502)[0, 0, 0]) == 502.0
+    assert sc.appended == 2 and sc.flushed == 1 and rt.STATS["pq_flush_calls"] == 1
+    assert rt.STATS["pq_append_calls"] == 2 and rt.STATS["pq_decode_calls"] == 3
+    assert float(step(impl, layer, kv_cache, 700)[0, 0, 0]) == 700.0              # non-sequential: rebuild
+    assert FakeSidecar.built == 2 and rt.STATS["prefix_miss_reasons"]["no_prefix_key"] == 1
+    # short sequence falls through to dense and records why
+    assert float(step(impl, layer, kv_cache, 100)[0, 0, 0]) == -1.0
+    assert rt.STATS["reject"]["seq_too_short"] == 1
+
+
+def test_hook_error_convention_reraise_or_dense_fallback(fake_stack, monkeypatch):
+    impl, layer, kv_cache = fake_stack
+    monkeypatch.setenv("PQ_HSA_ENABLE", "1")
+    step(impl, layer, kv_cache, 500)
+    rt.state_for(impl, layer)["sidecar"].fail = True
+    with pytest.raises(RuntimeError, match="boom"):
+        step(impl, layer, kv_cache, 501)
+    assert rt.STATS["last_error"] == "RuntimeError: boom" and rt.STATS["dense_fallback_calls"] == 1
+    monkeypatch.setenv("PQ_HSA_FALLBACK", "1")
+    rt.state_for(impl, layer)["seq_len"] = 501
+    assert float(step(impl, layer, kv_cache, 502)[0, 0, 0]) == -1.0
+    assert rt.STATS["dense_fallback_calls"] == 2
+
+
+def test_prefix_checkpoint_restore_on_same_prompt(fake_stack, monkeypatch):
+    impl, layer, kv_cache = fake_stack
+    monkeypatch.setenv("PQ_HSA_ENABLE", "1")
+    runner = types.SimpleNamespace(input_batch=types.SimpleNamespace(req_ids=["r0"]),
+                                   requests={"r0": types.SimpleNamespace(prompt_token_ids=list(range(499)))})
+
+    def go(seq_len):
+        md = meta(seq_len)
+        md._pq_runner = runner
+        out = torch.zeros(1, 8, 128)
+        return rt.pq_or_dense_forward(impl, layer, torch.zeros(1, 8, 128), torch.zeros(1, 2, 128),
+                                      torch.zeros(1, 2, 128), kv_cache, md, out, lambda: out)
+
+    go(500)
+    go(501)
+    assert float(go(500)[0, 0, 0]) == 500.0           # same prompt again: restored, not rebuilt
+    assert FakeSidecar.built == 1 and rt.STATS["prefix_persist_hits"] == 1
+
+
+def test_copy_ctx_and_as_decode_qkv():
+    out = torch.zeros(2, 8, 128, dtype=torch.bfloat16)
+    rt.copy_ctx(out, torch.ones(1, 8 * 128), 1)
+    assert float(out[0].sum()) == 8 * 128 and float(out[1].sum()) == 0
+    assert rt.as_decode_qkv(torch.zeros(3, 8, 128)).shape == (1, 8, 128)
+    assert rt.as_decode_qkv(torch.zeros(3, 128)).shape == (1, 1, 128)
+    with pytest.raises(ValueError):
+        rt.as_decode_qkv(torch.zeros(128))
+
+
+def test_write_kv_to_cache_uses_the_slot_mapping():
+    cache = torch.zeros(2, 5, 16, 2, 128)
+    md = types.SimpleNamespace(slot_mapping=torch.tensor([37]))
+    rt.write_kv_to_cache(torch.ones(1, 2, 128), 2 * torch.ones(1, 2, 128), cache, md)
+    assert float(cache[0, 2, 5].sum()) == 256 and float(cache[1, 2, 5].sum()) == 512 and float(cache.sum()) == 768
+
+
+def test_plugin_is_a_noop_unless_enabled_and_config_env_round_trip(clean_runtime, monkeypatch):
+    class Impl:
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, **extra):
+            return "dense"
+
+    monkeypatch.delenv("PQ_HSA_VLLM", raising=False)
+    plugin.vllm_general_plugin()
+    assert plugin.install(impl_cls=Impl) == {"installed": False, "reason": "PQ_HSA_VLLM!=1"}
+    assert not getattr(Impl.forward, "_pq_hsa_wrapped", False)
+    monkeypatch.setenv("PQ_HSA_VLLM", "1")
+    monkeypatch.setenv("PQ_HSA_TOP_FRAC", "0.02")
+    res = plugin.install(impl_cls=Impl)
+    assert res["installed"] and res["config"]["top_fraction"] == 0.02
+    assert "PQ_HSA_TOP_FRAC" not in res["env_defaults_written"]       # explicit value wins
+    assert os.environ["PQ_HSA_ENABLE"] == "1" and os.environ["PQ_HSA_LOCAL"] == "128"
+    assert os.environ["PQ_HSA_CUDA_SPLITS"] == "8"                     # H20 switches accepted as no-ops
+    assert getattr(Impl.forward, "_pq_hsa_wrapped", False)
+    assert not wrap.wrap_forward(Impl)                                 # idempotent
+    # prefill-like metadata goes to the original forward
+    assert Impl().forward(None, None, None, None, None, meta(qlen=7, tokens=7)) == "dense"
+    wrap.unwrap_forward(Impl)
+    assert not getattr(Impl.forward, "_pq_hsa_wrapped", False)
+    cfg = PQHSAConfig(top_fraction=0.05, local_window=64, batch=True)
+    env = cfg.as_env()
+    assert env["PQ_HSA_TOP_FRAC"] == "0.05" and env["PQ_HSA_LOCAL"] == "64" and env["PQ_HSA_BATCH"] == "1"
+    for k in list(os.environ):
+        if k.startswith("PQ_HSA_"):
+            monkeypatch.delenv(k)
+    cfg.apply_env_defaults()
+    back = PQHSAConfig.from_env()
+    assert (back.top_fraction, back.local_window, back.batch) == (0.05, 64, True)
