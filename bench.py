@@ -122,6 +122,7 @@ class Layer:
         self.index.set_counts(self.n)
         ops.encode(self.kv, self.index, SINK, [0] * B, self.n)
         ops.value_summaries(self.kv, self.index, SINK)
+        self.index.finalize_layout()
         self.seq_lens = torch.tensor(self.lens, dtype=torch.int32, device=device)
         k_cap = ops.resolve_topk(n_max, FRACTION, 0)
         self.ws = ops.DecodeWorkspace(self.index, G, k_cap)
@@ -154,8 +155,9 @@ def cpu_baseline(layer, seconds=12.0):
     kk, vv = ops.paged_gather_range(layer.kv, b, 0, ln) if layer.kv.view.paged else (layer.keys[b], layer.values[b])
     keys, values = kk[h].float().cpu(), vv[h].float().cpu()
     idx = layer.index
-    ref = tr.RefIndex(idx.coarse[bh].cpu(), idx.codebooks[bh].cpu(), idx.list_ids_long()[bh, :n].cpu(),
-                      idx.packed_bytes()[bh, :n].cpu().clone(), idx.norms[bh, :n].cpu())
+    _, lists_by_key, norms_by_key = idx.by_key(bh, n)
+    ref = tr.RefIndex(idx.coarse[bh].cpu(), idx.codebooks[bh].cpu(), (lists_by_key.to(torch.int64) & 0xFFFF).cpu(),
+                      idx.packed_bytes(bh, n).cpu().clone(), norms_by_key.cpu())
     vbar = idx.vbar[bh].cpu()
     q = layer.q[b, h * G : (h + 1) * G].float().cpu()
     cores = os.cpu_count() or 1

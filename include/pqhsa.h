@@ -13,15 +13,22 @@
  *   codes     u32 [BH, n_cap]   nibble m of the word = code of subspace m
  *                               (the little-endian view of the reference's [N, 4] uint8
  *                               packing, pq_hsa/index/packing.py:6-34)
- *   list_ids  u16 [BH, n_cap]   IVF list of each indexed key (pq_hsa/index/ivfpq.py:19-33)
+ *   list_ids  u16 [BH, n_cap]   IVF list of each stored key (pq_hsa/index/ivfpq.py:19-33)
  *   norms     f32 [BH, n_cap]   key norm (pq_hsa/index/ivfpq.py:1052-1059)
+ *   pos       i32 [BH, n_cap]   retrieval-local index of the key stored at each position
  *   coarse    f32 [BH, L, 128]  coarse centroids;  codebooks f32 [BH, 8, 16, 16]
  *   vbar      f32 [BH, L, 128]  per-list mean value (pq_hsa/attention/kv_cache.py:688-776)
  *   vsum      f32 [BH, L, 128], vcount f32 [BH, L]   running sums behind vbar
- *   n_idx     i32 [B]           indexed keys per sequence (device memory)
- * Indexed key i of a sequence is token position sink + i (insertion order); top-k indices
- * are reported in that retrieval-local space, like the reference's
- * (pq_hsa/attention/kv_cache.py:479-484).
+ *   n_idx     i32 [B]           keys stored per sequence (device memory)
+ *   n_sorted  i32 [B]           the first n_sorted stored keys are ordered by list id (the
+ *                               reference's list-sorted snapshot,
+ *                               benchmarks/e2e_pq_param_sweep.py:4163-4305); keys appended
+ *                               since the last sort follow in insertion order
+ *   s_codes / s_list_ids / s_norms [BH, s_cap], s_n i32 [B]
+ *                               a fixed random subset of the stored keys, scanned first to
+ *                               estimate the selection threshold
+ * Retrieval-local index i of a sequence is token position sink + i; top-k indices are
+ * reported in that space, like the reference's (pq_hsa/attention/kv_cache.py:479-484).
  */
 #ifndef PQHSA_H
 #define PQHSA_H
@@ -76,16 +83,23 @@ typedef struct pqhsa_index {
     uint32_t *codes;
     uint16_t *list_ids;
     float *norms;
+    int32_t *pos;
     const float *coarse;
     const float *codebooks;
     float *vbar;
     float *vsum;
     float *vcount;
-    const int32_t *n_idx; /* [B] */
-    int64_t n_cap;        /* row stride of codes / list_ids / norms */
+    const int32_t *n_idx;    /* [B] */
+    const int32_t *n_sorted; /* [B] */
+    const uint32_t *s_codes;
+    const uint16_t *s_list_ids;
+    const float *s_norms;
+    const int32_t *s_n;      /* [B] */
+    int64_t s_cap;           /* row stride of the s_* arrays */
+    int64_t n_cap;           /* row stride of codes / list_ids / norms / pos */
     int32_t num_lists;
-    int32_t batch;        /* B */
-    int32_t kv_heads;     /* H */
+    int32_t batch;           /* B */
+    int32_t kv_heads;        /* H */
 } pqhsa_index;
 
 /* Selection policy: k = min(max(ceil(n * fraction), 0), n) if fraction > 0
@@ -102,8 +116,10 @@ const char *pqhsa_last_error(void);
 /*
  * Encode key rows with a given trained index: norm, direction, nearest coarse list, residual,
  * nearest codeword per subspace, nibble packing.  For sequence b the token positions
- * sink + slot0[b] + j, j < count[b], of every KV head are encoded into index slots
- * slot0[b] + j.  count_max >= max_b count[b] sizes the grid.
+ * sink + slot0[b] + j, j < count[b], of every KV head are encoded into index positions
+ * slot0[b] + j, whose pos entry is set to the same number (insertion order; sorting the
+ * stored keys by list afterwards is the caller's job).  count_max >= max_b count[b] sizes
+ * the grid.
  * Replaces IVFPQIndex.build_with_codebooks (pq_hsa/index/ivfpq.py:350-433) with
  * slot0 = 0, count = n, and the encode half of IVFPQIndex.add (ivfpq.py:598-645).
  */
@@ -159,7 +175,7 @@ int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max, const flo
 /*
  * Exact top-k of each row of a logit matrix [rows, stride] by radix selection on the fp32
  * bit pattern (no sort); ties at the k boundary go to the lowest index; the k winners are
- * written in ascending index order with their logits.  n[r] and k[r] are per-row device
+ * written (in no particular order) with their logits.  n[r] and k[r] are per-row device
  * arrays.  Replaces torch.topk in the reference path
  * (pq_hsa/attention/sparse_attention.py:661-666) and the binding pq_topk_radix
  * (pq_hsa/kernels/cuda/pq_fused_h20.cu:3624-3688).
@@ -171,13 +187,16 @@ int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t rows, const in
 
 /*
  * The whole single-token decode attention of one layer, for every sequence of the batch:
- * LUT build -> scan + histogram -> threshold -> scan + select + per-list mass -> exact
- * attention over sink, local window and the selected keys read in place from `kv`, merged
- * with the per-list background (list mass x list mean value) in one softmax.
+ * LUT build -> threshold estimate from the sampled keys -> one fused scan that keeps the
+ * candidates above it and sums the other keys' weights per list -> exact radix selection of
+ * the top-k among the candidates (a row whose estimate kept fewer than k keys is re-scanned
+ * in full, so the result is always the exact top-k) -> exact attention over sink, local
+ * window and the selected keys read in place from `kv`, merged with the per-list background
+ * (list mass x list mean value) in one softmax.
  *   q, out     [B, H*G, 128] of q_dtype
  *   seq_lens   i32 [B] device: tokens currently in the cache of each sequence
  *   topk_idx   i32 [BH, G, k_cap], topk_val f32 same shape, topk_cnt i32 [BH, G]: the
- *              selected keys (retrieval-local, ascending) — optional outputs, may be NULL
+ *              selected keys (retrieval-local indices, unordered) — optional outputs, may be NULL
  * Replaces IVFPQSparseAttention.forward_many for mode "hybrid", value mode "centroid",
  * top-k source "all_pq", exact rerank (pq_hsa/attention/sparse_attention.py:245-335,
  * 759-1013), the batched GQA forward (benchmarks/e2e_pq_param_sweep.py:5026-5747) and the
@@ -194,18 +213,28 @@ int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_
                       size_t workspace_bytes, void *stream);
 
 /*
+ * Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full since
+ * the workspace was first used (a device-memory counter inside the workspace, for monitoring).
+ */
+const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t B, int32_t H, int32_t G,
+                                            int64_t n_cap, int32_t num_lists, int32_t k_cap);
+
+/*
  * Hybrid exact attention alone, given the selection and the per-list masses:
- *   list_mass f32 [BH, G, L] = sum over the list's indexed keys of exp(logit - row_max),
- *   row_max f32 [BH, G] (the maximum approximate logit of the row).
+ *   list_mass f32 [BH, G, L] = sum over ALL the list's indexed keys of exp(logit - row_max),
+ *   row_max f32 [BH, G] (the maximum approximate logit of the row),
+ *   key_lists u16 [BH, key_list_stride]: list id of each key by retrieval-local index (the
+ *   selected keys' approximate weights are taken out of their lists first).
  * Mirrors the reference binding pq_exact_attend_paged
  * (pq_hsa/kernels/cuda/pq_fused_h20.cu:905-1084, 3187-3205).
  */
-size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G);
+size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t num_lists);
 int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *out,
                               const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t G,
                               const int32_t *seq_lens, int32_t sink, int32_t full_max,
                               const int32_t *topk_idx, const float *topk_val,
-                              const int32_t *topk_cnt, int32_t k_cap, const float *list_mass,
+                              const int32_t *topk_cnt, int32_t k_cap, const uint16_t *key_lists,
+                              int64_t key_list_stride, const float *list_mass,
                               const float *row_max, float scale, void *workspace,
                               size_t workspace_bytes, void *stream);
 

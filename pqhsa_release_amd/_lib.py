@@ -42,12 +42,19 @@ class Index(ctypes.Structure):
         ("codes", c_void_p),
         ("list_ids", c_void_p),
         ("norms", c_void_p),
+        ("pos", c_void_p),
         ("coarse", c_void_p),
         ("codebooks", c_void_p),
         ("vbar", c_void_p),
         ("vsum", c_void_p),
         ("vcount", c_void_p),
         ("n_idx", c_void_p),
+        ("n_sorted", c_void_p),
+        ("s_codes", c_void_p),
+        ("s_list_ids", c_void_p),
+        ("s_norms", c_void_p),
+        ("s_n", c_void_p),
+        ("s_cap", c_int64),
         ("n_cap", c_int64),
         ("num_lists", c_int32),
         ("batch", c_int32),
@@ -85,10 +92,12 @@ SIGNATURES = {
     "pqhsa_decode_step": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32, c_void_p,
                                          c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_size_t, c_void_p]),
-    "pqhsa_attend_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
+    "pqhsa_decode_rescan_counter": (c_void_p, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
+    "pqhsa_attend_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "pqhsa_hybrid_attend_paged": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32,
                                                  c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
-                                                 c_void_p, c_void_p, c_float, c_void_p, c_size_t, c_void_p]),
+                                                 c_void_p, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_size_t,
+                                                 c_void_p]),
     "pqhsa_paged_gather_range": (ctypes.c_int, [_P(KvView), c_int32, c_int32, c_int64, c_int64, c_void_p, c_void_p,
                                                 c_void_p]),
     "pqhsa_profile_enable": (ctypes.c_int, [c_int32]),

@@ -32,6 +32,7 @@ class PQHSAEngine:
         if self.device.type != "cuda":
             raise RuntimeError("PQ-HSA decode attention needs a GPU: the MI355X kernels have no CPU path")
         self.growth_margin = int(growth_margin)
+        self.resort_tail = 4096     # appended keys tolerated in insertion order before a re-sort
         self.sink, self.local = attention_config.sink_tokens, attention_config.local_window
         self.kv: ops.KvSource | None = None
         self.keys_buf = self.values_buf = None      # dense storage owned by the engine (optional)
@@ -116,10 +117,14 @@ class PQHSAEngine:
         self._ws.clear()
         if old is not None and old.num_lists == num_lists:
             keep = min(old.n_cap, self.index.n_cap)
-            for name in ("codes", "list_ids", "norms"):
+            for name in ("codes", "list_ids", "norms", "pos"):
                 getattr(self.index, name)[:, :keep].copy_(getattr(old, name)[:, :keep])
-            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+            skeep = min(old.s_cap, self.index.s_cap)
+            for name in ("s_codes", "s_list_ids", "s_norms"):
+                getattr(self.index, name)[:, :skeep].copy_(getattr(old, name)[:, :skeep])
+            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount", "s_n"):
                 getattr(self.index, name).copy_(getattr(old, name))
+            self.index.n_sorted_host = list(old.n_sorted_host)
 
     def _retrieval_keys(self, b: int, h: int, start: int, count: int) -> torch.Tensor:
         s = self._sink_end(b)
@@ -167,6 +172,7 @@ class PQHSAEngine:
         if max(counts) > 0:
             ops.encode(self.kv, self.index, self.sink, [0] * self.B, counts, eps=ic.eps)
             ops.value_summaries(self.kv, self.index, self.sink)
+            self.index.finalize_layout(seed=ic.seed)
         self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
         self.index_rebuilds += 1
 
@@ -220,6 +226,8 @@ class PQHSAEngine:
             ops.encode_append(self.kv, self.index, self.sink, old, added, eps=self.index_config.eps)
             self.index_adds += 1
         self.index.set_counts(new)
+        if self.index.tail_max() >= self.resort_tail:
+            self.index.finalize_layout(seed=self.index_config.seed)
 
     def _online_refresh(self, old, added) -> None:
         """EMA move of the coarse centroids and PQ codewords towards the newly indexed keys, then
@@ -253,9 +261,11 @@ class PQHSAEngine:
                 for m in range(ops.SUBSPACES):
                     _ema_rows(idx.codebooks[bh, m], resid[:, m], (words >> (4 * m)) & 15, lr, ic.eps)
         new = [o + a for o, a in zip(old, added)]
+        idx.reset_layout()
         idx.set_counts(new)
         ops.encode(self.kv, idx, self.sink, [0] * self.B, new, eps=ic.eps)
         ops.value_summaries(self.kv, idx, self.sink)
+        idx.finalize_layout(seed=ic.seed)
 
     # ------------------------------------------------------------------ forward
     def forward(self, q: torch.Tensor, groups: int, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -293,8 +303,10 @@ class PQHSAEngine:
         }
         if idx is not None:
             state["index"] = {name: getattr(idx, name).detach().clone() for name in
-                              ("codes", "list_ids", "norms", "coarse", "codebooks", "vbar", "vsum", "vcount")}
+                              ("codes", "list_ids", "norms", "pos", "coarse", "codebooks", "vbar", "vsum", "vcount",
+                               "s_codes", "s_list_ids", "s_norms", "s_n")}
             state["index_counts"] = list(idx.n_host)
+            state["index_sorted"] = list(idx.n_sorted_host)
             state["num_lists"] = idx.num_lists
         if self.keys_buf is not None:
             top = max(self.lens)
@@ -316,10 +328,14 @@ class PQHSAEngine:
             self.index = None
             self._alloc_index(max(int(c) for c in state["index_counts"]), int(state["num_lists"]))
             keep = min(self.index.n_cap, tensors["codes"].shape[1])
-            for name in ("codes", "list_ids", "norms"):
+            for name in ("codes", "list_ids", "norms", "pos"):
                 getattr(self.index, name)[:, :keep].copy_(tensors[name][:, :keep])
-            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+            skeep = min(self.index.s_cap, tensors["s_codes"].shape[1])
+            for name in ("s_codes", "s_list_ids", "s_norms"):
+                getattr(self.index, name)[:, :skeep].copy_(tensors[name][:, :skeep])
+            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount", "s_n"):
                 getattr(self.index, name).copy_(tensors[name])
+            self.index.n_sorted_host = [int(x) for x in state["index_sorted"]]
             self.index.set_counts(state["index_counts"])
         self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
 

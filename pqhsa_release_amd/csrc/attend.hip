@@ -1,14 +1,15 @@
 // Kernel 4: hybrid exact attention over sink + local window + selected keys, read in place
 // from the (paged) K/V cache, merged with the per-list background in one softmax.
 //
-// attend_partial_kernel: grid (splits, G, BH).  Each workgroup takes a contiguous chunk of
-// the row list of one query row (sink rows, local rows, then the selected keys), resolves the
-// rows' addresses once into LDS, computes the exact logits with 16 lanes per 128-element row
-// (one 16-byte load per lane, four rows per wave instruction), and accumulates
-// exp(logit - chunk max) * V in fp32.
-// attend_reduce_kernel: grid (G, BH).  Folds the split partials, rescales the per-list masses
-// to the final row maximum, subtracts the selected keys' approximate weights from their lists,
-// multiplies the remaining masses with the per-list mean values and normalises.
+// attend_partial_kernel: grid (splits, G, BH).  Each workgroup takes a contiguous chunk of the
+// row list of one query row (sink rows, local rows, then the selected keys), resolves the rows'
+// addresses once into LDS, computes the exact logits with 16 lanes per 128-element row (one
+// 16-byte load per lane, four rows per wave instruction) and accumulates
+// exp(logit - chunk max) * V in fp32.  It also takes a slice of the IVF lists and multiplies
+// their background masses with the lists' mean values, so the mean-value table is read once
+// per query row, spread over all splits.
+// attend_reduce_kernel: grid (G, BH).  Folds the split partials under the final row maximum,
+// rescales the two background parts from their reference logits, and normalises.
 #include <cfloat>
 
 #include "common.h"
@@ -16,9 +17,9 @@
 namespace pqhsa {
 
 constexpr int kAttThreads = 256;
-constexpr int kGroupLanes = 16;                            // lanes per K/V row
-constexpr int kGroups = kAttThreads / kGroupLanes;         // rows in flight per pass
-constexpr int kPartWidth = 2 + kD + 2;                     // m, l, acc[128], pad
+constexpr int kGroupLanes = 16;                     // lanes per K/V row
+constexpr int kGroups = kAttThreads / kGroupLanes;  // rows in flight per pass
+constexpr int kPartWidth = 4 + 3 * kD;              // m, l, mass0, mass1, acc[128], bg0[128], bg1[128]
 constexpr int kMaxChunk = 2048;
 constexpr int kMaxSplits = 64;
 
@@ -31,22 +32,17 @@ struct AttendArgs {
     const int32_t *n_idx;     // [B]
     int sink;
     const int32_t *topk_idx;  // [BH*G, k_cap]
-    const float *topk_val;
     const int32_t *topk_cnt;  // [BH*G]
     int64_t k_cap;
     float scale;
     int splits;
     float *partials;          // [BH*G, splits, kPartWidth]
-    // reduce
-    const float *mass;        // element (bh, tile, l, g) at bh*mass_bh + tile*mass_tile + l*mass_l + g*mass_g
-    int64_t mass_bh, mass_tile, mass_l, mass_g;
-    int mass_tile_keys;       // tiles in use = ceil(n / mass_tile_keys)
-    int mass_extra_tile;      // >= 0: one more slot that is always read (fused path)
-    int subtract_selected;    // 1: list masses cover all indexed keys, selected ones are subtracted here
-    const float *row_max;     // [bh * row_max_stride + g]
-    int row_max_stride;
-    const uint16_t *list_ids;
-    int64_t n_cap;
+    // background: two per-list mass tables, element (bh, l, g) at bh*mass_bh + l*mass_l + g*mass_g,
+    // each relative to its own reference logit ref[bh*ref_stride + g]
+    const float *mass0, *mass1;
+    int64_t mass_bh, mass_l, mass_g;
+    const float *ref0, *ref1;
+    int ref_stride;
     const float *vbar;        // [BH, L, 128]
     int L;
 };
@@ -65,6 +61,8 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     __shared__ float red[kGroups][kD];
     __shared__ float red_m[kAttThreads / kWave];
     __shared__ float red_l[kGroups];
+    __shared__ float bg_s[2][2][kD];
+    __shared__ float ms_s[2][kAttThreads / kWave];
     const int tid = threadIdx.x;
     const int split = blockIdx.x, g = blockIdx.y, bh = blockIdx.z;
     const int b = bh / a.H, h = bh % a.H;
@@ -82,14 +80,51 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int cnt = end - start;
     float *part = a.partials + (orow * a.splits + split) * kPartWidth;
 
+    // ---- background slice: lists [l_lo, l_hi) -------------------------------------------
+    {
+        const int per = (a.L + a.splits - 1) / a.splits;
+        const int l_lo = min(split * per, a.L), l_hi = min(l_lo + per, a.L);
+        const int d = tid & (kD - 1);
+        const int half = tid / kD;
+        const float *vb = a.vbar + (size_t)bh * a.L * kD;
+        const float *m0 = a.mass0 ? a.mass0 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
+        const float *m1 = a.mass1 ? a.mass1 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
+        float bg0 = 0.0f, bg1 = 0.0f, s0 = 0.0f, s1 = 0.0f;
+        if (n > 0) {
+#pragma unroll 4
+            for (int l = l_lo + half; l < l_hi; l += 2) {
+                const float v = vb[(size_t)l * kD + d];
+                const float w0 = m0 ? m0[(size_t)l * a.mass_l] : 0.0f;
+                const float w1 = m1 ? m1[(size_t)l * a.mass_l] : 0.0f;
+                bg0 = __builtin_fmaf(w0, v, bg0);
+                bg1 = __builtin_fmaf(w1, v, bg1);
+                if (d == 0) { s0 += w0; s1 += w1; }
+            }
+        }
+        bg_s[0][half][d] = bg0;
+        bg_s[1][half][d] = bg1;
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        if ((tid & (kWave - 1)) == 0) { ms_s[0][tid / kWave] = s0; ms_s[1][tid / kWave] = s1; }
+        __syncthreads();
+        if (tid < kD) {
+            part[4 + kD + tid] = bg_s[0][0][tid] + bg_s[0][1][tid];
+            part[4 + 2 * kD + tid] = bg_s[1][0][tid] + bg_s[1][1][tid];
+        }
+        if (tid == 0) {
+            part[2] = ms_s[0][0] + ms_s[0][1] + ms_s[0][2] + ms_s[0][3];
+            part[3] = ms_s[1][0] + ms_s[1][1] + ms_s[1][2] + ms_s[1][3];
+        }
+    }
+
     if (cnt <= 0) {
         if (tid == 0) { part[0] = -INFINITY; part[1] = 0.0f; }
-        if (tid < kD) part[2 + tid] = 0.0f;
+        if (tid < kD) part[4 + tid] = 0.0f;
         return;
     }
 
-    int64_t *off_s = reinterpret_cast<int64_t *>(smem);           // [chunk] element offsets of the rows
-    float *x_s = reinterpret_cast<float *>(off_s + chunk);         // [chunk] logits, then weights
+    int64_t *off_s = reinterpret_cast<int64_t *>(smem);    // [chunk] element offsets of the rows
+    float *x_s = reinterpret_cast<float *>(off_s + chunk);  // [chunk] logits
 
     // resolve row addresses (block-table lookups happen here, once)
     const int32_t *tk = a.topk_idx + orow * a.k_cap;
@@ -177,7 +212,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         float s = 0.0f;
 #pragma unroll
         for (int r = 0; r < kGroups; ++r) s += red[r][tid];
-        part[2 + tid] = s;
+        part[4 + tid] = s;
     }
     if (tid == 0) {
         float l = 0.0f;
@@ -188,96 +223,70 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     }
 }
 
-__device__ inline float block_sum(float v, float *scratch) {
-    v = wave_sum(v);
-    __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
-    __syncthreads();
-    float s = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kAttThreads / kWave; ++w) s += scratch[w];
-    return s;
-}
-
 template <int QDT>
-__global__ __launch_bounds__(kAttThreads) void attend_reduce_kernel(AttendArgs a) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ float w_s[kMaxSplits];
-    __shared__ float scratch[kAttThreads / kWave];
-    __shared__ float bg_s[kAttThreads];
-    float *mass_s = reinterpret_cast<float *>(smem);  // [L]
-    const int tid = threadIdx.x;
+__global__ __launch_bounds__(kD) void attend_reduce_kernel(AttendArgs a) {
+    const int d = threadIdx.x;
     const int g = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.H, h = bh % a.H;
     const size_t orow = (size_t)bh * a.G + g;
     const int n = a.n_idx[b];
-    const int k = a.topk_cnt[orow];
-    const int L = a.L;
     const float *part = a.partials + orow * a.splits * kPartWidth;
-
-    // final row maximum over exact logits (split maxima) and approximate logits (row max)
-    float m_a = n > 0 ? a.row_max[(size_t)bh * a.row_max_stride + g] : -INFINITY;
-    float m = m_a;
-    for (int s = 0; s < a.splits; ++s) m = fmaxf(m, part[s * kPartWidth]);
+    const float r0 = (n > 0 && a.mass0) ? a.ref0[(size_t)bh * a.ref_stride + g] : -INFINITY;
+    const float r1 = (n > 0 && a.mass1) ? a.ref1[(size_t)bh * a.ref_stride + g] : -INFINITY;
+    float ms0 = 0.0f, ms1 = 0.0f;
+    float m = -INFINITY;
+    for (int s = 0; s < a.splits; ++s) {
+        m = fmaxf(m, part[s * kPartWidth]);
+        ms0 += part[s * kPartWidth + 2];
+        ms1 += part[s * kPartWidth + 3];
+    }
+    // a background part only matters (and only bounds the maximum) when it holds any weight
+    if (ms0 != 0.0f && r0 > -INFINITY) m = fmaxf(m, r0);
+    if (ms1 != 0.0f && r1 > -INFINITY) m = fmaxf(m, r1);
     const size_t qesz = QDT == PQHSA_F32 ? 4 : 2;
     char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
     if (m == -INFINITY) {  // nothing to attend to
-        if (tid < kD) store1<QDT>(orow_p, tid, 0.0f);
+        store1<QDT>(orow_p, d, 0.0f);
         return;
     }
-    if (tid < a.splits) {
-        const float ms = part[tid * kPartWidth];
-        w_s[tid] = ms == -INFINITY ? 0.0f : __expf(ms - m);
+    const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
+    const float f1 = (ms1 != 0.0f && r1 > -INFINITY) ? __expf(r1 - m) : 0.0f;
+    float acc = 0.0f, den = 0.0f;
+    for (int s = 0; s < a.splits; ++s) {
+        const float *p = part + s * kPartWidth;
+        const float w = p[0] == -INFINITY ? 0.0f : __expf(p[0] - m);
+        den = __builtin_fmaf(p[1], w, den);
+        acc = __builtin_fmaf(p[4 + d], w, acc);
+        acc = __builtin_fmaf(p[4 + kD + d], f0, acc);
+        acc = __builtin_fmaf(p[4 + 2 * kD + d], f1, acc);
     }
-    // per-list mass of all indexed keys, rescaled from the approximate row max to m
-    const float resc = m_a == -INFINITY ? 0.0f : __expf(m_a - m);
-    const int tiles = n > 0 ? (n + a.mass_tile_keys - 1) / a.mass_tile_keys : 0;
-    float msum = 0.0f;
-    for (int l = tid; l < L; l += kAttThreads) {
-        float v = 0.0f;
-        const float *src = a.mass + (size_t)bh * a.mass_bh + (size_t)l * a.mass_l + (size_t)g * a.mass_g;
-        for (int t = 0; t < tiles; ++t) v += src[(size_t)t * a.mass_tile];
-        if (a.mass_extra_tile >= 0 && n > 0) v += src[(size_t)a.mass_extra_tile * a.mass_tile];
-        v *= resc;
-        mass_s[l] = v;
-        msum += v;
-    }
-    __syncthreads();
-    float lsum = 0.0f;
-    float acc = 0.0f;
-    if (tid < kD) {
-        for (int s = 0; s < a.splits; ++s) acc = __builtin_fmaf(part[s * kPartWidth + 2 + tid], w_s[s], acc);
-    }
-    if (tid < a.splits) lsum = part[tid * kPartWidth + 1] * w_s[tid];
-    // stand-alone form: the masses cover every indexed key, so the selected keys leave their
-    // lists here (the fused decode step accumulates the masses without them instead)
-    float osum = 0.0f;
-    const int32_t *tk = a.topk_idx + orow * a.k_cap;
-    const float *tv = a.topk_val + orow * a.k_cap;
-    const uint16_t *lids = a.list_ids + (size_t)bh * a.n_cap;
-    if (a.subtract_selected) {
-        for (int t = tid; t < k; t += kAttThreads) {
-            const float o = __expf(tv[t] - m);
-            osum += o;
-            atomicAdd(&mass_s[lids[tk[t]]], -o);
-        }
-    }
-    msum = block_sum(msum, scratch);
-    lsum = block_sum(lsum, scratch);
-    osum = block_sum(osum, scratch);
-    float den = lsum + msum - osum;
+    den += ms0 * f0 + ms1 * f1;
     den = fmaxf(den, FLT_MIN);
+    store1<QDT>(orow_p, d, acc / den);
+}
+
+// Stand-alone form only: the caller's masses cover every indexed key of the row, so the
+// selected keys' approximate weights leave their lists before the background is formed.
+__global__ __launch_bounds__(kAttThreads) void subtract_selected_kernel(const float *list_mass, const float *row_max,
+                                                                        const int32_t *topk_idx, const float *topk_val,
+                                                                        const int32_t *topk_cnt, int64_t k_cap,
+                                                                        const uint16_t *key_lists, int64_t key_stride,
+                                                                        int G, int L, float *mass_adj) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *ms = reinterpret_cast<float *>(smem);
+    const int tid = threadIdx.x;
+    const int g = blockIdx.x, bh = blockIdx.y;
+    const size_t orow = (size_t)bh * G + g;
+    for (int l = tid; l < L; l += kAttThreads) ms[l] = list_mass[orow * L + l];
     __syncthreads();
-    // background: sum_l mass[l] * vbar[l, :]
-    const int d = tid & (kD - 1);
-    const int half = tid / kD;
-    const int per = (L + 1) / 2;
-    const float *vb = a.vbar + (size_t)bh * L * kD;
-    float bg = 0.0f;
-    for (int l = half * per; l < min(L, (half + 1) * per); ++l) bg = __builtin_fmaf(mass_s[l], vb[(size_t)l * kD + d], bg);
-    bg_s[tid] = bg;
+    const float rm = row_max[orow];
+    const int k = topk_cnt[orow];
+    for (int t = tid; t < k; t += kAttThreads) {
+        const int idx = topk_idx[orow * k_cap + t];
+        atomicAdd(&ms[key_lists[(size_t)bh * key_stride + idx]], -__expf(topk_val[orow * k_cap + t] - rm));
+    }
     __syncthreads();
-    if (tid < kD) store1<QDT>(orow_p, tid, (acc + bg_s[tid] + bg_s[tid + kD]) / den);
+    for (int l = tid; l < L; l += kAttThreads) mass_adj[orow * L + l] = ms[l];
 }
 
 int pick_splits(int streams_rows, int rows_max) {
@@ -291,7 +300,7 @@ int pick_splits(int streams_rows, int rows_max) {
 
 size_t attend_partials_bytes(int rows) { return (size_t)rows * kMaxSplits * kPartWidth * sizeof(float); }
 
-int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max, hipStream_t stream) {
+int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max, bool mark, hipStream_t stream) {
     if (BH == 0) return PQHSA_OK;
     PQHSA_REQUIRE(a.G >= 1 && a.G <= 16, "attend: G=%d outside [1, 16]", a.G);
     PQHSA_REQUIRE(a.L <= 4096, "attend: num_lists=%d too large", a.L);
@@ -304,7 +313,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
 #define PQHSA_ATT(KD, QD)                                                                              \
     {                                                                                                  \
         auto kern = attend_partial_kernel<KD, QD>;                                                     \
-        if (lds > 48 * 1024) {                                                                         \
+        if (lds > 32 * 1024) {                                                                         \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                   \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
             if (e != hipSuccess) {                                                                     \
@@ -326,61 +335,68 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
 #undef PQHSA_ATT
     int rc = check_launch("attend_partial");
     if (rc) return rc;
-    if (a.subtract_selected == 0) profile_mark(kProfReduce, stream);
-    const size_t lds2 = (size_t)a.L * sizeof(float);
-    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kAttThreads), lds2,
-                                                     stream, a));
-    if (a.subtract_selected == 0) profile_mark(kProfKernels, stream);
+    if (mark) profile_mark(kProfReduce, stream);
+    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kD), 0, stream, a));
+    if (mark) profile_mark(kProfKernels, stream);
     return check_launch("attend_reduce");
 }
 
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
-                  const float *topk_val, const int32_t *topk_cnt, int k_cap, const float *mass_partial,
-                  int emit_tile_keys, int tiles, const float *row_max_f, float scale, float *partials,
-                  hipStream_t stream) {
+                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
+                  const float *ref_val, const float *ref_extra, float scale, float *partials, hipStream_t stream) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
-    a.topk_idx = topk_idx; a.topk_val = topk_val; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
+    a.topk_idx = topk_idx; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
     a.partials = partials;
     const int64_t L = index->num_lists;
-    a.mass = mass_partial; a.mass_bh = (int64_t)(tiles + 1) * L * GP; a.mass_tile = L * GP; a.mass_l = GP; a.mass_g = 1;
-    a.mass_tile_keys = emit_tile_keys; a.mass_extra_tile = tiles; a.subtract_selected = 0;
-    a.row_max = row_max_f; a.row_max_stride = GP;
-    a.list_ids = index->list_ids; a.n_cap = index->n_cap; a.vbar = index->vbar; a.L = index->num_lists;
-    return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, stream);
+    a.mass0 = mass; a.mass1 = mass_extra; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
+    a.ref0 = ref_val; a.ref1 = ref_extra; a.ref_stride = GP;
+    a.vbar = index->vbar; a.L = index->num_lists;
+    return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream);
 }
 
 }  // namespace pqhsa
 
 using namespace pqhsa;
 
-extern "C" size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G) {
-    return attend_partials_bytes(B * H * G) + 256;
+extern "C" size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t num_lists) {
+    return attend_partials_bytes(B * H * G) + (size_t)B * H * G * num_lists * sizeof(float) + 512;
 }
 
 extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
                                          const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
                                          int32_t full_max, const int32_t *topk_idx, const float *topk_val,
-                                         const int32_t *topk_cnt, int32_t k_cap, const float *list_mass,
-                                         const float *row_max, float scale, void *workspace, size_t workspace_bytes,
-                                         void *stream) {
-    PQHSA_REQUIRE(q && out && index && seq_lens && topk_idx && topk_val && topk_cnt && list_mass && row_max && workspace,
+                                         const int32_t *topk_cnt, int32_t k_cap, const uint16_t *key_lists,
+                                         int64_t key_list_stride, const float *list_mass, const float *row_max,
+                                         float scale, void *workspace, size_t workspace_bytes, void *stream_v) {
+    PQHSA_REQUIRE(q && out && index && seq_lens && topk_idx && topk_val && topk_cnt && key_lists && list_mass &&
+                      row_max && workspace,
                   "hybrid_attend_paged: NULL argument");
     int rc = validate_view(kv);
     if (rc) return rc;
     const int BH = index->batch * index->kv_heads;
-    PQHSA_REQUIRE(workspace_bytes >= pqhsa_attend_workspace_bytes(index->batch, index->kv_heads, G),
+    const int L = index->num_lists;
+    PQHSA_REQUIRE(workspace_bytes >= pqhsa_attend_workspace_bytes(index->batch, index->kv_heads, G, L),
                   "hybrid_attend_paged: workspace too small");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    if (BH == 0) return PQHSA_OK;
+    char *w = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
+    float *partials = reinterpret_cast<float *>(w);
+    float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G));
+    hipLaunchKernelGGL(subtract_selected_kernel, dim3(G, BH), dim3(kAttThreads), (size_t)L * sizeof(float), stream,
+                       list_mass, row_max, topk_idx, topk_val, topk_cnt, (int64_t)k_cap, key_lists, key_list_stride, G,
+                       L, mass_adj);
+    rc = check_launch("subtract_selected");
+    if (rc) return rc;
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
-    a.topk_idx = topk_idx; a.topk_val = topk_val; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
-    a.partials = reinterpret_cast<float *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
-    a.mass = list_mass; a.mass_bh = (int64_t)G * index->num_lists; a.mass_tile = 0; a.mass_l = 1;
-    a.mass_g = index->num_lists; a.mass_tile_keys = 1 << 30; a.mass_extra_tile = -1; a.subtract_selected = 1;
-    a.row_max = row_max; a.row_max_stride = G;
-    a.list_ids = index->list_ids; a.n_cap = index->n_cap; a.vbar = index->vbar; a.L = index->num_lists;
-    return launch_attend(a, q_dtype, kv->dtype, BH, full_max + k_cap, static_cast<hipStream_t>(stream));
+    a.topk_idx = topk_idx; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
+    a.partials = partials;
+    a.mass0 = mass_adj; a.mass1 = nullptr; a.mass_bh = (int64_t)G * L; a.mass_l = 1; a.mass_g = L;
+    a.ref0 = row_max; a.ref1 = nullptr; a.ref_stride = G;
+    a.vbar = index->vbar; a.L = L;
+    return launch_attend(a, q_dtype, kv->dtype, BH, full_max + k_cap, false, stream);
 }

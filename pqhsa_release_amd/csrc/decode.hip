@@ -1,26 +1,21 @@
-// One decode-attention step of a layer: orchestration of the four kernels on one stream,
-// plus the carve-up of the caller's workspace.
+// One decode-attention step of a layer: orchestration of the kernels on one stream, plus the
+// carve-up of the caller's workspace.
 #include "common.h"
 
 namespace pqhsa {
-
-// declared in the kernel translation units
-struct ScanArgs;
-struct SelectArgs;
-struct AttendArgs;
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps, float *qnorm,
                      float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, hipStream_t stream);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select, uint32_t *hist,
-                       uint32_t *rowmax, uint32_t *emit_count, uint32_t *thr_bin, uint32_t *thr_above, int32_t *k_row,
-                       float *row_max_f, void *pairs, float *mass_partial, int emit_tile_keys, int32_t *topk_idx,
-                       float *topk_val, int32_t *topk_cnt, hipStream_t stream);
+                       uint32_t *emit_count, uint32_t *thr_bin, int32_t *k_row, float *ref_val, float *ref_extra,
+                       void *pairs, uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans,
+                       int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
+                       hipStream_t stream);
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
-                  const float *topk_val, const int32_t *topk_cnt, int k_cap, const float *mass_partial,
-                  int emit_tile_keys, int tiles, const float *row_max_f, float scale, float *partials,
-                  hipStream_t stream);
+                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
+                  const float *ref_val, const float *ref_extra, float scale, float *partials, hipStream_t stream);
 int emit_tile_keys_for(int64_t n_cap, int streams);
 size_t attend_partials_bytes(int rows);
 
@@ -28,19 +23,20 @@ static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Carve {
     float *qnorm, *lut, *ls;
-    uint32_t *hist, *rowmax, *emit_count;
+    uint32_t *hist, *emit_count, *rescans;
+    float *mass;
     size_t zero_words;
-    uint32_t *thr_bin, *thr_above;
+    uint32_t *thr_bin;
     int32_t *k_row;
-    float *row_max_f;
+    float *ref_val, *ref_extra, *mass_extra;
     void *pairs;
-    float *mass_partial;
+    uint16_t *aux;
     int32_t *topk_idx;
     float *topk_val;
     int32_t *topk_cnt;
     float *partials;
     size_t total;
-    int tile_keys, tiles;
+    int tile_keys;
 };
 
 static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_cap) {
@@ -49,7 +45,6 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     const size_t GP = padded_groups(G);
     const size_t rows = BH * GP;
     c.tile_keys = emit_tile_keys_for(n_cap, (int)BH);
-    c.tiles = (int)((n_cap + c.tile_keys - 1) / c.tile_keys);
     size_t off = 0;
     auto take = [&](size_t bytes) {
         char *p = base + off;
@@ -59,17 +54,19 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.qnorm = reinterpret_cast<float *>(take(rows * 4));
     c.lut = reinterpret_cast<float *>(take(rows * kM * kCodes * 4));
     c.ls = reinterpret_cast<float *>(take(rows * L * 4));
-    const size_t z0 = off;
+    const size_t z0 = off;  // everything from here to zero_words is cleared at the start of a step
     c.hist = reinterpret_cast<uint32_t *>(take(rows * kHistBins * 4));
-    c.rowmax = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
+    c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
+    c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
     c.thr_bin = reinterpret_cast<uint32_t *>(take(rows * 4));
-    c.thr_above = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.k_row = reinterpret_cast<int32_t *>(take(rows * 4));
-    c.row_max_f = reinterpret_cast<float *>(take(rows * 4));
+    c.ref_val = reinterpret_cast<float *>(take(rows * 4));
+    c.ref_extra = reinterpret_cast<float *>(take(rows * 4));
+    c.mass_extra = reinterpret_cast<float *>(take(rows * L * 4));
     c.pairs = take(rows * (size_t)n_cap * 8);
-    c.mass_partial = reinterpret_cast<float *>(take(BH * (c.tiles + 1) * (size_t)L * GP * 4));
+    c.aux = reinterpret_cast<uint16_t *>(take(rows * (size_t)n_cap * 2));
     c.topk_idx = reinterpret_cast<int32_t *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_val = reinterpret_cast<float *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_cnt = reinterpret_cast<int32_t *>(take(BH * G * 4));
@@ -87,6 +84,14 @@ extern "C" size_t pqhsa_decode_workspace_bytes(int32_t B, int32_t H, int32_t G, 
     return carve(nullptr, B, H, G, n_cap, num_lists, k_cap).total + 256;
 }
 
+// Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full, since
+// the workspace was created (device counter; reading it synchronises nothing by itself).
+extern "C" const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t B, int32_t H, int32_t G,
+                                                       int64_t n_cap, int32_t num_lists, int32_t k_cap) {
+    char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
+    return carve(base, B, H, G, n_cap, num_lists, k_cap).rescans;
+}
+
 extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
                                  const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
                                  int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,
@@ -98,6 +103,9 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     PQHSA_REQUIRE(G >= 1 && G <= 16, "decode_step: G=%d outside [1, 16]", G);
     PQHSA_REQUIRE(index->n_cap % 8 == 0 && index->n_cap > 0, "decode_step: n_cap=%lld must be a positive multiple of 8",
                   (long long)index->n_cap);
+    PQHSA_REQUIRE(index->s_cap % 8 == 0 && index->s_cap > 0 && index->s_codes && index->s_list_ids && index->s_norms &&
+                      index->s_n && index->n_sorted && index->pos,
+                  "decode_step: the index has no sorted layout / sample (s_cap=%lld)", (long long)index->s_cap);
     PQHSA_REQUIRE(n_max >= 0 && n_max <= index->n_cap, "decode_step: n_max=%d outside [0, n_cap]", n_max);
     PQHSA_REQUIRE(select->k_cap >= resolve_k(n_max, select->fraction, select->topk),
                   "decode_step: k_cap=%d is below the k of n_max=%d", select->k_cap, n_max);
@@ -120,11 +128,11 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     rc = launch_lut_build(q, q_dtype, index, G, eps, c.qnorm, c.lut, c.ls, c.hist, c.zero_words, stream);
     if (rc) return rc;
     profile_mark(kProfHist, stream);
-    rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.hist, c.rowmax, c.emit_count,
-                            c.thr_bin, c.thr_above, c.k_row, c.row_max_f, c.pairs, c.mass_partial, c.tile_keys,
-                            topk_idx, topk_val, topk_cnt, stream);
+    rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.hist, c.emit_count, c.thr_bin,
+                            c.k_row, c.ref_val, c.ref_extra, c.pairs, c.aux, c.mass, c.mass_extra, c.rescans,
+                            c.tile_keys, topk_idx, topk_val, topk_cnt, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
-                         topk_val, topk_cnt, select->k_cap, c.mass_partial, c.tile_keys, c.tiles, c.row_max_f, scale,
-                         c.partials, stream);
+                         topk_cnt, select->k_cap, c.mass, c.mass_extra, c.ref_val, c.ref_extra, scale, c.partials,
+                         stream);
 }

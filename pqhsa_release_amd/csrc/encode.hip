@@ -22,6 +22,7 @@ struct EncodeArgs {
     uint32_t *codes;
     uint16_t *list_ids;
     float *norms;
+    int32_t *pos;
     int64_t n_cap;
     float *vsum, *vcount, *vbar;
     const int32_t *n_idx;
@@ -121,6 +122,7 @@ __global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) 
     a.codes[o] = word;
     a.list_ids[o] = (uint16_t)best;
     a.norms[o] = nrm;
+    if (a.pos) a.pos[o] = slot;
 }
 
 __device__ inline unsigned long long wave_min_u64(unsigned long long v, int width) {
@@ -210,6 +212,7 @@ __global__ __launch_bounds__(kEncThreads) void encode_row_kernel(EncodeArgs a) {
         a.codes[o] = word;
         a.list_ids[o] = (uint16_t)list;
         a.norms[o] = nrm_s;
+        if (a.pos) a.pos[o] = slot;
     }
 }
 
@@ -256,16 +259,19 @@ __global__ __launch_bounds__(kD) void value_summaries_kernel(EncodeArgs a) {
     if (d < kListsPerWg) cnt_s[d] = 0.0f;
     __syncthreads();
     __shared__ int rel[kD];
+    __shared__ int tok[kD];
     const uint16_t *lids = a.list_ids + (size_t)bh * a.n_cap;
+    const int32_t *pos = a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr;
     for (int i0 = 0; i0 < n; i0 += kD) {
         __syncthreads();
         rel[d] = (i0 + d < n) ? (int)lids[i0 + d] - l0 : -1;
+        tok[d] = (i0 + d < n && pos) ? pos[i0 + d] : i0 + d;  // retrieval-local index of the stored key
         __syncthreads();
         const int lim = min(kD, n - i0);
         for (int t = 0; t < lim; ++t) {
             const int l = rel[t];
             if (l < 0 || l >= kListsPerWg) continue;
-            const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + i0 + t) * esz;
+            const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + tok[t]) * esz;
             acc[l][d] += load1<DT>(row, d);
             if (d == 0) cnt_s[l] += 1.0f;
         }
@@ -309,7 +315,8 @@ static int fill_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *
     a.kv = make_view(kv);
     a.H = index->kv_heads; a.L = index->num_lists; a.sink = sink; a.slot0 = slot0; a.count = count;
     a.coarse = index->coarse; a.codebooks = index->codebooks; a.eps = eps;
-    a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.n_cap = index->n_cap;
+    a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = index->pos;
+    a.n_cap = index->n_cap;
     a.vsum = index->vsum; a.vcount = index->vcount; a.vbar = index->vbar; a.n_idx = index->n_idx;
     return PQHSA_OK;
 }

@@ -122,7 +122,16 @@ def kv_paged(kv_cache: torch.Tensor, block_table: torch.Tensor) -> KvSource:
 
 # --------------------------------------------------------------------------- device index
 class DeviceIndex:
-    """Device-resident IVF-PQ index of B x H streams (structure of arrays, spare capacity)."""
+    """Device-resident IVF-PQ index of B x H streams (structure of arrays, spare capacity).
+
+    Stored keys sit in two regions: the first ``n_sorted`` positions are ordered by list id
+    (``pos`` maps a position back to the key's retrieval-local index), keys appended later
+    follow in insertion order until ``finalize_layout`` sorts everything again.  A fixed random
+    subset of the stored keys is kept in the ``s_*`` arrays for the threshold estimate.
+    """
+
+    SAMPLE_RATE = 32
+    SAMPLE_MIN = 1024
 
     def __init__(self, batch: int, kv_heads: int, num_lists: int, n_cap: int, device) -> None:
         n_cap = max(8, (int(n_cap) + 7) // 8 * 8)
@@ -133,32 +142,86 @@ class DeviceIndex:
         self.codes = torch.zeros(bh, n_cap, dtype=torch.int32, device=dev)       # bit pattern of u32
         self.list_ids = torch.zeros(bh, n_cap, dtype=torch.int16, device=dev)    # bit pattern of u16
         self.norms = torch.zeros(bh, n_cap, dtype=torch.float32, device=dev)
+        self.pos = torch.arange(n_cap, dtype=torch.int32, device=dev).repeat(bh, 1)
         self.coarse = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
         self.codebooks = torch.zeros(bh, SUBSPACES, CODES, SUBDIM, dtype=torch.float32, device=dev)
         self.vbar = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
         self.vsum = torch.zeros(bh, num_lists, HEAD_DIM, dtype=torch.float32, device=dev)
         self.vcount = torch.zeros(bh, num_lists, dtype=torch.float32, device=dev)
         self.n_idx = torch.zeros(batch, dtype=torch.int32, device=dev)
-        self.n_host = [0] * batch          # host mirror of n_idx
+        self.n_sorted = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.s_n = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.s_cap = max(8, (self.sample_size(n_cap) + 7) // 8 * 8)
+        self.s_codes = torch.zeros(bh, self.s_cap, dtype=torch.int32, device=dev)
+        self.s_list_ids = torch.zeros(bh, self.s_cap, dtype=torch.int16, device=dev)
+        self.s_norms = torch.zeros(bh, self.s_cap, dtype=torch.float32, device=dev)
+        self.n_host = [0] * batch          # host mirrors
+        self.n_sorted_host = [0] * batch
         self._struct = None
+
+    @classmethod
+    def sample_size(cls, n: int) -> int:
+        return min(n, max((n + cls.SAMPLE_RATE - 1) // cls.SAMPLE_RATE, cls.SAMPLE_MIN))
 
     @property
     def n_max(self) -> int:
         return max(self.n_host) if self.n_host else 0
 
     def set_counts(self, counts) -> None:
+        """Keys stored per sequence (a fresh encode leaves them in insertion order: nothing is
+        sorted, nothing sampled, until ``finalize_layout``)."""
         self.n_host = [int(c) for c in counts]
         if max(self.n_host, default=0) > self.n_cap:
             raise ValueError("index capacity exceeded")
-        self.n_idx.copy_(torch.tensor(self.n_host, dtype=torch.int32), non_blocking=False)
+        self.n_sorted_host = [min(s, n) for s, n in zip(self.n_sorted_host, self.n_host)]
+        self.n_idx.copy_(torch.tensor(self.n_host, dtype=torch.int32))
+        self.n_sorted.copy_(torch.tensor(self.n_sorted_host, dtype=torch.int32))
+
+    def reset_layout(self) -> None:
+        """Declare the stored keys to be in insertion order again (after a bulk re-encode)."""
+        self.n_sorted_host = [0] * self.batch
+        self.n_sorted.zero_()
+        self.s_n.zero_()
+        self.pos.copy_(torch.arange(self.n_cap, dtype=torch.int32, device=self.device).expand_as(self.pos))
+
+    def finalize_layout(self, seed: int = 0) -> None:
+        """Order every stream's stored keys by list id (stable, so keys of a list keep their
+        insertion order) and draw the sampled subset.  Host-side torch ops, off the decode path."""
+        h = self.kv_heads
+        gen = torch.Generator(device="cpu")
+        gen.manual_seed(int(seed))
+        for b, n in enumerate(self.n_host):
+            rows = slice(b * h, (b + 1) * h)
+            if n > 0:
+                lids = (self.list_ids[rows, :n].to(torch.int64) & 0xFFFF)
+                order = torch.argsort(lids, dim=1, stable=True)
+                for t in (self.codes, self.list_ids, self.norms, self.pos):
+                    t[rows, :n] = torch.gather(t[rows, :n], 1, order)
+                ns = self.sample_size(n)
+                pick = torch.randperm(n, generator=gen)[:ns].sort().values.to(self.device)
+                self.s_codes[rows, :ns] = self.codes[rows][:, pick]
+                self.s_list_ids[rows, :ns] = self.list_ids[rows][:, pick]
+                self.s_norms[rows, :ns] = self.norms[rows][:, pick]
+            else:
+                ns = 0
+            self.n_sorted_host[b] = n
+        self.n_sorted.copy_(torch.tensor(self.n_sorted_host, dtype=torch.int32))
+        self.s_n.copy_(torch.tensor([self.sample_size(n) if n > 0 else 0 for n in self.n_host], dtype=torch.int32))
+
+    def tail_max(self) -> int:
+        return max((n - s for n, s in zip(self.n_host, self.n_sorted_host)), default=0)
 
     def struct(self) -> Index:
         if self._struct is None:
             s = Index()
             s.codes, s.list_ids, s.norms = self.codes.data_ptr(), self.list_ids.data_ptr(), self.norms.data_ptr()
+            s.pos = self.pos.data_ptr()
             s.coarse, s.codebooks = self.coarse.data_ptr(), self.codebooks.data_ptr()
             s.vbar, s.vsum, s.vcount = self.vbar.data_ptr(), self.vsum.data_ptr(), self.vcount.data_ptr()
-            s.n_idx, s.n_cap = self.n_idx.data_ptr(), self.n_cap
+            s.n_idx, s.n_sorted = self.n_idx.data_ptr(), self.n_sorted.data_ptr()
+            s.s_codes, s.s_list_ids, s.s_norms = (self.s_codes.data_ptr(), self.s_list_ids.data_ptr(),
+                                                  self.s_norms.data_ptr())
+            s.s_n, s.s_cap, s.n_cap = self.s_n.data_ptr(), self.s_cap, self.n_cap
             s.num_lists, s.batch, s.kv_heads = self.num_lists, self.batch, self.kv_heads
             self._struct = s
         return self._struct
@@ -167,12 +230,29 @@ class DeviceIndex:
         return ctypes.byref(self.struct())
 
     def list_ids_long(self) -> torch.Tensor:
-        """List ids as int64 (the stored int16 tensor holds uint16 bit patterns)."""
+        """List ids by stored position as int64 (the int16 tensor holds uint16 bit patterns)."""
         return self.list_ids.to(torch.int64) & 0xFFFF
 
-    def packed_bytes(self) -> torch.Tensor:
-        """The reference's ``[N, 4]`` uint8 packing is the little-endian view of the code words."""
-        return self.codes.view(torch.uint8).reshape(self.codes.shape[0], self.n_cap, 4)
+    def by_key(self, bh: int, n: int):
+        """(codes, list_ids, norms) of stream ``bh`` indexed by retrieval-local key index."""
+        where = self.pos[bh, :n].to(torch.int64)
+        out = []
+        for t in (self.codes, self.list_ids, self.norms):
+            u = torch.empty_like(t[bh, :n])
+            u[where] = t[bh, :n]
+            out.append(u)
+        return tuple(out)
+
+    def key_lists(self) -> torch.Tensor:
+        """List id of every key by retrieval-local index, ``[BH, n_cap]`` int16 (u16 bits)."""
+        out = torch.zeros_like(self.list_ids)
+        out.scatter_(1, self.pos.to(torch.int64), self.list_ids)
+        return out
+
+    def packed_bytes(self, bh: int, n: int) -> torch.Tensor:
+        """The reference's ``[N, 4]`` uint8 packing (by key index) is the little-endian view of
+        the code words."""
+        return self.by_key(bh, n)[0].contiguous().view(torch.uint8).reshape(n, 4)
 
 
 def _i32(values, device) -> torch.Tensor:
@@ -269,6 +349,15 @@ class DecodeWorkspace:
         self.topk_idx = torch.full((rows, self.k_cap), -1, dtype=torch.int32, device=index.device)
         self.topk_val = torch.zeros(rows, self.k_cap, dtype=torch.float32, device=index.device)
         self.topk_cnt = torch.zeros(rows, dtype=torch.int32, device=index.device)
+        self.buf.zero_()
+        self._shape = (index.batch, index.kv_heads, groups, index.n_cap, index.num_lists, self.k_cap)
+
+    def rescans(self) -> int:
+        """Rows re-scanned in full because the sampled threshold kept fewer than k candidates
+        (synchronises: reads a device counter)."""
+        ptr = _lib.load().pqhsa_decode_rescan_counter(self.buf.data_ptr(), *self._shape)
+        off = ptr - self.buf.data_ptr()
+        return int(self.buf[off : off + 4].view(torch.int32).item())
 
 
 def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
@@ -335,17 +424,18 @@ class DecodeCall:
 
 def hybrid_attend_paged(q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int, full_max: int,
                         topk_idx, topk_val, topk_cnt, list_mass, row_max, scale: float) -> torch.Tensor:
-    """Exact hybrid attention given a selection and per-list masses (``list_mass [BH, G, L]``
-    relative to ``row_max [BH, G]``)."""
+    """Exact hybrid attention given a selection and per-list masses (``list_mass [BH, G, L]`` over
+    all indexed keys of each list, relative to ``row_max [BH, G]``)."""
     _need_cuda(q, out, topk_idx, topk_val, topk_cnt, list_mass, row_max)
     lib = _lib.load()
-    ws_bytes = lib.pqhsa_attend_workspace_bytes(index.batch, index.kv_heads, groups)
+    ws_bytes = lib.pqhsa_attend_workspace_bytes(index.batch, index.kv_heads, groups, index.num_lists)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    key_lists = index.key_lists()
     rc = lib.pqhsa_hybrid_attend_paged(q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(),
                                        groups, seq_lens.data_ptr(), int(sink), int(full_max), topk_idx.data_ptr(),
                                        topk_val.data_ptr(), topk_cnt.data_ptr(), topk_idx.shape[-1],
-                                       list_mass.data_ptr(), row_max.data_ptr(), float(scale), ws.data_ptr(),
-                                       ws_bytes, _stream())
+                                       key_lists.data_ptr(), index.n_cap, list_mass.data_ptr(), row_max.data_ptr(),
+                                       float(scale), ws.data_ptr(), ws_bytes, _stream())
     _lib.check(rc, "pqhsa_hybrid_attend_paged")
     return out
 

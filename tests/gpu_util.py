@@ -93,11 +93,13 @@ class Problem:
             vc[blk, pos % block_size, h] = self.values[b, h].to(self.dtype)
         return cache.to(device), table.to(device)
 
-    def device_index(self, device="cuda", spare=64, upload_codes=True) -> ops.DeviceIndex:
+    def device_index(self, device="cuda", spare=64, upload_codes=True, finalize=True) -> ops.DeviceIndex:
         idx = ops.DeviceIndex(self.B, self.H, self.L, self.n_max + spare, device)
         for (b, h), ix in self.index.items():
             bh = b * self.H + h
             n = self.n(b)
+            if ix is None:
+                continue
             idx.coarse[bh] = torch.from_numpy(ix["coarse"]).to(device)
             idx.codebooks[bh] = torch.from_numpy(ix["codebooks"]).to(device)
             if upload_codes:
@@ -106,6 +108,8 @@ class Problem:
                 idx.norms[bh, :n] = torch.from_numpy(ix["norms"]).to(device)
                 idx.vbar[bh] = torch.from_numpy(ix["vbar"]).to(device)
         idx.set_counts([self.n(b) for b in range(self.B)])
+        if upload_codes and finalize:
+            idx.finalize_layout()      # list-sorted storage + sampled subset, as after a build
         return idx
 
     def seq_lens(self, device="cuda") -> torch.Tensor:

@@ -30,7 +30,7 @@ def test_version_and_helpers_run_without_a_gpu():
     assert [lib.pqhsa_padded_groups(g) for g in (1, 2, 3, 4, 5, 7, 8, 9, 16)] == [1, 2, 4, 4, 8, 8, 8, 16, 16]
     assert lib.pqhsa_decode_workspace_bytes(1, 8, 4, 32704, 512, 654) > 0
     assert lib.pqhsa_topk_workspace_bytes(4, 1000) > 0
-    assert lib.pqhsa_attend_workspace_bytes(1, 8, 4) > 0
+    assert lib.pqhsa_attend_workspace_bytes(1, 8, 4, 512) > 0
 
 
 def test_struct_layouts_match_the_header():
@@ -38,5 +38,5 @@ def test_struct_layouts_match_the_header():
 
     # sizes implied by include/pqhsa.h on LP64: pointers and int64 8-byte aligned
     assert ctypes.sizeof(_lib.KvView) == 8 + 8 + 4 + 4 + 8 * 4 + 4 + 4 + 8
-    assert ctypes.sizeof(_lib.Index) == 9 * 8 + 8 + 4 * 3 + 4
+    assert ctypes.sizeof(_lib.Index) == 15 * 8 + 2 * 8 + 4 * 3 + 4
     assert ctypes.sizeof(_lib.Select) == 16

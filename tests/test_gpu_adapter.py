@@ -52,9 +52,10 @@ def _words(packed_np):
 def _index_of(engine, bh, n):
     """Download one stream's index in the oracle's format."""
     idx = engine.index
+    codes, lists, norms = idx.by_key(bh, n)          # stored list-sorted; the oracle wants key order
     return {"coarse": idx.coarse[bh].cpu().numpy(), "codebooks": idx.codebooks[bh].cpu().numpy(),
-            "codes": u32(idx.codes[bh, :n]), "list_ids": u16(idx.list_ids[bh, :n]),
-            "norms": idx.norms[bh, :n].cpu().numpy(), "vbar": idx.vbar[bh].cpu().numpy()}
+            "codes": u32(codes), "list_ids": u16(lists), "norms": norms.cpu().numpy(),
+            "vbar": idx.vbar[bh].cpu().numpy()}
 
 
 def _margin_ok(logits, got_idx, ref_idx):
@@ -96,11 +97,12 @@ def test_engine_reproduces_reference_vectors_with_the_reference_index(golden_dir
         tidx, tval, tcnt = eng.last_topk(G)
         for h in range(H):
             ref_lists, ref_words = fx[f"{tag}_list_ids"][h], _words(fx[f"{tag}_packed"][h])
-            lists, codes = u16(eng.index.list_ids[h, :n]), u32(eng.index.codes[h, :n])
+            codes_t, lists_t, norms_t = eng.index.by_key(h, n)
+            lists, codes = u16(lists_t), u32(codes_t)
             # integer parity with the reference (these fixtures hold no argmin near-tie: the
             # fixed-order oracle reproduces them exactly too, tests/test_oracle_golden.py)
             assert np.array_equal(lists, ref_lists) and np.array_equal(codes, ref_words)
-            np.testing.assert_allclose(eng.index.norms[h, :n].cpu().numpy(), fx[f"{tag}_norms"][h], rtol=1e-6)
+            np.testing.assert_allclose(norms_t.cpu().numpy(), fx[f"{tag}_norms"][h], rtol=1e-6)
             np.testing.assert_allclose(eng.index.vbar[h].cpu().numpy(), fx[f"{tag}_vbar"][h], atol=1e-5)
             k = fx[f"{tag}_topk_idx"].shape[2]
             got = tidx.reshape(H, G, -1)[h, :, :k].cpu().numpy()
@@ -147,7 +149,7 @@ def _oracle_check(eng, keys, values, q_step, groups, length, fraction, tol):
             k = want_idx.shape[1]
             got = tidx.reshape(eng.B, eng.H, groups, -1)[b, h, :, :k].cpu().numpy()
             for g in range(groups):
-                assert np.array_equal(got[g], np.sort(want_idx[g])), (b, h, g)
+                assert np.array_equal(np.sort(got[g]), np.sort(want_idx[g])), (b, h, g)
             outs.append(want_out)
     return np.stack(outs).reshape(eng.B, eng.H * groups, DIM), worst
 
@@ -207,7 +209,8 @@ def test_plain_adapter_multi_query_and_state_round_trip():
     state = ad.state_dict()
     clone = IVFPQDecodeAttentionAdapter.from_state_dict(state)
     again = clone.forward(queries)
-    assert torch.equal(again.context, res.context)
+    # same index, same selection; float sums may differ in the last bits (atomic accumulation order)
+    np.testing.assert_allclose(again.context.cpu().numpy(), res.context.cpu().numpy(), atol=1e-5)
     assert clone.leading_shape == (2, H)
 
 

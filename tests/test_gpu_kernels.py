@@ -44,7 +44,7 @@ def test_encode_bulk_and_row_kernels_match_oracle_bitwise(dtype, paged):
         assert np.array_equal(u16(idx.list_ids[bh, :n]), ix["list_ids"]), (b, h)
         assert np.array_equal(idx.norms[bh, :n].cpu().numpy(), ix["norms"]), (b, h)
     # the reference's [N, 4] uint8 packing is the byte view of the words
-    packed = idx.packed_bytes()[0, : p.n(0)].cpu().numpy()
+    packed = idx.packed_bytes(0, p.n(0)).cpu().numpy()
     w = p.index[0, 0]["codes"]
     assert np.array_equal(packed[:, 1] >> 4, (w >> 12) & 15) and np.array_equal(packed[:, 0] & 15, w & 15)
 
@@ -53,7 +53,7 @@ def test_encode_bulk_and_row_kernels_match_oracle_bitwise(dtype, paged):
 def test_value_summaries_and_append_match_oracle(dtype):
     dev = _cuda()
     p = Problem(lens=[700], heads=2, lists=32, dtype=dtype, seed=5)
-    idx = p.device_index(dev)
+    idx = p.device_index(dev, finalize=False)       # appends go to the insertion-order tail
     kv = ops.kv_contiguous(*p.dense_kv())
     idx.vbar.zero_()
     n = p.n(0)
@@ -118,7 +118,7 @@ def test_topk_radix_on_logit_matrix_with_ties():
     for r in range(rows):
         want_idx, _ = fixed.topk(logits[r, : n[r]], k[r])
         got = idx[r, : k[r]]
-        assert np.array_equal(got, np.sort(want_idx)), r      # ascending index order, exact set
+        assert np.array_equal(np.sort(got), np.sort(want_idx)), r      # exact set
         assert np.array_equal(val[r, : k[r]], logits[r, got]), r
 
 
@@ -163,7 +163,7 @@ def test_decode_step_topk_bitexact_and_output_close(case):
             for g in range(p.G):
                 assert cnt[b, h, g] == k
                 got = tidx[b, h, g, :k]
-                assert np.array_equal(got, np.sort(want_idx[g])), (b, h, g)          # bit-exact set
+                assert np.array_equal(np.sort(got), np.sort(want_idx[g])), (b, h, g)  # bit-exact set
                 assert np.array_equal(tval[b, h, g, :k], logits[g, got]), (b, h, g)  # and their logits
             err = np.abs(o[b, h] - want_out)
             assert (err <= tol + rel * np.abs(want_out)).all(), (b, h, q_dtype, err.max())
