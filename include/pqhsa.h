@@ -255,12 +255,15 @@ int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq,
  * read back only at collect time (the sync-free event log of the reference,
  * benchmarks/cuda_event_log.py:49-88).  pqhsa_profile_enable creates events for up to
  * max_steps decode steps; pqhsa_profile_collect synchronises the recorded events, writes the
- * average milliseconds of the 7 kernels (lut_build, scan_hist, thresh, scan_emit,
- * select_final, attend_partial, attend_reduce) and the number of steps seen, and turns
- * profiling off.  Not thread-safe; meant for benchmarks.
+ * average milliseconds of the 6 kernels (lut_build, sample_thresh, scan_emit, select_final,
+ * attend_partial, attend_reduce) and the number of steps seen, and turns profiling off.
+ * pqhsa_profile_only(kernel), called after enable, restricts the log to the two events around
+ * one kernel (-1: all), so that a timed run carries two event records per step instead of
+ * seven; the other entries of kernel_ms are then 0.  Not thread-safe; meant for benchmarks.
  */
-#define PQHSA_PROFILE_KERNELS 7
+#define PQHSA_PROFILE_KERNELS 6
 int pqhsa_profile_enable(int32_t max_steps);
+int pqhsa_profile_only(int32_t kernel);
 int pqhsa_profile_collect(float *kernel_ms, int32_t *steps);
 
 #ifdef __cplusplus

@@ -52,10 +52,12 @@ int validate_view(const pqhsa_kv_view *kv) {
 static std::vector<hipEvent_t> g_events;
 static int g_prof_steps = 0, g_prof_step = 0;
 static bool g_prof_on = false;
+static int g_prof_only = -1;  // >= 0: only this kernel is bracketed by events
 
 void profile_mark(int slot, hipStream_t stream) {
     if (!g_prof_on || g_prof_step >= g_prof_steps) return;
-    (void)hipEventRecord(g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot], stream);
+    if (g_prof_only < 0 || slot == g_prof_only || slot == g_prof_only + 1)
+        (void)hipEventRecord(g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot], stream);
     if (slot == kProfKernels) ++g_prof_step;
 }
 
@@ -75,6 +77,15 @@ extern "C" int pqhsa_profile_enable(int32_t max_steps) {
     g_prof_steps = max_steps;
     g_prof_step = 0;
     g_prof_on = true;
+    g_prof_only = -1;
+    return PQHSA_OK;
+}
+
+extern "C" int pqhsa_profile_only(int32_t kernel) {
+    using namespace pqhsa;
+    PQHSA_REQUIRE(kernel >= -1 && kernel < kProfKernels, "profile_only: kernel=%d outside [-1, %d)", kernel,
+                  (int)kProfKernels);
+    g_prof_only = kernel;
     return PQHSA_OK;
 }
 
@@ -87,12 +98,14 @@ extern "C" int pqhsa_profile_collect(float *kernel_ms, int32_t *steps) {
     for (int k = 0; k < kProfKernels; ++k) kernel_ms[k] = 0.0f;
     for (int s = 0; s < n; ++s) {
         hipEvent_t *ev = &g_events[(size_t)s * (kProfKernels + 1)];
-        if (hipEventSynchronize(ev[kProfKernels]) != hipSuccess) {
+        const int last = g_prof_only < 0 ? kProfKernels : g_prof_only + 1;
+        if (hipEventSynchronize(ev[last]) != hipSuccess) {
             set_error("profile_collect: event synchronize failed");
             return PQHSA_ELAUNCH;
         }
         for (int k = 0; k < kProfKernels; ++k) {
             float ms = 0.0f;
+            if (g_prof_only >= 0 && k != g_prof_only) continue;
             if (hipEventElapsedTime(&ms, ev[k], ev[k + 1]) != hipSuccess) {
                 set_error("profile_collect: elapsed time failed");
                 return PQHSA_ELAUNCH;

@@ -23,7 +23,7 @@ void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 // Records the next profiling event on `stream` when profiling is enabled (no-op otherwise).
 void profile_mark(int slot, hipStream_t stream);
-enum { kProfLut = 0, kProfHist, kProfThresh, kProfEmit, kProfSelect, kProfAttend, kProfReduce, kProfKernels };
+enum { kProfLut = 0, kProfSample, kProfEmit, kProfSelect, kProfAttend, kProfReduce, kProfKernels };
 
 #define PQHSA_REQUIRE(cond, ...)            \
     do {                                    \
@@ -198,6 +198,66 @@ __device__ inline uint32_t wave_max_u32(uint32_t v) {
 __device__ inline int wave_sum_i32(int v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// ---- wave64 operations on the data-parallel-primitive path (no LDS traffic) --------------
+// Every lane of the wave must be active at the call.
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf>
+__device__ inline int dpp_move(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, BANK_MASK, true);
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lanes of each 8 reversed
+constexpr int kDppMirror = 0x140;      // lanes of each 16 reversed
+constexpr int kDppRowShr = 0x110;      // + n: lane i reads lane i-n of its row of 16 (0 when outside)
+constexpr int kDppBcast15 = 0x142;     // lane 15 of each row to the next row
+constexpr int kDppBcast31 = 0x143;     // lane 31 to rows 2 and 3
+constexpr int kDppWaveShl1 = 0x130;    // lane i reads lane i+1 of the wave (0 for the last lane)
+constexpr int kDppWaveShr1 = 0x138;    // lane i reads lane i-1 of the wave (0 for lane 0)
+
+// sum over the wave, returned in every lane (the order of the additions differs from wave_sum)
+__device__ inline float wave_total(float v) {
+    v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppXor2>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppHalfMirror>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppMirror>(__float_as_int(v)));
+    const int x = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(x, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(x, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(x, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(x, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+__device__ inline uint32_t wave_total_u32(uint32_t u) {
+    int v = (int)u;
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    v += dpp_move<kDppMirror>(v);
+    return (uint32_t)(__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) +
+                      __builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
+}
+// inclusive prefix sum over the lanes of the wave
+__device__ inline uint32_t wave_prefix_u32(uint32_t u) {
+    int v = (int)u;
+    v += dpp_move<kDppRowShr + 1>(v);
+    v += dpp_move<kDppRowShr + 2>(v);
+    v += dpp_move<kDppRowShr + 4>(v);
+    v += dpp_move<kDppRowShr + 8>(v);
+    v += dpp_move<kDppBcast15, 0xa>(v);
+    v += dpp_move<kDppBcast31, 0xc>(v);
+    return (uint32_t)v;
+}
+
+__device__ inline float wave_prefix_f32(float v) {
+    v += __int_as_float(dpp_move<kDppRowShr + 1>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppRowShr + 2>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppRowShr + 4>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppRowShr + 8>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppBcast15, 0xa>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppBcast31, 0xc>(__float_as_int(v)));
     return v;
 }
 

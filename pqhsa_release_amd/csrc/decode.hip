@@ -7,8 +7,8 @@ namespace pqhsa {
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps, float *qnorm,
                      float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, hipStream_t stream);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
-                       const float *list_scores, float scale, const pqhsa_select *select, uint32_t *hist,
-                       uint32_t *emit_count, uint32_t *thr_bin, int32_t *k_row, float *ref_val, float *ref_extra,
+                       const float *list_scores, float scale, const pqhsa_select *select,
+                       uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra,
                        void *pairs, uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans,
                        int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                        hipStream_t stream);
@@ -23,10 +23,10 @@ static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Carve {
     float *qnorm, *lut, *ls;
-    uint32_t *hist, *emit_count, *rescans;
+    uint32_t *emit_count, *rescans;
     float *mass;
     size_t zero_words;
-    uint32_t *thr_bin;
+    uint32_t *thr_key;
     int32_t *k_row;
     float *ref_val, *ref_extra, *mass_extra;
     void *pairs;
@@ -55,12 +55,11 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.lut = reinterpret_cast<float *>(take(rows * kM * kCodes * 4));
     c.ls = reinterpret_cast<float *>(take(rows * L * 4));
     const size_t z0 = off;  // everything from here to zero_words is cleared at the start of a step
-    c.hist = reinterpret_cast<uint32_t *>(take(rows * kHistBins * 4));
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
     c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
-    c.thr_bin = reinterpret_cast<uint32_t *>(take(rows * 4));
+    c.thr_key = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.k_row = reinterpret_cast<int32_t *>(take(rows * 4));
     c.ref_val = reinterpret_cast<float *>(take(rows * 4));
     c.ref_extra = reinterpret_cast<float *>(take(rows * 4));
@@ -125,10 +124,10 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     if (!topk_cnt) topk_cnt = c.topk_cnt;
 
     profile_mark(kProfLut, stream);
-    rc = launch_lut_build(q, q_dtype, index, G, eps, c.qnorm, c.lut, c.ls, c.hist, c.zero_words, stream);
+    rc = launch_lut_build(q, q_dtype, index, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words, stream);
     if (rc) return rc;
-    profile_mark(kProfHist, stream);
-    rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.hist, c.emit_count, c.thr_bin,
+    profile_mark(kProfSample, stream);
+    rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
                             c.k_row, c.ref_val, c.ref_extra, c.pairs, c.aux, c.mass, c.mass_extra, c.rescans,
                             c.tile_keys, topk_idx, topk_val, topk_cnt, stream);
     if (rc) return rc;

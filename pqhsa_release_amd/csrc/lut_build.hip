@@ -26,6 +26,20 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
 
+    // list blocks: their 64 x 128 centroid tile (2048 float4, 8 per thread) is requested before
+    // anything else, so the loads are all in flight while the query rows are normalised
+    const int l0 = ((int)blockIdx.x - 1) * kListsPerBlock;
+    const int nl = blockIdx.x == 0 ? 0 : min(kListsPerBlock, L - l0);
+    float4 tile[8];
+    if (blockIdx.x != 0) {
+        const float4 *c4 = reinterpret_cast<const float4 *>(coarse + ((size_t)bh * L + l0) * kD);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = tid + u * kLutThreads;
+            tile[u] = i < nl * (kD / 4) ? c4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    }
+
     // scratch that the later kernels of a decode step accumulate into starts at zero
     if (zero_words) {
         const size_t nthreads = (size_t)gridDim.x * gridDim.y * kLutThreads;
@@ -73,10 +87,12 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         return;
     }
 
-    const int l0 = (blockIdx.x - 1) * kListsPerBlock;
-    const float *cbase = coarse + ((size_t)bh * L + l0) * kD;
-    const int nl = min(kListsPerBlock, L - l0);
-    for (int i = tid; i < nl * kD; i += kLutThreads) cs[i / kD][i % kD] = cbase[i];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = tid + u * kLutThreads;
+        float *dst = &cs[i / (kD / 4)][(i % (kD / 4)) * 4];
+        dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
+    }
     __syncthreads();
     const int lane = tid % kListsPerBlock;
     const int wave = tid / kListsPerBlock;

@@ -1,21 +1,23 @@
-// Kernels 2 and 3: fused LUT scan and radix top-k.
+// Kernels 2 and 3: fused LUT scan and exact top-k.
 //
 // scan_kernel streams stored keys of one stream (4-bit packed codes, list ids, key norms) with
 // 128-bit loads, scores every key for all query rows of the GQA group from tables held in LDS,
 // and finishes in one of three ways:
 //   kWrite  store the logits (by retrieval-local index)
-//   kHist   histogram the top 11 bits of each logit's order-preserving key in LDS (used on the
-//           small sampled subset to estimate the selection threshold, and on logit matrices)
-//   kEmit   keep every key whose top bits reach the threshold bin as a (key, index, list)
-//           candidate, and sum exp(logit - reference) of all other keys per IVF list.  Stored
-//           keys are ordered by list, so the per-list sums are wave-level segment sums with one
-//           LDS update per (wave, list) instead of one per key.
-// thresh_sample_kernel turns the sample histogram into a threshold bin that keeps, with a wide
-// safety margin, more than k keys; select_final_kernel finds the exact k-th largest key among
-// the candidates by bisection on the 32-bit key (ties at the boundary go to the lowest index),
-// compacts the winners, and returns the losers' weights to their lists.  A row whose estimate
-// kept fewer than k candidates is re-scanned in full by its select workgroup, so the result is
-// always the exact top-k.
+//   kHist   histogram the top 11 bits of each logit's order-preserving key in LDS (logit
+//           matrices only: the first digit of the stand-alone radix top-k)
+//   kEmit   keep every key whose order-preserving key reaches the row's threshold as a
+//           (key, index, list) candidate, and sum exp(logit - reference) of all other keys per
+//           IVF list.  Candidate slots come from a wave prefix sum into wave-private staging
+//           (no atomics in the loop); stored keys are ordered by list, so the per-list sums are
+//           wave-level segment sums with one LDS update per (wave, list) instead of one per key.
+// sample_thresh_kernel scores a fixed random subset of the stored keys and takes, as the
+// threshold, the sampled key whose rank keeps, with a wide safety margin, more than k keys of the
+// full row; select_final_kernel finds the exact k-th largest key among the candidates by
+// bisection on the 32-bit key (ties at the boundary go to the lowest index), compacts the
+// winners, and returns the losers' weights to their lists.  A row whose estimate kept fewer than
+// k candidates is re-scanned in full by its select workgroup, so the result is always the exact
+// top-k.
 #include <cstdlib>
 
 #include "common.h"
@@ -23,6 +25,7 @@
 namespace pqhsa {
 
 constexpr int kScanThreads = 256;
+constexpr int kScanWaves = kScanThreads / kWave;
 constexpr int kKeysPerThread = 4;
 constexpr int kKeysPerIter = kScanThreads * kKeysPerThread;
 constexpr int kWaveKeys = kWave * kKeysPerThread;
@@ -57,14 +60,14 @@ struct ScanArgs {
     // kHist
     uint32_t *hist;  // [rows, 2048]
     // kEmit
-    const uint32_t *thr_bin;  // [rows]
+    const uint32_t *thr_key;  // [rows] keys at or above it are candidates
     const float *ref_val;     // [rows] reference logit of the background sums
     uint32_t *emit_count;     // [rows]
-    uint2 *emit_pairs;        // [rows, emit_cap] (key, retrieval-local index)
+    uint2 *emit_pairs;        // [rows, emit_cap] (key, stored position)
     uint16_t *emit_aux;       // [rows, emit_cap] list id of the candidate (NULL: none)
     int64_t emit_cap;
     float *mass;              // [BH, L, GP] accumulated with atomics (NULL: none)
-    int stage_cap;            // candidates staged in LDS per row before the global reservation
+    int stage_cap;            // candidates one wave stages in LDS per row before it writes straight to memory
 };
 
 template <int GP>
@@ -93,11 +96,21 @@ __device__ inline uint32_t wave_incl_scan_u32(uint32_t v) {
     return v;
 }
 
+// logit of one stored key for one query row, in the fixed summation order of the CPU oracle
+__device__ inline float score_one(const float *lut_col, const float *ls_col, uint32_t code, uint32_t lid, float qn,
+                                  float kn, float scale) {
+    float s = 0.0f;
+#pragma unroll
+    for (int m = 0; m < kM; ++m) s = s + lut_col[m * kCodes + ((code >> (4 * m)) & 15u)];
+    return (((s + ls_col[lid]) * qn) * kn) * scale;
+}
+
 template <int GP, int MODE, int SRC>
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
     const int bh = blockIdx.y;
     const int n = a.n_arr[bh / a.n_div];
     const int tile0 = blockIdx.x * a.tile_keys;
@@ -115,10 +128,11 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     float *mass_s = reinterpret_cast<float *>(after);                      // kEmit: [L][GP]
     const bool want_mass = MODE == kEmit && a.mass != nullptr;
     const size_t mass_bytes = want_mass ? (((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15) : 0;
-    uint32_t *cnt_s = reinterpret_cast<uint32_t *>(after + mass_bytes);    // [GP] (+pad)
-    uint32_t *base_s = cnt_s + 16;                                          // [GP]
-    uint2 *stage_s = reinterpret_cast<uint2 *>(cnt_s + 32);                 // [GP][stage_cap]
-    uint16_t *stage_aux = reinterpret_cast<uint16_t *>(stage_s + (size_t)GP * (MODE == kEmit ? a.stage_cap : 0));
+    uint32_t *wcnt_s = reinterpret_cast<uint32_t *>(after + mass_bytes);   // [waves][GP]
+    uint32_t *base_s = wcnt_s + kScanWaves * 16;                           // [waves][GP]
+    uint2 *stage_s = reinterpret_cast<uint2 *>(base_s + kScanWaves * 16);  // [waves][GP][stage_cap]
+    const int cap_w = MODE == kEmit ? a.stage_cap : 0;
+    uint16_t *stage_aux = reinterpret_cast<uint16_t *>(stage_s + (size_t)kScanWaves * GP * cap_w);
 
     float qn[GP];
     if constexpr (SRC == kIndex) {
@@ -137,16 +151,23 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     if constexpr (MODE == kHist) {
         for (int i = tid; i < GP * kHistBins; i += kScanThreads) hist_s[i] = 0u;
     }
-    uint32_t thr[GP];
-    float ref[GP];
+    // A key is a candidate when its logit, as a float, reaches the threshold: the same order as
+    // on the 32-bit keys (-0 and +0 compare equal, as their keys do).  Threshold key 0 keeps every
+    // key, key 0xffffffff (a NaN as a float) keeps none.
+    float thr_f[GP];
+    float nref2[GP];    // -reference * log2(e); -inf for padded rows so that their weights are 0
+    uint32_t wcnt[GP];  // candidates this wave has staged per row (wave-uniform)
+    constexpr float kLog2e = 1.4426950408889634f;
     if constexpr (MODE == kEmit) {
         if (want_mass)
             for (int i = tid; i < L * GP; i += kScanThreads) mass_s[i] = 0.0f;
-        if (tid < 32) cnt_s[tid] = 0u;
 #pragma unroll
         for (int g = 0; g < GP; ++g) {
-            thr[g] = a.thr_bin[(size_t)bh * GP + g];
-            ref[g] = a.ref_val[(size_t)bh * GP + g];
+            const uint32_t tk = a.thr_key[(size_t)bh * GP + g];
+            const float rv = a.ref_val[(size_t)bh * GP + g];
+            thr_f[g] = tk == 0u ? -3.402823466e38f : key_to_float(tk);
+            nref2[g] = g < a.G ? (__builtin_isfinite(rv) ? -rv * kLog2e : 0.0f) : -INFINITY;
+            wcnt[g] = 0u;
         }
     }
     __syncthreads();
@@ -232,86 +253,110 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
                 }
             }
         } else {
-            // ---- candidates: wave-aggregated slot reservation (two rows per packed scan) ------
-            uint32_t keyv[4][GP];
+            // ---- candidates and background weights ------------------------------------------
+            // Keys past the end of the tile score -inf: never candidates, weight 0.
+            const int wave_first = i0 - lane * kKeysPerThread;
+            if (wave_first + kWaveKeys > tile_end) {  // wave-uniform: only the last window of a row
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (i0 + j < tile_end) continue;
+#pragma unroll
+                    for (int g = 0; g < GP; ++g) s[j][g] = -INFINITY;
+                }
+            }
             uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
             float e[4][GP];
+            bool any = false;
 #pragma unroll
             for (int g = 0; g < GP; ++g) {
                 emit_mask[g] = 0u;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    keyv[j][g] = order_key(s[j][g]);
-                    const bool valid = (i0 + j < tile_end) && (g < a.G);
-                    const bool cand = valid && (keyv[j][g] >> (32 - kHistBits)) >= thr[g];
+                    const bool cand = s[j][g] >= thr_f[g];
                     if (cand) emit_mask[g] |= 1u << j;
-                    e[j][g] = (valid && !cand && want_mass) ? __expf(s[j][g] - ref[g]) : 0.0f;
+                    if (want_mass) e[j][g] = cand ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
                 }
+                any |= emit_mask[g] != 0u;
             }
-            int32_t idxv[4] = {0, 0, 0, 0};
-            bool any = false;
+            if (__ballot(any) != 0ull) {  // wave-uniform
 #pragma unroll
-            for (int g = 0; g < GP; ++g) any |= emit_mask[g] != 0u;
-            if (any) {
+                for (int g2 = 0; g2 < GP; g2 += 2) {
+                    uint32_t packed = __popc(emit_mask[g2]);
+                    if constexpr (GP > 1) packed |= (uint32_t)__popc(emit_mask[g2 + 1 < GP ? g2 + 1 : g2]) << 16;
+                    const uint32_t incl = wave_prefix_u32(packed);
+                    const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+                    if (total == 0u) continue;
+                    const uint32_t excl = incl - packed;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) idxv[j] = a.pos ? a.pos[base + min(i0 + j, tile_end - 1)] : i0 + j;
-            }
-#pragma unroll
-            for (int g2 = 0; g2 < GP; g2 += 2) {
-                uint32_t packed = __popc(emit_mask[g2]);
-                if (g2 + 1 < GP) packed |= (uint32_t)__popc(emit_mask[g2 + 1 < GP ? g2 + 1 : g2]) << 16;
-                if (__ballot(packed != 0u) == 0ull) continue;  // wave-uniform
-                const uint32_t incl = wave_incl_scan_u32(packed);
-                const uint32_t total = (uint32_t)__shfl((int)incl, kWave - 1, kWave);
-                uint32_t bases = 0u;
-                if (lane == kWave - 1) {
-                    const uint32_t t0 = total & 0xffffu, t1 = total >> 16;
-                    const uint32_t b0 = t0 ? atomicAdd(&cnt_s[g2], t0) : 0u;
-                    const uint32_t b1 = (g2 + 1 < GP && t1) ? atomicAdd(&cnt_s[g2 + 1 < GP ? g2 + 1 : g2], t1) : 0u;
-                    bases = (b0 & 0xffffu) | (b1 << 16);  // tiles hold at most 16384 keys
-                }
-                bases = (uint32_t)__shfl((int)bases, kWave - 1, kWave);
-                const uint32_t excl = incl - packed;
-#pragma unroll
-                for (int gg = 0; gg < 2; ++gg) {
-                    const int g = g2 + gg;
-                    if (g < GP) {
-                        uint32_t slot = ((bases >> (16 * gg)) & 0xffffu) + ((excl >> (16 * gg)) & 0xffffu);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            if (!((emit_mask[g] >> j) & 1u)) continue;
-                            const uint2 pr = make_uint2(keyv[j][g], (uint32_t)idxv[j]);
-                            if (slot < (uint32_t)a.stage_cap) {
-                                stage_s[(size_t)g * a.stage_cap + slot] = pr;
-                                if (a.emit_aux) stage_aux[(size_t)g * a.stage_cap + slot] = (uint16_t)lid[j];
-                            } else {  // staging full: reserve one global slot directly
-                                const uint32_t p = atomicAdd(&a.emit_count[(size_t)bh * GP + g], 1u);
-                                a.emit_pairs[((size_t)bh * GP + g) * a.emit_cap + p] = pr;
-                                if (a.emit_aux) a.emit_aux[((size_t)bh * GP + g) * a.emit_cap + p] = (uint16_t)lid[j];
+                    for (int gg = 0; gg < 2; ++gg) {
+                        const int g = g2 + gg;
+                        if (g < GP) {
+                            const uint32_t tot = (total >> (16 * gg)) & 0xffffu;
+                            if (tot == 0u) continue;  // wave-uniform
+                            const size_t srow = ((size_t)wave * GP + g) * cap_w;
+                            if (wcnt[g] != 0u && wcnt[g] + tot > (uint32_t)cap_w) {
+                                // staging area full: the wave moves it to memory (wave-uniform branch)
+                                const uint32_t c = min(wcnt[g], (uint32_t)cap_w);
+                                uint32_t at = 0u;
+                                if (lane == 0) at = atomicAdd(&a.emit_count[(size_t)bh * GP + g], c);
+                                at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+                                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                                __builtin_amdgcn_wave_barrier();
+                                const size_t o = ((size_t)bh * GP + g) * a.emit_cap + at;
+                                for (uint32_t i = lane; i < c; i += kWave) {
+                                    a.emit_pairs[o + i] = stage_s[srow + i];
+                                    if (a.emit_aux) a.emit_aux[o + i] = stage_aux[srow + i];
+                                }
+                                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                                __builtin_amdgcn_wave_barrier();
+                                wcnt[g] = 0u;
                             }
-                            ++slot;
+                            uint32_t slot = wcnt[g] + ((excl >> (16 * gg)) & 0xffffu);
+                            wcnt[g] += tot;
+                            if (emit_mask[g] == 0u) continue;
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                if (!((emit_mask[g] >> j) & 1u)) continue;
+                                const uint2 pr = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
+                                if (slot < (uint32_t)cap_w) {
+                                    stage_s[srow + slot] = pr;
+                                    if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
+                                } else {  // staging full: reserve one slot in memory directly
+                                    const uint32_t p = atomicAdd(&a.emit_count[(size_t)bh * GP + g], 1u);
+                                    a.emit_pairs[((size_t)bh * GP + g) * a.emit_cap + p] = pr;
+                                    if (a.emit_aux) a.emit_aux[((size_t)bh * GP + g) * a.emit_cap + p] = (uint16_t)lid[j];
+                                }
+                                ++slot;
+                            }
                         }
                     }
                 }
             }
-            // ---- background: exp(logit - ref) of every other key, summed per list ------------
+            // ---- background: weights summed per list -------------------------------------------
+            // Stored keys are ordered by list, so the lanes of a wave form a few runs of equal
+            // list id.  One prefix sum over the lanes gives every run's total as a difference of
+            // two prefix values: the last lane of a run adds its prefix, the first lane takes
+            // back the prefix of the lane before it.  (Unordered keys only make more runs.)
             if (want_mass) {
-                const int wave_first = i0 - lane * kKeysPerThread;
-                const bool sorted_window = wave_first + kWaveKeys <= min(nsorted, tile_end);
-                const int first = __shfl((int)lid[0], 0, kWave);
-                const int last = __shfl((int)lid[3], kWave - 1, kWave);
-                if (sorted_window && last - first <= 8) {
-                    for (int t = first; t <= last; ++t) {
+                const bool simple = lid[0] == lid[3] && lid[0] == lid[1] && lid[0] == lid[2];
+                const int prev = dpp_move<kDppWaveShr1>((int)lid[0]);
+                const int next = dpp_move<kDppWaveShl1>((int)lid[0]);
+                const bool is_start = lane == 0 || prev != (int)lid[0];
+                const bool is_end = lane == kWave - 1 || next != (int)lid[0];
+                float v[GP], pre[GP];
 #pragma unroll
-                        for (int g = 0; g < GP; ++g) {
-                            float v = 0.0f;
+                for (int g = 0; g < GP; ++g) {
+                    v[g] = simple ? (e[0][g] + e[1][g]) + (e[2][g] + e[3][g]) : 0.0f;
+                    pre[g] = wave_prefix_f32(v[g]);
+                }
+                if (is_start || is_end) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) v += (lid[j] == (uint32_t)t) ? e[j][g] : 0.0f;
-                            v = wave_sum(v);
-                            if (lane == 0 && v != 0.0f) atomicAdd(&mass_s[t * GP + g], v);
-                        }
+                    for (int g = 0; g < GP; ++g) {
+                        const float add = is_start ? (is_end ? v[g] : v[g] - pre[g]) : pre[g];
+                        if (add != 0.0f) atomicAdd(&mass_s[lid[0] * GP + g], add);
                     }
-                } else {
+                }
+                if (!simple) {  // a lane whose four keys straddle lists adds them one by one
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -331,20 +376,32 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             if (v) atomicAdd(&dst[i], v);
         }
     } else if constexpr (MODE == kEmit) {
+        // one reservation per (workgroup, row); every wave then copies its own staging area out
+        if (lane == 0) {
+#pragma unroll
+            for (int g = 0; g < GP; ++g) wcnt_s[wave * GP + g] = min(wcnt[g], (uint32_t)cap_w);
+        }
         __syncthreads();
         if (tid < GP) {
-            const uint32_t c = min(cnt_s[tid], (uint32_t)a.stage_cap);
-            base_s[tid] = c ? atomicAdd(&a.emit_count[(size_t)bh * GP + tid], c) : 0u;
-            cnt_s[tid] = c;
+            uint32_t total = 0;
+#pragma unroll
+            for (int w = 0; w < kScanWaves; ++w) total += wcnt_s[w * GP + tid];
+            uint32_t at = total ? atomicAdd(&a.emit_count[(size_t)bh * GP + tid], total) : 0u;
+#pragma unroll
+            for (int w = 0; w < kScanWaves; ++w) {
+                base_s[w * GP + tid] = at;
+                at += wcnt_s[w * GP + tid];
+            }
         }
         __syncthreads();
 #pragma unroll
         for (int g = 0; g < GP; ++g) {
-            const uint32_t c = cnt_s[g];
-            const size_t o = ((size_t)bh * GP + g) * a.emit_cap + base_s[g];
-            for (uint32_t i = tid; i < c; i += kScanThreads) {
-                a.emit_pairs[o + i] = stage_s[(size_t)g * a.stage_cap + i];
-                if (a.emit_aux) a.emit_aux[o + i] = stage_aux[(size_t)g * a.stage_cap + i];
+            const uint32_t c = min(wcnt[g], (uint32_t)cap_w);
+            const size_t o = ((size_t)bh * GP + g) * a.emit_cap + base_s[wave * GP + g];
+            const size_t srow = ((size_t)wave * GP + g) * cap_w;
+            for (uint32_t i = lane; i < c; i += kWave) {
+                a.emit_pairs[o + i] = stage_s[srow + i];
+                if (a.emit_aux) a.emit_aux[o + i] = stage_aux[srow + i];
             }
         }
         if (want_mass) {
@@ -383,14 +440,11 @@ __device__ inline void find_from_top(const uint32_t *hist, int nbins, uint32_t w
     }
 }
 
-// smallest float whose order key falls in histogram bin `bin`
-__device__ inline float bin_floor(uint32_t bin) { return key_to_float(bin << (32 - kHistBits)); }
-
 // One wave per row: exact first-digit threshold from a full histogram (logit-matrix top-k).
 __global__ __launch_bounds__(kWave) void thresh_kernel(const uint32_t *__restrict__ hist,
                                                        const int32_t *__restrict__ n_arr,
                                                        const int32_t *__restrict__ k_arr,
-                                                       uint32_t *__restrict__ thr_bin, int32_t *__restrict__ k_row,
+                                                       uint32_t *__restrict__ thr_key, int32_t *__restrict__ k_row,
                                                        float *__restrict__ ref_val) {
     __shared__ uint32_t res[2];
     const int row = blockIdx.x;
@@ -405,56 +459,191 @@ __global__ __launch_bounds__(kWave) void thresh_kernel(const uint32_t *__restric
     find_from_top(hist + (size_t)row * kHistBins, kHistBins, (uint32_t)k, &res[0], &res[1]);
     __syncthreads();
     if (lane == 0) {
-        thr_bin[row] = res[0];
+        thr_key[row] = res[0] >= (uint32_t)kHistBins ? 0xffffffffu : res[0] << (32 - kHistBits);
         k_row[row] = k;
         ref_val[row] = 0.0f;
     }
 }
 
-// One wave per row: threshold estimate from the histogram of the sampled keys.  With ns
-// sampled keys out of n, keeping every key down to the c-th largest sampled logit keeps about
-// c * n / ns keys with a relative spread of 1/sqrt(c); c is chosen so that this stays above k
-// by 7 standard deviations.  The reference value of the background sums is the lower edge of
-// the threshold bin, so every summed weight is at most 1.
-__global__ __launch_bounds__(kWave) void thresh_sample_kernel(const uint32_t *__restrict__ hist,
-                                                              const int32_t *__restrict__ n_arr,
-                                                              const int32_t *__restrict__ ns_arr, int rows_per_n,
-                                                              int GP, int G, double fraction, int topk,
-                                                              uint32_t *__restrict__ thr_bin,
-                                                              int32_t *__restrict__ k_row,
-                                                              float *__restrict__ ref_val) {
-    __shared__ uint32_t res[2];
-    const int row = blockIdx.x;
-    const int lane = threadIdx.x;
-    const int n = n_arr[row / rows_per_n];
-    const int ns = ns_arr[row / rows_per_n];
-    int k = resolve_k(n, fraction, topk);
-    if ((row % GP) >= G) k = 0;
+// ---- block-wide helpers of the selection kernels (1024 threads, all active) -----------------
+constexpr int kSelThreads = 1024;
+constexpr int kSelWaves = kSelThreads / kWave;
+
+// Sum over the workgroup of a per-wave (wave-uniform) count, with one barrier: `red` holds two
+// alternating sets of per-wave partials, so consecutive calls (step, step + 1, ...) do not
+// overwrite sums that slower waves are still reading.
+__device__ inline uint32_t block_total_of_waves(uint32_t wave_count, uint32_t (*red)[kSelWaves], int step) {
+    uint32_t *r = red[step & 1];
+    if ((threadIdx.x & (kWave - 1)) == 0) r[threadIdx.x / kWave] = wave_count;
+    __syncthreads();
+    uint32_t t = 0;
+#pragma unroll
+    for (int w = 0; w < kSelWaves / 4; ++w) {
+        const uint4 q = reinterpret_cast<const uint4 *>(r)[w];
+        t += (q.x + q.y) + (q.z + q.w);
+    }
+    return t;
+}
+
+__device__ inline uint32_t wave_count_if(bool pred) { return (uint32_t)__popcll(__ballot(pred)); }
+
+// Keys held in registers, R per thread.  Returns the largest T with count(key >= T) >= want (the
+// want-th largest key); padding keys are 0 and never counted (T >= 1).  Stops early, with
+// `exact` set, at a prefix T whose count is exactly want: then {key >= T} is the answer set.
+template <int R>
+__device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, uint32_t (*red)[kSelWaves],
+                                       int &step, bool &exact) {
+    uint32_t t = 0u;
+    exact = false;
+    for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t trial = t | (1u << bit);
+        uint32_t c = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) c += wave_count_if(key[r] >= trial);
+        c = block_total_of_waves(c, red, step++);
+        if (c >= want) t = trial;
+        if (c == want) {
+            exact = true;
+            break;
+        }
+    }
+    return t;
+}
+
+// The same search over keys in memory (any count).
+template <typename KeyAt>
+__device__ inline uint32_t bisect_mem(KeyAt key_at, uint32_t cnt, uint32_t want, uint32_t (*red)[kSelWaves],
+                                      int &step, bool &exact) {
+    uint32_t t = 0u;
+    exact = false;
+    const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
+    for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t trial = t | (1u << bit);
+        uint32_t c = 0;
+#pragma unroll 8
+        for (uint32_t r = 0; r < rounds; ++r) {
+            const uint32_t p = r * kSelThreads + threadIdx.x;
+            c += wave_count_if(p < cnt && key_at(p) >= trial);
+        }
+        c = block_total_of_waves(c, red, step++);
+        if (c >= want) t = trial;
+        if (c == want) {
+            exact = true;
+            break;
+        }
+    }
+    return t;
+}
+
+// ---- threshold estimate from the sampled keys ---------------------------------------------------
+// One workgroup per (query row, stream).  With ns sampled keys out of n, keeping every key down
+// to the c-th largest sampled logit keeps about c * n / ns keys with a relative spread of
+// 1/sqrt(c); c is chosen so that this stays above k by 7 standard deviations.  The reference
+// value of the background sums is the threshold itself, so every summed weight is below 1.
+struct SampleArgs {
+    const uint32_t *codes;     // [BH, s_cap]
+    const uint16_t *list_ids;
+    const float *norms;
+    int64_t s_cap;
+    const int32_t *n_arr;      // [B] stored keys
+    const int32_t *ns_arr;     // [B] sampled keys
+    int n_div;
+    const float *qnorm, *lut, *list_scores;
+    float scale;
+    int L, GP, G;
+    double fraction;
+    int topk;
+    uint32_t *thr_key;         // [BH * GP]
+    int32_t *k_row;
+    float *ref_val;
+};
+
+constexpr int kSampleRegsMax = 32;  // sampled keys per thread: at most 32768 per row
+
+template <int R>
+__device__ inline uint32_t sample_kth(const SampleArgs &a, int bh, int ns, const float *lut_s, const float *ls_s,
+                                      float qn, uint32_t want, uint32_t (*red)[kSelWaves]) {
+    const size_t base = (size_t)bh * a.s_cap;
+    uint32_t key[R];
+    constexpr int kBatch = R < 8 ? R : 8;  // loads of one batch are all in flight before their first use
+#pragma unroll
+    for (int r0 = 0; r0 < R; r0 += kBatch) {
+        uint32_t code[kBatch], lid[kBatch];
+        float kn[kBatch];
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int p = (r0 + r) * kSelThreads + (int)threadIdx.x;
+            const bool ok = p < ns;
+            code[r] = ok ? a.codes[base + p] : 0u;
+            lid[r] = ok ? a.list_ids[base + p] : 0u;
+            kn[r] = ok ? a.norms[base + p] : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int p = (r0 + r) * kSelThreads + (int)threadIdx.x;
+            if (lid[r] >= (uint32_t)a.L) lid[r] = 0u;
+            key[r0 + r] = p < ns ? order_key(score_one(lut_s, ls_s, code[r], lid[r], qn, kn[r], a.scale)) : 0u;
+        }
+    }
+    int step = 0;
+    bool exact;
+    return bisect_regs<R>(key, want, red, step, exact);
+}
+
+__global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ __align__(16) uint32_t red[2][kSelWaves];
+    const int tid = threadIdx.x;
+    const int g = blockIdx.x;
+    const int bh = blockIdx.y;
+    const size_t row = (size_t)bh * a.GP + g;
+    const int n = a.n_arr[bh / a.n_div];
+    const int ns = a.ns_arr[bh / a.n_div];
+    int k = resolve_k(n, a.fraction, a.topk);
+    if (g >= a.G) {
+        if (tid == 0) {
+            a.thr_key[row] = 0xffffffffu;
+            a.k_row[row] = 0;
+            a.ref_val[row] = -INFINITY;
+        }
+        return;
+    }
     // expected sampled keys among the top max(k, 1), plus the margin
     const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
     const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
-    const uint32_t want = (uint32_t)min((double)ns, ceil(x * x) + 1.0);
-    if (lane == 0) {
-        res[0] = 0u;  // sample too small to say anything: every key is a candidate
-        res[1] = 0u;
+    const double want_d = ceil(x * x) + 1.0;
+    if (ns <= 0 || want_d >= (double)ns) {
+        // sample too small to say anything: every key is a candidate and no background sum is formed
+        if (tid == 0) {
+            a.thr_key[row] = 0u;
+            a.k_row[row] = k;
+            a.ref_val[row] = -INFINITY;
+        }
+        return;
     }
+    const uint32_t want = (uint32_t)want_d;
+
+    float *lut_s = reinterpret_cast<float *>(smem);   // [128]
+    float *ls_s = lut_s + kM * kCodes;                // [L]
+    for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
+    for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
+    const float qn = a.qnorm[row];
     __syncthreads();
-    if (want < (uint32_t)ns) find_from_top(hist + (size_t)row * kHistBins, kHistBins, want, &res[0], &res[1]);
-    __syncthreads();
-    if (lane == 0) {
-        const uint32_t bin = (row % GP) >= G ? (uint32_t)kHistBins : res[0];
-        thr_bin[row] = bin;
-        k_row[row] = k;
-        // bin 0 keeps every key: no background sum is formed and its reference is never used
-        ref_val[row] = bin == 0u ? -INFINITY : bin_floor(min(bin, (uint32_t)kHistBins - 1));
+    uint32_t t;
+    if (ns <= 4 * kSelThreads) t = sample_kth<4>(a, bh, ns, lut_s, ls_s, qn, want, red);
+    else if (ns <= 8 * kSelThreads) t = sample_kth<8>(a, bh, ns, lut_s, ls_s, qn, want, red);
+    else if (ns <= 16 * kSelThreads) t = sample_kth<16>(a, bh, ns, lut_s, ls_s, qn, want, red);
+    else t = sample_kth<kSampleRegsMax>(a, bh, ns, lut_s, ls_s, qn, want, red);
+    if (tid == 0) {
+        a.thr_key[row] = t;
+        a.k_row[row] = k;
+        a.ref_val[row] = t == 0u ? -INFINITY : key_to_float(t);
     }
 }
 
 // ---- exact selection among the candidates -----------------------------------------------
-constexpr int kSelThreads = 256;
-
 struct SelectArgs {
-    uint2 *pairs;          // [rows, emit_cap] (key, index)
+    uint2 *pairs;          // [rows, emit_cap] (key, stored position)
     uint16_t *aux;         // [rows, emit_cap] list ids (NULL: none)
     int64_t emit_cap;
     uint32_t *emit_count;  // [rows]
@@ -466,17 +655,16 @@ struct SelectArgs {
     float *topk_val;
     int32_t *topk_cnt;
     int64_t k_cap;
-    int key_cap;           // candidate keys that fit in dynamic LDS
     // background mass of the candidates that lose the selection (optional)
     float *mass;           // [BH, L, GP]: zeroed for a row that is re-scanned in full
     float *mass_extra;     // [BH, L, GP]
     float *ref_extra;      // [rows] reference logit of mass_extra
     int L;
-    // what a full re-scan of one row needs
+    // the index: retrieval-local index of every stored position, and what a full re-scan needs
+    const int32_t *pos;    // [BH, n_cap] (NULL: a candidate's position is its index)
     const uint32_t *codes;
     const uint16_t *list_ids;
     const float *norms;
-    const int32_t *pos;
     int64_t n_cap;
     const float *qnorm;
     const float *lut;
@@ -485,23 +673,200 @@ struct SelectArgs {
     uint32_t *rescans;     // [1] counter of rows that needed the full re-scan (diagnostics)
 };
 
-__device__ inline uint32_t block_sum_u32(uint32_t v, uint32_t *scratch) {
-    v = (uint32_t)wave_sum_i32((int)v);
+// Exclusive prefix over the workgroup of a per-thread count (one barrier pair).
+__device__ inline uint32_t block_exclusive_u32(uint32_t mine, uint32_t *wsum /*[kSelWaves]*/) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint32_t incl = wave_prefix_u32(mine);
     __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    if (lane == kWave - 1) wsum[wave] = incl;
     __syncthreads();
-    uint32_t s = 0;
+    uint32_t before = 0;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    return before + incl - mine;
+}
+
+// What every variant of the selection ends with: winners to the output, losers' weights per list.
+struct SelectOut {
+    int32_t *out_idx;
+    float *out_val;
+    uint32_t k_cap;
+    const int32_t *pos_row;  // NULL: identity
+    float *mx;               // LDS [L] (NULL: no background)
+    float ref1;
+    __device__ inline void winner(uint32_t at, uint32_t key, uint32_t where) const {
+        if (at < k_cap) {
+            out_idx[at] = pos_row ? pos_row[where] : (int32_t)where;
+            if (out_val) out_val[at] = key_to_float(key);
+        }
+    }
+    __device__ inline void loser(uint32_t key, uint32_t list) const {
+        if (mx) atomicAdd(&mx[list], __expf(key_to_float(key) - ref1));
+    }
+};
+
+// Candidates in registers (cnt <= R * 1024).
+template <int R>
+__device__ inline void select_regs(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
+                                   const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                   uint32_t *wsum, float *ref1_out) {
+    const int tid = threadIdx.x;
+    uint32_t key[R], where[R], list[R];
 #pragma unroll
-    for (int w = 0; w < kSelThreads / kWave; ++w) s += scratch[w];
-    return s;
+    for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
+        const uint32_t p = (uint32_t)r * kSelThreads + tid;
+        const uint2 pr = p < cnt ? pairs[p] : make_uint2(0u, 0u);
+        key[r] = pr.x;
+        where[r] = pr.y;
+        list[r] = (aux && p < cnt) ? aux[p] : 0u;
+    }
+    int step = 0;
+    bool exact = false;
+    uint32_t tkey = 0u;
+    if (k > 0) {
+        tkey = bisect_regs<R>(key, (uint32_t)k, red, step, exact);
+    } else {  // nothing is selected: the reference of the losers' weights is the largest key
+        uint32_t kmax = 0u;
+#pragma unroll
+        for (int r = 0; r < R; ++r) kmax = max(kmax, key[r]);
+        kmax = wave_max_u32(kmax);
+        __syncthreads();
+        if ((tid & (kWave - 1)) == 0) wsum[tid / kWave] = kmax;
+        __syncthreads();
+        for (int w = 0; w < kSelWaves; ++w) tkey = max(tkey, wsum[w]);
+    }
+    // ties at the boundary (only when the search ran to the last bit): keep the lowest indices
+    uint32_t idx_thr = 0xffffffffu;
+    bool ties = false;
+    if (k > 0 && !exact) {
+        uint32_t c_gt = 0, c_eq = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            c_gt += wave_count_if(key[r] > tkey);
+            c_eq += wave_count_if(key[r] == tkey);
+        }
+        c_gt = block_total_of_waves(c_gt, red, step++);
+        c_eq = block_total_of_waves(c_eq, red, step++);
+        const uint32_t want_ties = (uint32_t)k - c_gt;
+        if (c_eq > want_ties) {
+            // largest I with count(key == T && index < I) < want_ties: the want_ties-th lowest tie index
+            ties = true;
+            uint32_t tidx[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                tidx[r] = key[r] == tkey ? (pos_row ? (uint32_t)pos_row[where[r]] : where[r]) : 0xffffffffu;
+            uint32_t lo = 0u;
+            for (int bit = 31; bit >= 0; --bit) {
+                const uint32_t trial = lo | (1u << bit);
+                uint32_t c = 0;
+#pragma unroll
+                for (int r = 0; r < R; ++r) c += wave_count_if(tidx[r] < trial);
+                c = block_total_of_waves(c, red, step++);
+                if (c < want_ties) lo = trial;
+            }
+            idx_thr = lo;
+#pragma unroll
+            for (int r = 0; r < R; ++r)  // fold the tie rule into the keys: losers of the tie drop below T
+                if (key[r] == tkey && tidx[r] > idx_thr) key[r] = tkey - 1u, where[r] |= 0x80000000u;
+        }
+    }
+    out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
+    *ref1_out = out.ref1;
+    uint32_t mine = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) mine += (k > 0 && key[r] >= tkey) ? 1u : 0u;
+    uint32_t at = block_exclusive_u32(mine, wsum);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t p = (uint32_t)r * kSelThreads + tid;
+        if (p >= cnt) continue;
+        if (k > 0 && key[r] >= tkey) {
+            out.winner(at++, key[r], where[r]);
+        } else {
+            const bool tie_loser = ties && (where[r] & 0x80000000u);
+            out.loser(tie_loser ? tkey : key[r], list[r]);
+        }
+    }
+}
+
+// Candidates in memory (any count): the same selection, streaming the pairs on every pass.
+__device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
+                                  const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                  uint32_t *wsum, float *ref1_out) {
+    const int tid = threadIdx.x;
+    const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
+    auto key_at = [=](uint32_t p) { return pairs[p].x; };
+    auto index_of = [=](uint32_t where) { return pos_row ? (uint32_t)pos_row[where] : where; };
+    int step = 0;
+    bool exact = false;
+    uint32_t tkey = 0u;
+    if (k > 0) {
+        tkey = bisect_mem(key_at, cnt, (uint32_t)k, red, step, exact);
+    } else {
+        uint32_t kmax = 0u;
+        for (uint32_t p = tid; p < cnt; p += kSelThreads) kmax = max(kmax, key_at(p));
+        kmax = wave_max_u32(kmax);
+        __syncthreads();
+        if ((tid & (kWave - 1)) == 0) wsum[tid / kWave] = kmax;
+        __syncthreads();
+        for (int w = 0; w < kSelWaves; ++w) tkey = max(tkey, wsum[w]);
+    }
+    uint32_t idx_thr = 0xffffffffu;
+    if (k > 0 && !exact) {
+        uint32_t c_gt = 0, c_eq = 0;
+#pragma unroll 4
+        for (uint32_t r = 0; r < rounds; ++r) {
+            const uint32_t p = r * kSelThreads + tid;
+            const uint32_t kk = p < cnt ? key_at(p) : 0u;
+            c_gt += wave_count_if(p < cnt && kk > tkey);
+            c_eq += wave_count_if(p < cnt && kk == tkey);
+        }
+        c_gt = block_total_of_waves(c_gt, red, step++);
+        c_eq = block_total_of_waves(c_eq, red, step++);
+        const uint32_t want_ties = (uint32_t)k - c_gt;
+        if (c_eq > want_ties) {
+            uint32_t lo = 0u;
+            for (int bit = 31; bit >= 0; --bit) {
+                const uint32_t trial = lo | (1u << bit);
+                uint32_t c = 0;
+                for (uint32_t r = 0; r < rounds; ++r) {
+                    const uint32_t p = r * kSelThreads + tid;
+                    bool hit = false;
+                    if (p < cnt) {
+                        const uint2 pr = pairs[p];
+                        hit = pr.x == tkey && index_of(pr.y) < trial;
+                    }
+                    c += wave_count_if(hit);
+                }
+                c = block_total_of_waves(c, red, step++);
+                if (c < want_ties) lo = trial;
+            }
+            idx_thr = lo;
+        }
+    }
+    auto selected = [=](uint2 pr) {
+        if (k <= 0) return false;
+        if (pr.x != tkey || idx_thr == 0xffffffffu) return pr.x >= tkey;
+        return index_of(pr.y) <= idx_thr;
+    };
+    out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
+    *ref1_out = out.ref1;
+    uint32_t mine = 0;
+#pragma unroll 4
+    for (uint32_t p = tid; p < cnt; p += kSelThreads) mine += selected(pairs[p]) ? 1u : 0u;
+    uint32_t at = block_exclusive_u32(mine, wsum);
+#pragma unroll 4
+    for (uint32_t p = tid; p < cnt; p += kSelThreads) {
+        const uint2 pr = pairs[p];
+        if (selected(pr)) out.winner(at++, pr.x, pr.y);
+        else out.loser(pr.x, aux ? aux[p] : 0u);
+    }
 }
 
 __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ uint32_t scratch[kSelThreads / kWave];
-    __shared__ uint32_t scan_s[kSelThreads];
-    uint32_t *keys_s = reinterpret_cast<uint32_t *>(smem);          // [key_cap]
-    float *mx = reinterpret_cast<float *>(keys_s + a.key_cap);      // [L]
+    __shared__ __align__(16) uint32_t red[2][kSelWaves];
+    __shared__ uint32_t wsum[kSelWaves];
+    float *mx = reinterpret_cast<float *>(smem);  // [L] (the re-scan parks its [128 + L] tables here first)
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
     const int bh = blockIdx.y;
@@ -511,6 +876,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     const int k = a.k_row[row];
     uint2 *pairs = a.pairs + row * a.emit_cap;
     uint16_t *aux = a.aux ? a.aux + row * a.emit_cap : nullptr;
+    const int32_t *pos_row = a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr;
     uint32_t cnt = a.emit_count[row];
     float *mass_out = a.mass_extra ? a.mass_extra + (size_t)bh * a.L * a.GP + g : nullptr;
 
@@ -518,7 +884,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
         // The estimate kept too few keys: score the whole row again and treat every key as a
         // candidate.  The row's background sums start over (all of them land in mass_extra).
         if (tid == 0 && a.rescans) atomicAdd(a.rescans, 1u);
-        float *lut_s = reinterpret_cast<float *>(smem);  // [128] then [L]; the key area is not in use yet
+        float *lut_s = reinterpret_cast<float *>(smem);
         float *ls_s = lut_s + kM * kCodes;
         for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
         for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
@@ -527,15 +893,12 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
         const float qn = a.qnorm[row];
         __syncthreads();
         const size_t base = (size_t)bh * a.n_cap;
+#pragma unroll 4
         for (int p = tid; p < n; p += kSelThreads) {
-            const uint32_t w = a.codes[base + p];
             uint32_t lid = a.list_ids[base + p];
             if (lid >= (uint32_t)a.L) lid = 0u;
-            float s = 0.0f;
-#pragma unroll
-            for (int m = 0; m < kM; ++m) s = s + lut_s[m * kCodes + ((w >> (4 * m)) & 15u)];
-            s = (((s + ls_s[lid]) * qn) * a.norms[base + p]) * a.scale;
-            pairs[p] = make_uint2(order_key(s), (uint32_t)(a.pos ? a.pos[base + p] : p));
+            const float s = score_one(lut_s, ls_s, a.codes[base + p], lid, qn, a.norms[base + p], a.scale);
+            pairs[p] = make_uint2(order_key(s), (uint32_t)p);
             if (aux) aux[p] = (uint16_t)lid;
         }
         cnt = (uint32_t)n;
@@ -543,94 +906,21 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
         __syncthreads();
     }
 
-    // candidate keys into LDS (when they fit) for the bisection
-    const bool in_lds = cnt <= (uint32_t)a.key_cap;
-    if (in_lds)
-        for (uint32_t p = tid; p < cnt; p += kSelThreads) keys_s[p] = pairs[p].x;
-    __syncthreads();
-    auto key_at = [&](uint32_t p) { return in_lds ? keys_s[p] : pairs[p].x; };
-
-    // largest T with count(key >= T) >= k, one bit at a time: T is the k-th largest key
-    uint32_t tkey = 0u;
-    uint32_t kmax = 0u;
-    if (k > 0) {
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t trial = tkey | (1u << bit);
-            uint32_t c = 0;
-            for (uint32_t p = tid; p < cnt; p += kSelThreads) c += key_at(p) >= trial ? 1u : 0u;
-            c = block_sum_u32(c, scratch);
-            if (c >= (uint32_t)k) tkey = trial;
-        }
-    } else {
-        for (uint32_t p = tid; p < cnt; p += kSelThreads) kmax = max(kmax, key_at(p));
-        kmax = wave_max_u32(kmax);
-        __syncthreads();
-        if ((tid & (kWave - 1)) == 0) scratch[tid / kWave] = kmax;
-        __syncthreads();
-        kmax = max(max(scratch[0], scratch[1]), max(scratch[2], scratch[3]));
-    }
-    // ties at the boundary: keep the lowest indices
-    uint32_t c_gt = 0, c_eq = 0;
-    for (uint32_t p = tid; p < cnt; p += kSelThreads) {
-        const uint32_t kk = key_at(p);
-        c_gt += kk > tkey ? 1u : 0u;
-        c_eq += kk == tkey ? 1u : 0u;
-    }
-    c_gt = block_sum_u32(c_gt, scratch);
-    c_eq = block_sum_u32(c_eq, scratch);
-    const uint32_t want_ties = k > 0 ? (uint32_t)k - c_gt : 0u;
-    uint32_t idx_thr = 0xffffffffu;
-    if (k > 0 && c_eq > want_ties) {
-        // largest I with count(key == T && index < I) < want_ties: the want_ties-th lowest tie index
-        uint32_t lo = 0u;
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t trial = lo | (1u << bit);
-            uint32_t c = 0;
-            for (uint32_t p = tid; p < cnt; p += kSelThreads) {
-                const uint2 pr = pairs[p];
-                c += (pr.x == tkey && pr.y < trial) ? 1u : 0u;
-            }
-            c = block_sum_u32(c, scratch);
-            if (c < want_ties) lo = trial;
-        }
-        idx_thr = lo;
-    }
-    auto selected = [=](uint2 p) { return k > 0 && (p.x > tkey || (p.x == tkey && p.y <= idx_thr)); };
-
-    // compaction of the winners (thread-contiguous chunks, block exclusive scan; no atomics)
-    // (no candidate at all: nothing will be added, and the reference says so)
-    const float ref1 = (k > 0 || cnt > 0) ? key_to_float(k > 0 ? tkey : kmax) : -INFINITY;
-    if (mass_out) {
+    if (mass_out)
         for (int l = tid; l < a.L; l += kSelThreads) mx[l] = 0.0f;
-    }
     __syncthreads();
-    const uint32_t chunk = (cnt + kSelThreads - 1) / kSelThreads;
-    const uint32_t lo = min((uint32_t)tid * chunk, cnt), hi = min(lo + chunk, cnt);
-    uint32_t mine = 0;
-    for (uint32_t p = lo; p < hi; ++p) mine += selected(pairs[p]) ? 1u : 0u;
-    scan_s[tid] = mine;
-    __syncthreads();
-    for (int off = 1; off < kSelThreads; off <<= 1) {
-        const uint32_t v = tid >= off ? scan_s[tid - off] : 0u;
-        __syncthreads();
-        scan_s[tid] += v;
-        __syncthreads();
-    }
-    uint32_t at = scan_s[tid] - mine;
-    int32_t *out_idx = a.topk_idx + orow * a.k_cap;
-    float *out_val = a.topk_val ? a.topk_val + orow * a.k_cap : nullptr;
-    for (uint32_t p = lo; p < hi; ++p) {
-        const uint2 pr = pairs[p];
-        if (selected(pr)) {
-            if (at < (uint32_t)a.k_cap) {
-                out_idx[at] = (int32_t)pr.y;
-                if (out_val) out_val[at] = key_to_float(pr.x);
-            }
-            ++at;
-        } else if (mass_out) {
-            atomicAdd(&mx[aux[p]], __expf(key_to_float(pr.x) - ref1));
-        }
-    }
+    SelectOut out;
+    out.out_idx = a.topk_idx + orow * a.k_cap;
+    out.out_val = a.topk_val ? a.topk_val + orow * a.k_cap : nullptr;
+    out.k_cap = (uint32_t)a.k_cap;
+    out.pos_row = pos_row;
+    out.mx = mass_out ? mx : nullptr;
+    out.ref1 = 0.0f;
+    float ref1;
+    if (cnt <= 4u * kSelThreads) select_regs<4>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+    else if (cnt <= 8u * kSelThreads) select_regs<8>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+    else if (cnt <= 16u * kSelThreads) select_regs<16>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+    else select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
     __syncthreads();
     if (mass_out) {
         for (int l = tid; l < a.L; l += kSelThreads) mass_out[(size_t)l * a.GP] = mx[l];
@@ -660,8 +950,8 @@ static size_t scan_lds_bytes(int GP, int L, int mode, int src, bool mass, bool a
     if (mode == kHist) b += (size_t)GP * kHistBins * sizeof(uint32_t);
     if (mode == kEmit) {
         if (mass) b += ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;
-        b += 32 * sizeof(uint32_t) + (size_t)GP * stage_cap * sizeof(uint2);
-        if (aux) b += (size_t)GP * stage_cap * sizeof(uint16_t);
+        b += 2 * kScanWaves * 16 * sizeof(uint32_t) + (size_t)kScanWaves * GP * stage_cap * sizeof(uint2);
+        if (aux) b += (size_t)kScanWaves * GP * stage_cap * sizeof(uint16_t);
     }
     return b;
 }
@@ -669,6 +959,17 @@ static size_t scan_lds_bytes(int GP, int L, int mode, int src, bool mass, bool a
 static int env_int(const char *name, int fallback) {
     const char *v = getenv(name);
     return v ? atoi(v) : fallback;
+}
+
+static int raise_lds_limit(const void *kernel, size_t lds, const char *what) {
+    if (lds <= 64 * 1024) return PQHSA_OK;
+    PQHSA_REQUIRE(lds <= 160 * 1024, "%s: %zu bytes of LDS needed", what, lds);
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) {
+        set_error("%s: cannot raise LDS limit to %zu: %s", what, lds, hipGetErrorString(e));
+        return PQHSA_ELAUNCH;
+    }
+    return PQHSA_OK;
 }
 
 int pick_tile_keys(int64_t n_max, int streams) {
@@ -683,10 +984,12 @@ int pick_tile_keys(int64_t n_max, int streams) {
     return (int)keys;
 }
 
+// per-wave, per-row staging capacity of the candidate scan
 int stage_cap_for(int GP, int tile_keys) {
-    int cap = tile_keys / 4;  // a quarter of the tile may be kept before the slow path starts
-    if (cap > 4096 / GP) cap = 4096 / GP;
-    if (cap < 64) cap = 64;
+    int cap = 512 / GP;
+    const int wave_keys = tile_keys / kScanWaves;
+    if (cap > wave_keys) cap = wave_keys;
+    if (cap < 32) cap = 32;
     return cap;
 }
 
@@ -696,19 +999,12 @@ static int launch_scan_mode(const ScanArgs &a, int GP, int streams, int64_t n_ma
     const int tiles = (int)((n_max + a.tile_keys - 1) / a.tile_keys);
     dim3 grid(tiles, streams);
     const size_t lds = scan_lds_bytes(GP, a.L, MODE, SRC, a.mass != nullptr, a.emit_aux != nullptr, a.stage_cap);
-    PQHSA_REQUIRE(lds <= 160 * 1024, "scan: %zu bytes of LDS needed (GP=%d, L=%d)", lds, GP, a.L);
-#define PQHSA_SCAN_CASE(gp)                                                                          \
-    case gp: {                                                                                       \
-        auto kern = scan_kernel<gp, MODE, SRC>;                                                      \
-        if (lds > 64 * 1024) {                                                                       \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                 \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-            if (e != hipSuccess) {                                                                   \
-                set_error("scan: cannot raise LDS limit to %zu: %s", lds, hipGetErrorString(e));     \
-                return PQHSA_ELAUNCH;                                                                \
-            }                                                                                        \
-        }                                                                                            \
-        hipLaunchKernelGGL(kern, grid, dim3(kScanThreads), lds, stream, a);                          \
+#define PQHSA_SCAN_CASE(gp)                                                               \
+    case gp: {                                                                            \
+        auto kern = scan_kernel<gp, MODE, SRC>;                                           \
+        int rc = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, "scan");      \
+        if (rc) return rc;                                                                \
+        hipLaunchKernelGGL(kern, grid, dim3(kScanThreads), lds, stream, a);               \
     } break;
     if constexpr (SRC == kLogits) {
         PQHSA_REQUIRE(GP == 1, "logit-matrix source handles one row per stream");
@@ -732,33 +1028,28 @@ static int launch_scan_mode(const ScanArgs &a, int GP, int streams, int64_t n_ma
 int launch_scan(const ScanArgs &a, int mode, int src, int GP, int streams, int64_t n_max, hipStream_t stream) {
     if (src == kIndex) {
         if (mode == kWrite) return launch_scan_mode<kWrite, kIndex>(a, GP, streams, n_max, stream);
-        if (mode == kHist) return launch_scan_mode<kHist, kIndex>(a, GP, streams, n_max, stream);
-        return launch_scan_mode<kEmit, kIndex>(a, GP, streams, n_max, stream);
+        if (mode == kEmit) return launch_scan_mode<kEmit, kIndex>(a, GP, streams, n_max, stream);
+    } else {
+        if (mode == kHist) return launch_scan_mode<kHist, kLogits>(a, GP, streams, n_max, stream);
+        if (mode == kEmit) return launch_scan_mode<kEmit, kLogits>(a, GP, streams, n_max, stream);
     }
-    if (mode == kHist) return launch_scan_mode<kHist, kLogits>(a, GP, streams, n_max, stream);
-    if (mode == kEmit) return launch_scan_mode<kEmit, kLogits>(a, GP, streams, n_max, stream);
     set_error("scan: bad mode/source");
     return PQHSA_EINVAL;
 }
 
-int launch_select_final(SelectArgs a, int streams, int64_t n_max, hipStream_t stream) {
+int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
     if (streams == 0) return PQHSA_OK;
-    int64_t key_cap = n_max < 24576 ? n_max : 24576;
-    key_cap = (key_cap + 3) / 4 * 4;
-    if (key_cap < 256) key_cap = 256;
-    // the re-scan path parks a (128 + L)-float table where the keys go later
-    const size_t need_tables = (size_t)(kM * kCodes + a.L) * sizeof(float);
-    size_t lds = (size_t)key_cap * sizeof(uint32_t) + (size_t)a.L * sizeof(float);
-    if (lds < need_tables) lds = need_tables;
-    a.key_cap = (int)key_cap;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(select_final_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) {
-            set_error("select: cannot raise LDS limit to %zu: %s", lds, hipGetErrorString(e));
-            return PQHSA_ELAUNCH;
-        }
-    }
+    PQHSA_REQUIRE(a.s_cap <= (int64_t)kSampleRegsMax * kSelThreads, "sample_thresh: at most %d sampled keys per row, got %lld",
+                  kSampleRegsMax * kSelThreads, (long long)a.s_cap);
+    const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
+    hipLaunchKernelGGL(sample_thresh_kernel, dim3(a.GP, streams), dim3(kSelThreads), lds, stream, a);
+    return check_launch("sample_thresh");
+}
+
+int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
+    if (streams == 0) return PQHSA_OK;
+    // list weights of the losers; the re-scan path parks a (128 + L)-float table there first
+    const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
     hipLaunchKernelGGL(select_final_kernel, dim3(a.G, streams), dim3(kSelThreads), lds, stream, a);
     return check_launch("select_final");
 }
@@ -777,32 +1068,29 @@ int emit_tile_keys_for(int64_t n_cap, int streams) {
 
 // sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
-                       const float *list_scores, float scale, const pqhsa_select *select, uint32_t *hist,
-                       uint32_t *emit_count, uint32_t *thr_bin, int32_t *k_row, float *ref_val, float *ref_extra,
-                       void *pairs, uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans,
-                       int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
-                       hipStream_t stream) {
+                       const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
+                       uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra, void *pairs,
+                       uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans, int emit_tile_keys,
+                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
-    ScanArgs a = {};
-    a.qnorm = qnorm; a.lut = lut; a.list_scores = list_scores; a.scale = scale; a.L = index->num_lists;
-    a.n_div = index->kv_heads; a.G = G;
-    // 1. histogram of the sampled keys (the sample is small: spread it over many workgroups)
-    a.codes = index->s_codes; a.list_ids = index->s_list_ids; a.norms = index->s_norms; a.pos = nullptr;
-    a.n_cap = index->s_cap; a.n_arr = index->s_n; a.tile_keys = kKeysPerIter; a.hist = hist;
-    int rc = launch_scan(a, kHist, kIndex, GP, streams, index->s_cap, stream);
-    if (rc) return rc;
-    profile_mark(kProfThresh, stream);
-    hipLaunchKernelGGL(thresh_sample_kernel, dim3(streams * GP), dim3(kWave), 0, stream, hist, index->n_idx,
-                       index->s_n, index->kv_heads * GP, GP, G, select->fraction, select->topk, thr_bin, k_row,
-                       ref_val);
-    rc = check_launch("thresh_sample");
+    // 1. threshold per row from the sampled keys
+    SampleArgs sa = {};
+    sa.codes = index->s_codes; sa.list_ids = index->s_list_ids; sa.norms = index->s_norms; sa.s_cap = index->s_cap;
+    sa.n_arr = index->n_idx; sa.ns_arr = index->s_n; sa.n_div = index->kv_heads;
+    sa.qnorm = qnorm; sa.lut = lut; sa.list_scores = list_scores; sa.scale = scale;
+    sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
+    sa.thr_key = thr_key; sa.k_row = k_row; sa.ref_val = ref_val;
+    int rc = launch_sample_thresh(sa, streams, stream);
     if (rc) return rc;
     profile_mark(kProfEmit, stream);
     // 2. the full scan
+    ScanArgs a = {};
+    a.qnorm = qnorm; a.lut = lut; a.list_scores = list_scores; a.scale = scale; a.L = index->num_lists;
+    a.n_div = index->kv_heads; a.G = G;
     a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = index->pos;
     a.n_cap = index->n_cap; a.n_arr = index->n_idx; a.nsorted_arr = index->n_sorted;
     a.tile_keys = emit_tile_keys;
-    a.thr_bin = thr_bin; a.ref_val = ref_val; a.emit_count = emit_count;
+    a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
     a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = index->n_cap;
     a.mass = mass; a.stage_cap = stage_cap_for(GP, emit_tile_keys);
     rc = launch_scan(a, kEmit, kIndex, GP, streams, n_max, stream);
@@ -817,7 +1105,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
     s.n_cap = index->n_cap; s.qnorm = qnorm; s.lut = lut; s.list_scores = list_scores; s.scale = scale;
     s.rescans = rescans;
-    rc = launch_select_final(s, streams, n_max, stream);
+    rc = launch_select_final(s, streams, stream);
     profile_mark(kProfAttend, stream);
     return rc;
 }
@@ -844,7 +1132,7 @@ extern "C" int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max
     return launch_scan(a, kWrite, kIndex, padded_groups(G), streams, n_max, static_cast<hipStream_t>(stream));
 }
 
-// workspace of the logit-matrix top-k: hist | emit_count | thr_bin | k_row | ref_val | topk_cnt | pairs
+// workspace of the logit-matrix top-k: hist | emit_count | thr_key | k_row | ref_val | topk_cnt | pairs
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" size_t pqhsa_topk_workspace_bytes(int32_t rows, int64_t n_max) {
@@ -864,12 +1152,12 @@ extern "C" int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t row
     char *w = static_cast<char *>(workspace);
     uint32_t *hist = reinterpret_cast<uint32_t *>(w); w += align256((size_t)rows * kHistBins * 4);
     uint32_t *emit_count = reinterpret_cast<uint32_t *>(w); w += align256((size_t)rows * 4);
-    uint32_t *thr_bin = reinterpret_cast<uint32_t *>(w); w += align256((size_t)rows * 4);
+    uint32_t *thr_key = reinterpret_cast<uint32_t *>(w); w += align256((size_t)rows * 4);
     int32_t *k_row = reinterpret_cast<int32_t *>(w); w += align256((size_t)rows * 4);
     float *ref_val = reinterpret_cast<float *>(w); w += align256((size_t)rows * 4);
     int32_t *cnt_out = reinterpret_cast<int32_t *>(w); w += align256((size_t)rows * 4);
     uint2 *pairs = reinterpret_cast<uint2 *>(w);
-    const size_t zero_bytes = (size_t)(reinterpret_cast<char *>(thr_bin) - reinterpret_cast<char *>(hist));
+    const size_t zero_bytes = (size_t)(reinterpret_cast<char *>(thr_key) - reinterpret_cast<char *>(hist));
     int rc = launch_fill_zero(hist, zero_bytes, stream);
     if (rc) return rc;
     ScanArgs a = {};
@@ -878,15 +1166,15 @@ extern "C" int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t row
     a.hist = hist;
     rc = launch_scan(a, kHist, kLogits, 1, rows, n_max, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(thresh_kernel, dim3(rows), dim3(kWave), 0, stream, hist, n, k, thr_bin, k_row, ref_val);
+    hipLaunchKernelGGL(thresh_kernel, dim3(rows), dim3(kWave), 0, stream, hist, n, k, thr_key, k_row, ref_val);
     rc = check_launch("thresh");
     if (rc) return rc;
-    a.thr_bin = thr_bin; a.ref_val = ref_val; a.emit_count = emit_count; a.emit_pairs = pairs; a.emit_cap = cap;
+    a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count; a.emit_pairs = pairs; a.emit_cap = cap;
     a.stage_cap = stage_cap_for(1, a.tile_keys);
     rc = launch_scan(a, kEmit, kLogits, 1, rows, n_max, stream);
     if (rc) return rc;
     SelectArgs s = {};
     s.pairs = pairs; s.emit_cap = cap; s.emit_count = emit_count; s.k_row = k_row; s.n_arr = n; s.rows_per_n = 1;
     s.GP = 1; s.G = 1; s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = cnt_out; s.k_cap = k_cap;
-    return launch_select_final(s, rows, n_max, stream);
+    return launch_select_final(s, rows, stream);
 }

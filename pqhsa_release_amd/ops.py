@@ -132,6 +132,7 @@ class DeviceIndex:
 
     SAMPLE_RATE = 32
     SAMPLE_MIN = 1024
+    SAMPLE_MAX = 32768   # the threshold kernel keeps the sampled keys of one row in LDS
 
     def __init__(self, batch: int, kv_heads: int, num_lists: int, n_cap: int, device) -> None:
         n_cap = max(8, (int(n_cap) + 7) // 8 * 8)
@@ -161,7 +162,7 @@ class DeviceIndex:
 
     @classmethod
     def sample_size(cls, n: int) -> int:
-        return min(n, max((n + cls.SAMPLE_RATE - 1) // cls.SAMPLE_RATE, cls.SAMPLE_MIN))
+        return min(n, cls.SAMPLE_MAX, max((n + cls.SAMPLE_RATE - 1) // cls.SAMPLE_RATE, cls.SAMPLE_MIN))
 
     @property
     def n_max(self) -> int:
