@@ -303,6 +303,9 @@ def main():
         "kernels": kernels,
         "kernel_sum_us": round(sum(kus.values()), 3),
         "ms_per_step_without_event_log": round(ms_plain, 6),
+        "selection": {"k": math.ceil(layer.n[0] * FRACTION), "rescanned_rows": sum(l.ws.rescans() for l in layers),
+                      "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
+                      "candidates_max": int(layer.ws.candidate_counts().max())},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(layer, args.cpu_seconds)

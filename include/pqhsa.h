@@ -220,6 +220,13 @@ const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t B, int32_t 
                                             int64_t n_cap, int32_t num_lists, int32_t k_cap);
 
 /*
+ * Candidates the last step's scan kept per query row: u32 [B*H, padded_groups(G)] inside the
+ * workspace (device memory, for monitoring the threshold estimate; rows of a padded group hold 0).
+ */
+const uint32_t *pqhsa_decode_candidate_counts(void *workspace, int32_t B, int32_t H, int32_t G,
+                                              int64_t n_cap, int32_t num_lists, int32_t k_cap);
+
+/*
  * Hybrid exact attention alone, given the selection and the per-list masses:
  *   list_mass f32 [BH, G, L] = sum over ALL the list's indexed keys of exp(logit - row_max),
  *   row_max f32 [BH, G] (the maximum approximate logit of the row),

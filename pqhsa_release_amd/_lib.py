@@ -93,6 +93,7 @@ SIGNATURES = {
                                          c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_size_t, c_void_p]),
     "pqhsa_decode_rescan_counter": (c_void_p, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
+    "pqhsa_decode_candidate_counts": (c_void_p, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
     "pqhsa_attend_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "pqhsa_hybrid_attend_paged": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32,
                                                  c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
@@ -115,12 +116,13 @@ def load() -> ctypes.CDLL:
     global _LIB
     if _LIB is not None:
         return _LIB
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("PQHSA_LIBRARY", LIB_PATH)  # another build of the same ABI, e.g. a tuning build
+    if not os.path.exists(path):
         raise PqhsaError(
-            f"{LIB_PATH} is missing: build it with `python -m pqhsa_release_amd.build` "
+            f"{path} is missing: build it with `python -m pqhsa_release_amd.build` "
             "(hipcc, gfx950); there is no fallback path"
         )
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = restype

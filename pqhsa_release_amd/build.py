@@ -28,14 +28,17 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = False, extra: list[str] | None = None) -> str:
+def build(verbose: bool = False, extra: list[str] | None = None, out: str | None = None) -> str:
+    """Compile the library; ``extra`` adds compiler flags and ``out`` names another output file
+    (a tuning build next to the shipped one, loaded through the PQHSA_LIBRARY variable)."""
     os.makedirs(LIBDIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *FLAGS, *(extra or []), *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB]
+    out = out or LIB
+    cmd = [hipcc, *FLAGS, *(extra or []), *[os.path.join(CSRC, s) for s in SOURCES], "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":

@@ -11,6 +11,7 @@
 // attend_reduce_kernel: grid (G, BH).  Folds the split partials under the final row maximum,
 // rescales the two background parts from their reference logits, and normalises.
 #include <cfloat>
+#include <cstdlib>
 
 #include "common.h"
 
@@ -47,19 +48,58 @@ struct AttendArgs {
     int L;
 };
 
+// sum over the 16 lanes of a row group (one DPP row), returned in each of them
 __device__ inline float group_sum16(float v) {
-    v += __shfl_xor(v, 8, kGroupLanes);
-    v += __shfl_xor(v, 4, kGroupLanes);
-    v += __shfl_xor(v, 2, kGroupLanes);
-    v += __shfl_xor(v, 1, kGroupLanes);
+    v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppXor2>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppHalfMirror>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppMirror>(__float_as_int(v)));
     return v;
 }
+
+// One lane's 8 elements of a 128-element row as loaded (16 bytes for 2-byte types, 32 for fp32),
+// converted to floats only when the row is used: a row in flight costs 4 (or 8) registers.
+template <int DT>
+struct RawSlice {
+    static constexpr int kWords = DT == PQHSA_F32 ? 2 : 1;
+    uint4 w[kWords];
+    __device__ inline void zero() {
+#pragma unroll
+        for (int i = 0; i < kWords; ++i) w[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    __device__ inline void load(const char *row, int j) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(row) + (size_t)j * kWords;
+#pragma unroll
+        for (int i = 0; i < kWords; ++i) w[i] = p[i];
+    }
+    __device__ inline void to_float(float (&f)[8]) const {
+        if constexpr (DT == PQHSA_F32) {
+            f[0] = __uint_as_float(w[0].x); f[1] = __uint_as_float(w[0].y);
+            f[2] = __uint_as_float(w[0].z); f[3] = __uint_as_float(w[0].w);
+            f[4] = __uint_as_float(w[1].x); f[5] = __uint_as_float(w[1].y);
+            f[6] = __uint_as_float(w[1].z); f[7] = __uint_as_float(w[1].w);
+        } else {
+            const uint32_t u[4] = {w[0].x, w[0].y, w[0].z, w[0].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (DT == PQHSA_BF16) {
+                    f[2 * i] = __uint_as_float(u[i] << 16);
+                    f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+                } else {
+                    const float2 t = __half22float2(__builtin_bit_cast(__half2, u[i]));
+                    f[2 * i] = t.x;
+                    f[2 * i + 1] = t.y;
+                }
+            }
+        }
+    }
+};
 
 template <int KDT, int QDT>
 __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[kGroups][kD];
-    __shared__ float red_m[kAttThreads / kWave];
+    __shared__ float red_m[kGroups];
     __shared__ float red_l[kGroups];
     __shared__ float bg_s[2][2][kD];
     __shared__ float ms_s[2][kAttThreads / kWave];
@@ -80,6 +120,20 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int cnt = end - start;
     float *part = a.partials + (orow * a.splits + split) * kPartWidth;
 
+    // ---- row addresses of this chunk (block-table lookups happen here, once) ---------------
+    int64_t *off_s = reinterpret_cast<int64_t *>(smem);  // [chunk] element offsets of the rows
+    {
+        const int32_t *tk = a.topk_idx + orow * a.k_cap;
+        for (int i = tid; i < cnt; i += kAttThreads) {
+            const int r = start + i;
+            int64_t pos;
+            if (r < sink_end) pos = r;
+            else if (r < F) pos = local_start + (r - sink_end);
+            else pos = sink_end + tk[r - F];
+            off_s[i] = row_offset(a.kv, b, h, pos);
+        }
+    }
+
     // ---- background slice: lists [l_lo, l_hi) -------------------------------------------
     {
         const int per = (a.L + a.splits - 1) / a.splits;
@@ -91,7 +145,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         const float *m1 = a.mass1 ? a.mass1 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
         float bg0 = 0.0f, bg1 = 0.0f, s0 = 0.0f, s1 = 0.0f;
         if (n > 0) {
-#pragma unroll 4
+#pragma unroll 8
             for (int l = l_lo + half; l < l_hi; l += 2) {
                 const float v = vb[(size_t)l * kD + d];
                 const float w0 = m0 ? m0[(size_t)l * a.mass_l] : 0.0f;
@@ -106,7 +160,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         if ((tid & (kWave - 1)) == 0) { ms_s[0][tid / kWave] = s0; ms_s[1][tid / kWave] = s1; }
-        __syncthreads();
+        __syncthreads();  // also publishes off_s
         if (tid < kD) {
             part[4 + kD + tid] = bg_s[0][0][tid] + bg_s[0][1][tid];
             part[4 + 2 * kD + tid] = bg_s[1][0][tid] + bg_s[1][1][tid];
@@ -123,20 +177,9 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         return;
     }
 
-    int64_t *off_s = reinterpret_cast<int64_t *>(smem);    // [chunk] element offsets of the rows
-    float *x_s = reinterpret_cast<float *>(off_s + chunk);  // [chunk] logits
-
-    // resolve row addresses (block-table lookups happen here, once)
-    const int32_t *tk = a.topk_idx + orow * a.k_cap;
-    for (int i = tid; i < cnt; i += kAttThreads) {
-        const int r = start + i;
-        int64_t pos;
-        if (r < sink_end) pos = r;
-        else if (r < F) pos = local_start + (r - sink_end);
-        else pos = sink_end + tk[r - F];
-        off_s[i] = row_offset(a.kv, b, h, pos);
-    }
-    // this lane's slice of the query row
+    // ---- exact rows: K and V of a row travel together, softmax kept online per row group -----
+    // Each group of 16 lanes owns rows grp, grp + 16, ...; U rows per batch, and the loads of the
+    // next batch are issued before the current one is used.
     const int lane16 = tid & (kGroupLanes - 1);
     const int grp = tid / kGroupLanes;
     float qv[8];
@@ -145,68 +188,82 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         const char *qrow = a.q + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
         load8<QDT>(qrow, lane16, qv);
     }
-    __syncthreads();
-
+    constexpr int U = KDT == PQHSA_F32 ? 2 : 4;
     const size_t kesz = KDT == PQHSA_F32 ? 4 : 2;
-    float lmax = -INFINITY;
-    for (int i = grp; i < cnt; i += 4 * kGroups) {
-        float kv[4][8];
+    using Raw = RawSlice<KDT>;
+    const int my_rows = cnt > grp ? (cnt - grp + kGroups - 1) / kGroups : 0;
+    const int batches = (my_rows + U - 1) / U;
+    auto fetch = [&](Raw (&kb)[U], Raw (&vb)[U], int t) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int ii = i + u * kGroups;
-            if (ii < cnt) load8<KDT>(a.kv.k_base + off_s[ii] * kesz, lane16, kv[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int ii = i + u * kGroups;
-            float d = 0.0f;
+        for (int u = 0; u < U; ++u) {
+            const int ii = grp + kGroups * (t * U + u);
             if (ii < cnt) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) d = __builtin_fmaf(kv[u][e], qv[e], d);
-            }
-            d = group_sum16(d) * a.scale;
-            if (ii < cnt) {
-                lmax = fmaxf(lmax, d);
-                if (lane16 == 0) x_s[ii] = d;
+                const int64_t off = off_s[ii] * (int64_t)kesz;
+                kb[u].load(a.kv.k_base + off, lane16);
+                vb[u].load(a.kv.v_base + off, lane16);
+            } else {
+                kb[u].zero();
+                vb[u].zero();
             }
         }
-    }
-    lmax = wave_max(lmax);
-    if ((tid & (kWave - 1)) == 0) red_m[tid / kWave] = lmax;
-    __syncthreads();
-    float m = red_m[0];
-#pragma unroll
-    for (int w = 1; w < kAttThreads / kWave; ++w) m = fmaxf(m, red_m[w]);
-
+    };
+    float m_g = -INFINITY, l_g = 0.0f;
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-    float lsum = 0.0f;
-    for (int i = grp; i < cnt; i += 4 * kGroups) {
-        float vv[4][8];
-        float p[4];
+    auto consume = [&](const Raw (&kb)[U], const Raw (&vb)[U], int t) {
+        float d[U];
+        float bm = -INFINITY;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int ii = i + u * kGroups;
-            p[u] = 0.0f;
-            if (ii < cnt) {
-                load8<KDT>(a.kv.v_base + off_s[ii] * kesz, lane16, vv[u]);
-                p[u] = __expf(x_s[ii] - m);
-            }
+        for (int u = 0; u < U; ++u) {
+            float kf[8];
+            kb[u].to_float(kf);
+            float x = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x = __builtin_fmaf(kf[e], qv[e], x);
+            x = group_sum16(x) * a.scale;
+            d[u] = (grp + kGroups * (t * U + u) < cnt) ? x : -INFINITY;
+            bm = fmaxf(bm, d[u]);
         }
+        if (bm == -INFINITY) return;  // no row of this batch belongs to the chunk (uniform per group)
+        const float m_new = fmaxf(m_g, bm);
+        const float keep = __expf(m_g - m_new);  // 0 for the first batch (m_g = -inf)
+        l_g *= keep;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int ii = i + u * kGroups;
-            if (ii < cnt) {
-                lsum += p[u];
+        for (int e = 0; e < 8; ++e) acc[e] *= keep;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(p[u], vv[u][e], acc[e]);
+        for (int u = 0; u < U; ++u) {
+            const float p = __expf(d[u] - m_new);  // 0 for rows outside the chunk
+            float vf[8];
+            vb[u].to_float(vf);
+            l_g += p;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(p, vf[e], acc[e]);
+        }
+        m_g = m_new;
+    };
+    {
+        Raw k0[U], v0[U], k1[U], v1[U];
+        if (batches > 0) fetch(k0, v0, 0);
+        for (int t = 0; t < batches; t += 2) {
+            if (t + 1 < batches) fetch(k1, v1, t + 1);
+            consume(k0, v0, t);
+            if (t + 1 < batches) {
+                if (t + 2 < batches) fetch(k0, v0, t + 2);
+                consume(k1, v1, t + 1);
             }
         }
     }
+    // fold the 16 groups under the chunk maximum
+    if (lane16 == 0) red_m[grp] = m_g;
+    __syncthreads();
+    float m = red_m[0];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) red[grp][lane16 * 8 + e] = acc[e];
-    if (lane16 == 0) red_l[grp] = lsum;
+    for (int r = 1; r < kGroups; ++r) m = fmaxf(m, red_m[r]);
+    const float w = m_g == -INFINITY ? 0.0f : __expf(m_g - m);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[grp][lane16 * 8 + e] = acc[e] * w;
+    if (lane16 == 0) red_l[grp] = l_g * w;
     __syncthreads();
     if (tid < kD) {
         float s = 0.0f;
@@ -290,7 +347,8 @@ __global__ __launch_bounds__(kAttThreads) void subtract_selected_kernel(const fl
 }
 
 int pick_splits(int streams_rows, int rows_max) {
-    int s = (1024 + streams_rows - 1) / (streams_rows > 0 ? streams_rows : 1);
+    static const int target = getenv("PQHSA_ATT_WGS") ? atoi(getenv("PQHSA_ATT_WGS")) : 1024;
+    int s = (target + streams_rows - 1) / (streams_rows > 0 ? streams_rows : 1);
     const int need = (rows_max + kMaxChunk - 1) / kMaxChunk;
     if (s < need) s = need;
     if (s < 1) s = 1;
@@ -308,7 +366,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     const int chunk = (rows_max + a.splits - 1) / a.splits;
     PQHSA_REQUIRE(chunk <= 4 * kMaxChunk, "attend: %d rows per query exceed what %d splits can take", rows_max,
                   kMaxSplits);
-    const size_t lds = (size_t)chunk * (sizeof(int64_t) + sizeof(float)) + 16;
+    const size_t lds = (size_t)chunk * sizeof(int64_t) + 16;
     dim3 grid(a.splits, a.G, BH);
 #define PQHSA_ATT(KD, QD)                                                                              \
     {                                                                                                  \

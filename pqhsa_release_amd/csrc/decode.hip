@@ -91,6 +91,12 @@ extern "C" const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t 
     return carve(base, B, H, G, n_cap, num_lists, k_cap).rescans;
 }
 
+extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace, int32_t B, int32_t H, int32_t G,
+                                                         int64_t n_cap, int32_t num_lists, int32_t k_cap) {
+    char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
+    return carve(base, B, H, G, n_cap, num_lists, k_cap).emit_count;
+}
+
 extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
                                  const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
                                  int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,

@@ -360,6 +360,15 @@ class DecodeWorkspace:
         off = ptr - self.buf.data_ptr()
         return int(self.buf[off : off + 4].view(torch.int32).item())
 
+    def candidate_counts(self) -> torch.Tensor:
+        """Candidates the last step's scan kept per query row, int32 [B*H, padded groups]
+        (a view of device memory inside the workspace; rows of a padded group hold 0)."""
+        ptr = _lib.load().pqhsa_decode_candidate_counts(self.buf.data_ptr(), *self._shape)
+        off = ptr - self.buf.data_ptr()
+        b, h, g = self._shape[:3]
+        gp = _lib.load().pqhsa_padded_groups(g)
+        return self.buf[off : off + 4 * b * h * gp].view(torch.int32).view(b * h, gp)
+
 
 def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
                 seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
