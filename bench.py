@@ -43,6 +43,16 @@ CONFIGS = {
 SINK, LOCAL, FRACTION, LISTS, BLOCK = 4, 64, 0.02, 512, 16
 KERNELS = ["lut_build", "sample_thresh", "scan_emit", "select_final", "attend_partial", "attend_reduce"]
 
+# HBM bytes per launch (read + written) of each kernel, from two rocprofv3 counter runs of this
+# script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for a plain
+# 256 MiB device copy (factor 2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE, KiB per dispatch).  Counters
+# cannot be read from inside the timed run, so the figure is carried here per workload; it is
+# reported only for the configuration it was measured on.
+MEASURED_TRAFFIC_BYTES = {
+    2: {"lut_build": 9_582_000, "sample_thresh": 6_723_000, "scan_emit": 53_010_000, "select_final": 17_415_000,
+        "attend_partial": 183_375_000, "attend_reduce": 1_833_000},
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -186,6 +196,7 @@ def cpu_baseline(layer, seconds=12.0):
         "sample": f"torch-CPU restatement of forward_many on 1 of {streams} (sequence, KV head) streams "
                   f"(n={n}, G={G}), {reps} reps, scaled by indexed keys to the whole layer",
         "max_abs_diff_vs_gpu": err,
+        "gpu_out_dtype": str(layer.out.dtype).replace("torch.", ""),  # a bf16 output carries 2^-9 relative rounding
     }
 
 
@@ -198,6 +209,9 @@ def main():
     ap.add_argument("--layers", type=int, default=3, help="distinct resident layers rotated through (defeats cache reuse)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="also run one device copy of this many MiB after the warm-up (a kernel of known HBM "
+                         "traffic, the yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (every sequence and KV head of the layer is on it); "
@@ -221,6 +235,13 @@ def main():
 
     run_steps(args.warmup)
     torch.cuda.synchronize()
+    if args.calibrate_copy_mib > 0:
+        src = torch.empty(args.calibrate_copy_mib * 262144, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def logged_run(count, only):
         """count steps with the HIP-event log on the stream; returns (ms per step, per-kernel ms)."""
@@ -271,7 +292,7 @@ def main():
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(dom_bytes / 1e3 / dom_us / HBM_PEAK_GBPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get(dominant),
         "algorithmic_bytes": dom_bytes,
         "launch_us": round(dom_us, 3),
     }

@@ -292,7 +292,8 @@ __global__ __launch_bounds__(kD) void attend_reduce_kernel(AttendArgs a) {
     const float r1 = (n > 0 && a.mass1) ? a.ref1[(size_t)bh * a.ref_stride + g] : -INFINITY;
     float ms0 = 0.0f, ms1 = 0.0f;
     float m = -INFINITY;
-    for (int s = 0; s < a.splits; ++s) {
+#pragma unroll 8
+    for (int s = 0; s < a.splits; ++s) {  // independent loads: several splits in flight at once
         m = fmaxf(m, part[s * kPartWidth]);
         ms0 += part[s * kPartWidth + 2];
         ms1 += part[s * kPartWidth + 3];
@@ -309,6 +310,7 @@ __global__ __launch_bounds__(kD) void attend_reduce_kernel(AttendArgs a) {
     const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
     const float f1 = (ms1 != 0.0f && r1 > -INFINITY) ? __expf(r1 - m) : 0.0f;
     float acc = 0.0f, den = 0.0f;
+#pragma unroll 8
     for (int s = 0; s < a.splits; ++s) {
         const float *p = part + s * kPartWidth;
         const float w = p[0] == -INFINITY ? 0.0f : __expf(p[0] - m);
