@@ -234,3 +234,145 @@ def test_missing_or_bad_arguments_fail_loudly():
         ops.kv_contiguous(torch.zeros(1, 1, 8, 128), torch.zeros(1, 1, 8, 128))   # CPU tensors
     with pytest.raises(ValueError):
         ops.lut_build(torch.zeros(1, 17, 128, device=dev), idx, 17)         # G too large
+
+
+def _check_step(p, idx, kv, ws, fraction, tol=1e-4):
+    q = p.q_tensor()
+    out = torch.empty_like(q)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
+                    topk=0, scale=SCALE, workspace=ws)
+    torch.cuda.synchronize()
+    tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+    o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    for (b, h) in p.index:
+        want_out, want_idx, _ = p.oracle_step(b, h, fraction)
+        k = want_idx.shape[1]
+        for g in range(p.G):
+            assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (b, h, g)
+        assert np.abs(o[b, h] - want_out).max() <= tol, (b, h)
+
+
+def test_decode_step_rescans_rows_when_the_sampled_threshold_keeps_too_few():
+    """A sample made of the stream's best-scoring keys puts the threshold far too high: every row
+    keeps fewer than k candidates, is re-scored in full by its selection workgroup, and the
+    result is still the exact top-k with the right background."""
+    dev = _cuda()
+    p = Problem(lens=[6000], heads=1, groups=2, lists=32, seed=29)
+    idx = p.device_index(dev)
+    _, _, logits = p.oracle_step(0, 0, 0.02)
+    ns = int(idx.s_n[0])
+    best = np.argsort(-logits.max(axis=0), kind="stable")[:ns].copy()      # retrieval-local key indices
+    codes, lists, norms = idx.by_key(0, p.n(0))
+    pick = torch.from_numpy(best).to(dev)
+    idx.s_codes[0, :ns], idx.s_list_ids[0, :ns], idx.s_norms[0, :ns] = codes[pick], lists[pick], norms[pick]
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.02, 0))
+    before = ws.rescans()
+    _check_step(p, idx, ops.kv_contiguous(*p.dense_kv()), ws, 0.02)
+    assert ws.rescans() - before == p.G, "both rows should have taken the full re-scan"
+    assert int(ws.candidate_counts()[0, : p.G].max()) < ops.resolve_topk(p.n_max, 0.02, 0)
+
+
+def test_decode_step_on_unsorted_and_partly_sorted_layouts():
+    """The same step over (i) an index that was never sorted or sampled (every key is a candidate),
+    (ii) a sorted prefix followed by an insertion-order tail, as after appends."""
+    dev = _cuda()
+    p = Problem(lens=[3000, 2100], heads=2, groups=3, lists=32, seed=31)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    raw = p.device_index(dev, finalize=False)
+    ws = ops.DecodeWorkspace(raw, p.G, ops.resolve_topk(p.n_max, 0.05, 0))
+    _check_step(p, raw, kv, ws, 0.05)
+    counts = [p.n(b) for b in range(p.B)]
+    part = p.device_index(dev, finalize=False)
+    part.set_counts([c - 700 for c in counts])     # sort and sample the first keys only ...
+    part.finalize_layout()
+    part.set_counts(counts)                         # ... the last 700 stay in insertion order
+    assert part.tail_max() == 700
+    ws2 = ops.DecodeWorkspace(part, p.G, ops.resolve_topk(p.n_max, 0.05, 0))
+    _check_step(p, part, kv, ws2, 0.05)
+    assert ws2.rescans() == 0
+
+
+def test_hybrid_attend_paged_alone_matches_oracle():
+    """The stand-alone attention entry point, fed the oracle's own selection and per-list masses."""
+    dev = _cuda()
+    p = Problem(lens=[1500, 900], heads=2, groups=2, lists=16, dtype=torch.bfloat16, seed=37)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("4d"))
+    frac = 0.03
+    k_cap = ops.resolve_topk(p.n_max, frac, 0)
+    rows = p.B * p.H * p.G
+    tidx = torch.full((rows, k_cap), 0, dtype=torch.int32)
+    tval = torch.zeros(rows, k_cap)
+    tcnt = torch.zeros(rows, dtype=torch.int32)
+    mass = torch.zeros(rows, p.L)
+    rmax = torch.zeros(rows)
+    want = {}
+    for (b, h), ix in p.index.items():
+        out, sel, logits = p.oracle_step(b, h, frac)
+        want[b, h] = out
+        for g in range(p.G):
+            r = (b * p.H + h) * p.G + g
+            k = sel.shape[1]
+            tidx[r, :k] = torch.from_numpy(sel[g].astype(np.int32))
+            tval[r, :k] = torch.from_numpy(logits[g, sel[g]])
+            tcnt[r] = k
+            rmax[r] = float(logits[g].max())
+            w = np.exp(logits[g].astype(np.float64) - float(logits[g].max()))
+            mass[r] = torch.from_numpy(np.bincount(ix["list_ids"].astype(np.int64), weights=w, minlength=p.L)).float()
+    q = p.q_tensor().float()
+    out = torch.empty_like(q)
+    ops.hybrid_attend_paged(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
+                            topk_idx=tidx.to(dev), topk_val=tval.to(dev), topk_cnt=tcnt.to(dev),
+                            list_mass=mass.to(dev), row_max=rmax.to(dev), scale=SCALE)
+    torch.cuda.synchronize()
+    o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    for (b, h), w in want.items():
+        assert np.abs(o[b, h] - w).max() <= 2e-3, (b, h, np.abs(o[b, h] - w).max())
+
+
+def test_full_size_step_properties_at_the_cfg1_shape():
+    """At a full configuration size (context 32 768, 8 KV heads, GQA 4, bf16 paged) the oracle is
+    too slow, so the step is checked through properties: the selected set is exactly the k best of
+    the logits pqhsa_lut_scan writes for the same tables, nothing was re-scanned, and the output
+    equals a dense torch attention in which unselected stored keys are replaced by their list's
+    mean value under the approximate logits."""
+    import bench
+
+    dev = _cuda()
+    layer = bench.Layer(1, 4242, torch.device(dev))
+    layer.call.run(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    idx, G, H = layer.index, layer.G, layer.H
+    n = layer.n[0]
+    k = ops.resolve_topk(n, bench.FRACTION, 0)
+    qnorm, lut, ls = ops.lut_build(layer.q, idx, G)
+    logits = ops.lut_scan(idx, G, qnorm, lut, ls, 1.0 / np.sqrt(128.0))       # [BH, G, n_cap] by key index
+    tidx = layer.ws.topk_idx.view(H, G, -1)[:, :, :k].to(torch.int64)
+    tval = layer.ws.topk_val.view(H, G, -1)[:, :, :k]
+    lg = logits.view(H, G, -1)[:, :, :n]
+    assert torch.equal(torch.gather(lg, 2, tidx), tval)                        # the selected logits, bit for bit
+    kth = torch.topk(lg, k, dim=2).values[:, :, -1:]
+    assert bool((tval >= kth).all()) and bool((tidx.sort(dim=2).values.diff(dim=2) > 0).all())   # k distinct keys, none below the k-th
+    assert layer.ws.rescans() == 0
+    # reference combination in fp64 on the device for one KV head
+    h = 3
+    kk, vv = ops.paged_gather_range(layer.kv, 0, 0, layer.lens[0])
+    K, V = kk[h].double(), vv[h].double()
+    q = layer.q[0, h * G : (h + 1) * G].double()
+    sink = bench.SINK
+    sel = torch.zeros(G, n, dtype=torch.bool, device=dev)
+    sel.scatter_(1, tidx[h], True)
+    exact = (q @ K.T) / np.sqrt(128.0)
+    _, lists, _ = idx.by_key(h, n)
+    lists = lists.to(torch.int64) & 0xFFFF
+    m = torch.maximum(exact.max(dim=1).values, lg[h].double().max(dim=1).values)[:, None]
+    w_exact = torch.exp(exact - m)
+    w_exact[:, sink : sink + n] *= sel                                            # unselected stored keys leave the exact part
+    w_bg = torch.exp(lg[h].double() - m) * (~sel)
+    mass = torch.zeros(G, idx.num_lists, dtype=torch.float64, device=dev).index_add_(1, lists, w_bg)
+    num = w_exact @ V + mass @ idx.vbar[h].double()
+    den = w_exact.sum(dim=1, keepdim=True) + mass.sum(dim=1, keepdim=True)
+    want = (num / den).float()
+    got = layer.out[0, h * G : (h + 1) * G].float()
+    err = (got - want).abs()
+    assert bool((err <= 2e-3 + 2.0 ** -8 * want.abs()).all()), float(err.max())
