@@ -488,11 +488,12 @@ __device__ inline uint32_t block_total_of_waves(uint32_t wave_count, uint32_t (*
 __device__ inline uint32_t wave_count_if(bool pred) { return (uint32_t)__popcll(__ballot(pred)); }
 
 // Keys held in registers, R per thread.  Returns the largest T with count(key >= T) >= want (the
-// want-th largest key); padding keys are 0 and never counted (T >= 1).  Stops early, with
-// `exact` set, at a prefix T whose count is exactly want: then {key >= T} is the answer set.
+// want-th largest key); padding keys are 0 and never counted (T >= 1).  Stops early at a prefix T
+// whose count is within [want, want + slack]; `exact` is set when that count is exactly want:
+// then {key >= T} is the answer set.
 template <int R>
-__device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, uint32_t (*red)[kSelWaves],
-                                       int &step, bool &exact) {
+__device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, uint32_t slack,
+                                       uint32_t (*red)[kSelWaves], int &step, bool &exact) {
     uint32_t t = 0u;
     exact = false;
     for (int bit = 31; bit >= 0; --bit) {
@@ -501,10 +502,12 @@ __device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, 
 #pragma unroll
         for (int r = 0; r < R; ++r) c += wave_count_if(key[r] >= trial);
         c = block_total_of_waves(c, red, step++);
-        if (c >= want) t = trial;
-        if (c == want) {
-            exact = true;
-            break;
+        if (c >= want) {
+            t = trial;
+            if (c - want <= slack) {  // close enough for the caller (slack 0: exactly want keys)
+                exact = c == want;
+                break;
+            }
         }
     }
     return t;
@@ -560,36 +563,10 @@ struct SampleArgs {
 
 constexpr int kSampleRegsMax = 32;  // sampled keys per thread: at most 32768 per row
 
+// R sampled keys per thread (s_cap <= R * 1024, chosen by the host).  The sampled keys are
+// requested before anything else, together with the row's tables and counts, so the kernel has
+// one round trip to memory before it computes.
 template <int R>
-__device__ inline uint32_t sample_kth(const SampleArgs &a, int bh, int ns, const float *lut_s, const float *ls_s,
-                                      float qn, uint32_t want, uint32_t (*red)[kSelWaves]) {
-    const size_t base = (size_t)bh * a.s_cap;
-    uint32_t key[R];
-    constexpr int kBatch = R < 8 ? R : 8;  // loads of one batch are all in flight before their first use
-#pragma unroll
-    for (int r0 = 0; r0 < R; r0 += kBatch) {
-        uint32_t code[kBatch], lid[kBatch];
-        float kn[kBatch];
-#pragma unroll
-        for (int r = 0; r < kBatch; ++r) {
-            const int p = (r0 + r) * kSelThreads + (int)threadIdx.x;
-            const bool ok = p < ns;
-            code[r] = ok ? a.codes[base + p] : 0u;
-            lid[r] = ok ? a.list_ids[base + p] : 0u;
-            kn[r] = ok ? a.norms[base + p] : 0.0f;
-        }
-#pragma unroll
-        for (int r = 0; r < kBatch; ++r) {
-            const int p = (r0 + r) * kSelThreads + (int)threadIdx.x;
-            if (lid[r] >= (uint32_t)a.L) lid[r] = 0u;
-            key[r0 + r] = p < ns ? order_key(score_one(lut_s, ls_s, code[r], lid[r], qn, kn[r], a.scale)) : 0u;
-        }
-    }
-    int step = 0;
-    bool exact;
-    return bisect_regs<R>(key, want, red, step, exact);
-}
-
 __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
@@ -597,9 +574,6 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     const int g = blockIdx.x;
     const int bh = blockIdx.y;
     const size_t row = (size_t)bh * a.GP + g;
-    const int n = a.n_arr[bh / a.n_div];
-    const int ns = a.ns_arr[bh / a.n_div];
-    int k = resolve_k(n, a.fraction, a.topk);
     if (g >= a.G) {
         if (tid == 0) {
             a.thr_key[row] = 0xffffffffu;
@@ -608,6 +582,29 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         }
         return;
     }
+    constexpr int kBatch = R < 8 ? R : 8;  // loads of one batch are all in flight before their first use
+    const size_t base = (size_t)bh * a.s_cap;
+    uint32_t code[kBatch], lid[kBatch];
+    float kn[kBatch];
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int64_t p = (int64_t)(r0 + r) * kSelThreads + tid;
+            const bool ok = p < a.s_cap;  // the arrays are allocated (and zero) up to s_cap
+            code[r] = ok ? a.codes[base + p] : 0u;
+            lid[r] = ok ? a.list_ids[base + p] : 0u;
+            kn[r] = ok ? a.norms[base + p] : 0.0f;
+        }
+    };
+    fetch(0);
+    const int n = a.n_arr[bh / a.n_div];
+    const int ns = a.ns_arr[bh / a.n_div];
+    float *lut_s = reinterpret_cast<float *>(smem);   // [128]
+    float *ls_s = lut_s + kM * kCodes;                // [L]
+    for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
+    for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
+    const float qn = a.qnorm[row];
+    const int k = resolve_k(n, a.fraction, a.topk);
     // expected sampled keys among the top max(k, 1), plus the margin
     const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
     const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
@@ -622,18 +619,22 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         return;
     }
     const uint32_t want = (uint32_t)want_d;
-
-    float *lut_s = reinterpret_cast<float *>(smem);   // [128]
-    float *ls_s = lut_s + kM * kCodes;                // [L]
-    for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
-    for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
-    const float qn = a.qnorm[row];
     __syncthreads();
-    uint32_t t;
-    if (ns <= 4 * kSelThreads) t = sample_kth<4>(a, bh, ns, lut_s, ls_s, qn, want, red);
-    else if (ns <= 8 * kSelThreads) t = sample_kth<8>(a, bh, ns, lut_s, ls_s, qn, want, red);
-    else if (ns <= 16 * kSelThreads) t = sample_kth<16>(a, bh, ns, lut_s, ls_s, qn, want, red);
-    else t = sample_kth<kSampleRegsMax>(a, bh, ns, lut_s, ls_s, qn, want, red);
+    uint32_t key[R];
+#pragma unroll
+    for (int r0 = 0; r0 < R; r0 += kBatch) {
+        if (r0 > 0) fetch(r0);
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int p = (r0 + r) * kSelThreads + tid;
+            if (lid[r] >= (uint32_t)a.L) lid[r] = 0u;
+            key[r0 + r] = p < ns ? max(order_key(score_one(lut_s, ls_s, code[r], lid[r], qn, kn[r], a.scale)), 1u) : 0u;
+        }
+    }
+    int step = 0;
+    bool exact;
+    // any threshold that keeps between want and 9/8 want sampled keys serves: fewer search steps
+    const uint32_t t = bisect_regs<R>(key, want, want / 8u, red, step, exact);
     if (tid == 0) {
         a.thr_key[row] = t;
         a.k_row[row] = k;
@@ -671,6 +672,7 @@ struct SelectArgs {
     const float *list_scores;
     float scale;
     uint32_t *rescans;     // [1] counter of rows that needed the full re-scan (diagnostics)
+    int64_t expected_candidates;  // host's upper estimate of candidates per row (0: unknown)
 };
 
 // Exclusive prefix over the workgroup of a per-thread count (one barrier pair).
@@ -704,26 +706,18 @@ struct SelectOut {
     }
 };
 
-// Candidates in registers (cnt <= R * 1024).
+// Candidates in registers (cnt <= R * 1024): candidate p = r * 1024 + tid sits in slot r of thread
+// tid; slots at or past cnt hold key 0.
 template <int R>
-__device__ inline void select_regs(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
-                                   const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
-                                   uint32_t *wsum, float *ref1_out) {
+__device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
+                                     int k, const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                     uint32_t *wsum, float *ref1_out) {
     const int tid = threadIdx.x;
-    uint32_t key[R], where[R], list[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
-        const uint32_t p = (uint32_t)r * kSelThreads + tid;
-        const uint2 pr = p < cnt ? pairs[p] : make_uint2(0u, 0u);
-        key[r] = pr.x;
-        where[r] = pr.y;
-        list[r] = (aux && p < cnt) ? aux[p] : 0u;
-    }
     int step = 0;
     bool exact = false;
     uint32_t tkey = 0u;
     if (k > 0) {
-        tkey = bisect_regs<R>(key, (uint32_t)k, red, step, exact);
+        tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact);
     } else {  // nothing is selected: the reference of the losers' weights is the largest key
         uint32_t kmax = 0u;
 #pragma unroll
@@ -786,6 +780,22 @@ __device__ inline void select_regs(const SelectArgs &a, uint32_t cnt, int k, con
             out.loser(tie_loser ? tkey : key[r], list[r]);
         }
     }
+}
+
+template <int R>
+__device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
+                                   const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                   uint32_t *wsum, float *ref1_out) {
+    uint32_t key[R], where[R], list[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
+        const uint32_t p = (uint32_t)r * kSelThreads + threadIdx.x;
+        const uint2 pr = p < cnt ? pairs[p] : make_uint2(0u, 0u);
+        key[r] = pr.x;
+        where[r] = pr.y;
+        list[r] = (aux && p < cnt) ? aux[p] : 0u;
+    }
+    select_loaded<R>(key, where, list, cnt, k, pos_row, out, red, wsum, ref1_out);
 }
 
 // Candidates in memory (any count): the same selection, streaming the pairs on every pass.
@@ -862,6 +872,10 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
     }
 }
 
+// RS > 0: the host expects at most RS * 1024 candidates per row, and the kernel requests that many
+// candidate slots before it knows the count, together with the count itself (one round trip to
+// memory instead of two); slots past the count hold leftovers of earlier steps and are masked.
+template <int RS>
 __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
@@ -877,10 +891,24 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     uint2 *pairs = a.pairs + row * a.emit_cap;
     uint16_t *aux = a.aux ? a.aux + row * a.emit_cap : nullptr;
     const int32_t *pos_row = a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr;
+    constexpr int RA = RS > 0 ? RS : 1;
+    uint32_t skey[RA], swhere[RA], slist[RA];
+    if constexpr (RS > 0) {
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            const int64_t p = (int64_t)r * kSelThreads + tid;
+            const bool ok = p < a.emit_cap;
+            const uint2 pr = ok ? pairs[p] : make_uint2(0u, 0u);
+            skey[r] = pr.x;
+            swhere[r] = pr.y;
+            slist[r] = (aux && ok) ? aux[p] : 0u;
+        }
+    }
     uint32_t cnt = a.emit_count[row];
     float *mass_out = a.mass_extra ? a.mass_extra + (size_t)bh * a.L * a.GP + g : nullptr;
+    const bool rescan = cnt < (uint32_t)k && a.codes;
 
-    if (cnt < (uint32_t)k && a.codes) {
+    if (rescan) {
         // The estimate kept too few keys: score the whole row again and treat every key as a
         // candidate.  The row's background sums start over (all of them land in mass_extra).
         if (tid == 0 && a.rescans) atomicAdd(a.rescans, 1u);
@@ -917,10 +945,27 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     out.mx = mass_out ? mx : nullptr;
     out.ref1 = 0.0f;
     float ref1;
-    if (cnt <= 4u * kSelThreads) select_regs<4>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-    else if (cnt <= 8u * kSelThreads) select_regs<8>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-    else if (cnt <= 16u * kSelThreads) select_regs<16>(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-    else select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+    bool done = false;
+    if constexpr (RS > 0) {
+        if (!rescan && cnt <= (uint32_t)RS * kSelThreads) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) {
+                if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, swhere[r] = 0u, slist[r] = 0u;
+            }
+            select_loaded<RS>(skey, swhere, slist, cnt, k, pos_row, out, red, wsum, &ref1);
+            done = true;
+        }
+    }
+    if (!done) {
+        if constexpr (RS == 0) {  // no estimate: pick the register variant from the count
+            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+            else select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+        } else {  // the estimate was exceeded, or the row was re-scanned (rare): stream from memory
+            select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+        }
+    }
     __syncthreads();
     if (mass_out) {
         for (int l = tid; l < a.L; l += kSelThreads) mass_out[(size_t)l * a.GP] = mx[l];
@@ -1042,7 +1087,11 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
     PQHSA_REQUIRE(a.s_cap <= (int64_t)kSampleRegsMax * kSelThreads, "sample_thresh: at most %d sampled keys per row, got %lld",
                   kSampleRegsMax * kSelThreads, (long long)a.s_cap);
     const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
-    hipLaunchKernelGGL(sample_thresh_kernel, dim3(a.GP, streams), dim3(kSelThreads), lds, stream, a);
+    const dim3 grid(a.GP, streams), block(kSelThreads);
+    if (a.s_cap <= 4 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<4>, grid, block, lds, stream, a);
+    else if (a.s_cap <= 8 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<8>, grid, block, lds, stream, a);
+    else if (a.s_cap <= 16 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<16>, grid, block, lds, stream, a);
+    else hipLaunchKernelGGL(sample_thresh_kernel<kSampleRegsMax>, grid, block, lds, stream, a);
     return check_launch("sample_thresh");
 }
 
@@ -1050,7 +1099,12 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     if (streams == 0) return PQHSA_OK;
     // list weights of the losers; the re-scan path parks a (128 + L)-float table there first
     const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
-    hipLaunchKernelGGL(select_final_kernel, dim3(a.G, streams), dim3(kSelThreads), lds, stream, a);
+    const dim3 grid(a.G, streams), block(kSelThreads);
+    if (a.expected_candidates <= 0) hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
+    else if (a.expected_candidates <= 4 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<4>, grid, block, lds, stream, a);
+    else if (a.expected_candidates <= 8 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<8>, grid, block, lds, stream, a);
+    else if (a.expected_candidates <= 16 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<16>, grid, block, lds, stream, a);
+    else hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
     return check_launch("select_final");
 }
 
@@ -1105,6 +1159,14 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
     s.n_cap = index->n_cap; s.qnorm = qnorm; s.lut = lut; s.list_scores = list_scores; s.scale = scale;
     s.rescans = rescans;
+    {
+        // what the threshold estimate aims at for the longest row, plus its tolerance and a margin
+        const double ns = (double)(index->s_cap < n_max ? index->s_cap : n_max);
+        const int kmax = resolve_k((int)n_max, select->fraction, select->topk);
+        const double ks = (double)(kmax > 1 ? kmax : 1) * ns / (double)(n_max > 1 ? n_max : 1);
+        const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
+        s.expected_candidates = (int64_t)((ceil(x * x) + 1.0) * 1.125 * ((double)n_max / (ns > 1.0 ? ns : 1.0)) * 1.12) + 64;
+    }
     rc = launch_select_final(s, streams, stream);
     profile_mark(kProfAttend, stream);
     return rc;
