@@ -273,6 +273,19 @@ def main():
     torch.cuda.synchronize()
     ms_plain = (time.perf_counter() - t2) * 1000.0 / args.steps
 
+    # the same steps replayed from HIP graphs (one per resident layer): what a serving loop that
+    # captures its steady state would see
+    for l in layers:
+        l.call.capture()
+    for i in range(args.warmup):
+        layers[i % len(layers)].call.replay()
+    torch.cuda.synchronize()
+    t3 = time.perf_counter()
+    for i in range(args.steps):
+        layers[i % len(layers)].call.replay()
+    torch.cuda.synchronize()
+    ms_graph = (time.perf_counter() - t3) * 1000.0 / args.steps
+
     layer = layers[0]
     ab = layer.algorithmic_bytes()
     kus = {name: survey[i] * 1000.0 for i, name in enumerate(KERNELS)}
@@ -324,6 +337,7 @@ def main():
         "kernels": kernels,
         "kernel_sum_us": round(sum(kus.values()), 3),
         "ms_per_step_without_event_log": round(ms_plain, 6),
+        "ms_per_step_graph_replay": round(ms_graph, 6),
         "selection": {"k": math.ceil(layer.n[0] * FRACTION), "rescanned_rows": sum(l.ws.rescans() for l in layers),
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},

@@ -50,7 +50,6 @@ struct ScanArgs {
     int64_t logits_in_stride;
     // shape
     const int32_t *n_arr;       // n = n_arr[stream / n_div]
-    const int32_t *nsorted_arr; // leading keys ordered by list (NULL: none)
     int n_div;
     int G;
     int tile_keys;
@@ -116,7 +115,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int tile0 = blockIdx.x * a.tile_keys;
     if (tile0 >= n) return;
     const int tile_end = min(n, tile0 + a.tile_keys);
-    const int nsorted = (MODE == kEmit && a.nsorted_arr) ? a.nsorted_arr[bh / a.n_div] : 0;
     const int L = a.L;
 
     // ---- LDS carve-up ----------------------------------------------------------------
@@ -1142,7 +1140,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.qnorm = qnorm; a.lut = lut; a.list_scores = list_scores; a.scale = scale; a.L = index->num_lists;
     a.n_div = index->kv_heads; a.G = G;
     a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = index->pos;
-    a.n_cap = index->n_cap; a.n_arr = index->n_idx; a.nsorted_arr = index->n_sorted;
+    a.n_cap = index->n_cap; a.n_arr = index->n_idx;
     a.tile_keys = emit_tile_keys;
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
     a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = index->n_cap;

@@ -431,6 +431,23 @@ class DecodeCall:
         if rc:
             _lib.check(rc, "pqhsa_decode_step")
 
+    def capture(self) -> "torch.cuda.CUDAGraph":
+        """Record the step's kernels into a HIP graph (the graphed steady state of the reference's
+        sidecar, benchmarks e2e:6052-6235).  The step clears its scratch with kernels, so the
+        graph holds no memset nodes.  A replay runs on the tensors' current contents (new queries
+        are copied into ``q``, counts live in device memory); ``n_max``, ``full_max`` and the
+        launch shapes are those of the capture, so the index must not outgrow them."""
+        self.run()                      # once outside: kernel attributes are set before capture
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.run()
+        self.graph = graph
+        return graph
+
+    def replay(self) -> None:
+        self.graph.replay()
+
 
 def hybrid_attend_paged(q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int, full_max: int,
                         topk_idx, topk_val, topk_cnt, list_mass, row_max, scale: float) -> torch.Tensor:

@@ -376,3 +376,34 @@ def test_full_size_step_properties_at_the_cfg1_shape():
     got = layer.out[0, h * G : (h + 1) * G].float()
     err = (got - want).abs()
     assert bool((err <= 2e-3 + 2.0 ** -8 * want.abs()).all()), float(err.max())
+
+
+def test_decode_step_graph_replays_match_eager_runs():
+    """The step recorded into a HIP graph and replayed several times, with eager work and
+    synchronisations between the replays, gives what the eager step gives for the same query."""
+    dev = _cuda()
+    p = Problem(lens=[2600, 1900], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=43)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    q = p.q_tensor().float()
+    out = torch.empty_like(q)
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
+    call = ops.DecodeCall(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
+                          fraction=0.03, topk=0, scale=SCALE, workspace=ws)
+    call.capture()
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    base = q.clone()
+    for round_ in range(4):
+        q.copy_(base + 0.3 * round_ * torch.randn(base.shape, generator=gen).to(dev))
+        call.run()
+        torch.cuda.synchronize()
+        want_out, want_idx = out.clone(), ws.topk_idx.clone().sort(dim=1).values
+        out.zero_()
+        ws.topk_idx.fill_(-1)
+        junk = (torch.randn(512, 512, device=dev) @ torch.randn(512, 512, device=dev)).sum()   # unrelated eager work
+        torch.cuda.synchronize()
+        call.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ws.topk_idx.sort(dim=1).values, want_idx), round_
+        np.testing.assert_allclose(out.cpu().numpy(), want_out.cpu().numpy(), atol=1e-5, err_msg=str(round_))
+        assert torch.isfinite(junk)
