@@ -213,6 +213,30 @@ int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_
                       size_t workspace_bytes, void *stream);
 
 /*
+ * The steady-state serving step: append, then attend, in the same launches.  Every sequence b
+ * with append_count[b] > 0 (i32 [B], device) first gets ONE key encoded into each of its
+ * streams: the key at retrieval-local index n_idx[b] (token sink + n_idx[b], which the caller
+ * has already written to `kv`), with its norm, list id and PQ codes stored at the end of the
+ * stream's keys and its value row added to the list's sum, count and mean.  The decode step then
+ * runs over n_idx[b] + 1 keys, and its last kernel stores the new counts into index->n_idx, so
+ * the device-side index needs no host update between steps.  n_max and select->k_cap must
+ * already account for the appended key; the sampled subset and the list-sorted prefix are not
+ * touched (the new key joins the insertion-order tail).  Everything else is as for
+ * pqhsa_decode_step.
+ * Replaces the per-step IVFPQIndex.add + value-summary append of the reference
+ * (pq_hsa/index/ivfpq.py:598-645; pq_hsa/attention/kv_cache.py:730-764) and the sidecar's
+ * one-launch lean append (benchmarks/vllm_backend/gqa_sidecar_fast.py lean_append; pq_append_prep,
+ * pq_hsa/kernels/cuda/pq_fused_h20.cu:2888-2922), followed by the decode step above.
+ */
+int pqhsa_append_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                             const pqhsa_index *index, int32_t G, const int32_t *seq_lens,
+                             int32_t sink, int32_t n_max, int32_t full_max,
+                             const pqhsa_select *select, float scale, float eps,
+                             int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
+                             void *workspace, size_t workspace_bytes,
+                             const int32_t *append_count, void *stream);
+
+/*
  * Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full since
  * the workspace was first used (a device-memory counter inside the workspace, for monitoring).
  */

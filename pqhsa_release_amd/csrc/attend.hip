@@ -46,6 +46,9 @@ struct AttendArgs {
     int ref_stride;
     const float *vbar;        // [BH, L, 128]
     int L;
+    // after a fused append: the step's last kernel stores the new key counts into the index
+    const int32_t *n_commit_src;  // [B] (NULL: nothing to store)
+    int32_t *n_commit_dst;        // [B]
 };
 
 // sum over the 16 lanes of a row group (one DPP row), returned in each of them
@@ -112,7 +115,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int sink_end = min(a.sink, len);
     const int local_start = sink_end + n;
     const int F = sink_end + max(len - local_start, 0);
-    const int k = a.topk_cnt[orow];
+    const int k = min(a.topk_cnt[orow], (int)a.k_cap);  // never read past the row of the index array
     const int total = F + k;
     const int chunk = (total + a.splits - 1) / a.splits;
     const int start = min(split * chunk, total);
@@ -287,6 +290,7 @@ __global__ __launch_bounds__(kD) void attend_reduce_kernel(AttendArgs a) {
     const int b = bh / a.H, h = bh % a.H;
     const size_t orow = (size_t)bh * a.G + g;
     const int n = a.n_idx[b];
+    if (a.n_commit_dst && g == 0 && h == 0 && d == 0) a.n_commit_dst[b] = a.n_commit_src[b];
     const float *part = a.partials + orow * a.splits * kPartWidth;
     const float r0 = (n > 0 && a.mass0) ? a.ref0[(size_t)bh * a.ref_stride + g] : -INFINITY;
     const float r1 = (n > 0 && a.mass1) ? a.ref1[(size_t)bh * a.ref_stride + g] : -INFINITY;
@@ -404,7 +408,8 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
-                  const float *ref_val, const float *ref_extra, float scale, float *partials, hipStream_t stream) {
+                  const float *ref_val, const float *ref_extra, float scale, float *partials,
+                  const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
@@ -414,6 +419,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
     a.mass0 = mass; a.mass1 = mass_extra; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
     a.ref0 = ref_val; a.ref1 = ref_extra; a.ref_stride = GP;
     a.vbar = index->vbar; a.L = index->num_lists;
+    a.n_commit_src = n_commit_src; a.n_commit_dst = n_commit_dst;
     return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream);
 }
 

@@ -1,11 +1,14 @@
 // One decode-attention step of a layer: orchestration of the kernels on one stream, plus the
 // carve-up of the caller's workspace.
 #include "common.h"
+#include "encode_row.h"
 
 namespace pqhsa {
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps, float *qnorm,
-                     float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, hipStream_t stream);
+                     float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words,
+                     const EncodeArgs *append, int kv_dtype, const int32_t *append_count, int32_t *n_after,
+                     hipStream_t stream);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select,
                        uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra,
@@ -15,7 +18,8 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
-                  const float *ref_val, const float *ref_extra, float scale, float *partials, hipStream_t stream);
+                  const float *ref_val, const float *ref_extra, float scale, float *partials,
+                  const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream);
 int emit_tile_keys_for(int64_t n_cap, int streams);
 size_t attend_partials_bytes(int rows);
 
@@ -35,6 +39,7 @@ struct Carve {
     float *topk_val;
     int32_t *topk_cnt;
     float *partials;
+    int32_t *n_after;  // [B] keys per sequence after this step's append
     size_t total;
     int tile_keys;
 };
@@ -70,6 +75,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.topk_val = reinterpret_cast<float *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_cnt = reinterpret_cast<int32_t *>(take(BH * G * 4));
     c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G))));
+    c.n_after = reinterpret_cast<int32_t *>(take((size_t)B * 4));
     c.total = off;
     return c;
 }
@@ -97,11 +103,11 @@ extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace, int32_
     return carve(base, B, H, G, n_cap, num_lists, k_cap).emit_count;
 }
 
-extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
-                                 const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
-                                 int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,
-                                 int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, void *workspace,
-                                 size_t workspace_bytes, void *stream_v) {
+static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                            const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
+                            int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,
+                            int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, void *workspace,
+                            size_t workspace_bytes, const int32_t *append_count, void *stream_v) {
     PQHSA_REQUIRE(q && out && index && seq_lens && select && workspace, "decode_step: NULL argument");
     int rc = validate_view(kv);
     if (rc) return rc;
@@ -129,8 +135,22 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     if (!topk_val) topk_val = c.topk_val;
     if (!topk_cnt) topk_cnt = c.topk_cnt;
 
+    // with an append, the first launch also encodes the new keys and publishes the new counts;
+    // every later kernel of the step reads those, and the last one stores them into the index
+    EncodeArgs enc = {};
+    pqhsa_index after = *index;
+    if (append_count) {
+        PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar && index->pos,
+                      "append_decode_step: the index has no value summaries / position map");
+        rc = fill_encode_args(enc, kv, index, sink, nullptr, nullptr, eps);
+        if (rc) return rc;
+        after.n_idx = c.n_after;
+    }
+    const pqhsa_index *index_in = index;
+    index = &after;
     profile_mark(kProfLut, stream);
-    rc = launch_lut_build(q, q_dtype, index, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words, stream);
+    rc = launch_lut_build(q, q_dtype, index_in, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words,
+                          append_count ? &enc : nullptr, kv->dtype, append_count, c.n_after, stream);
     if (rc) return rc;
     profile_mark(kProfSample, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
@@ -139,5 +159,26 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.mass_extra, c.ref_val, c.ref_extra, scale, c.partials,
-                         stream);
+                         append_count ? c.n_after : nullptr,
+                         append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
+}
+
+extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                                 const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
+                                 int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,
+                                 int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+    return decode_step_impl(q, q_dtype, out, kv, index, G, seq_lens, sink, n_max, full_max, select, scale, eps,
+                            topk_idx, topk_val, topk_cnt, workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int pqhsa_append_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                                        const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
+                                        int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale,
+                                        float eps, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
+                                        void *workspace, size_t workspace_bytes, const int32_t *append_count,
+                                        void *stream) {
+    PQHSA_REQUIRE(append_count != nullptr, "append_decode_step: NULL append_count");
+    return decode_step_impl(q, q_dtype, out, kv, index, G, seq_lens, sink, n_max, full_max, select, scale, eps,
+                            topk_idx, topk_val, topk_cnt, workspace, workspace_bytes, append_count, stream);
 }

@@ -5,28 +5,9 @@
 // argmin keeps the first strict minimum, so list ids and codes are bit-identical to the scalar
 // CPU oracle whichever of the two encode kernels produced them.
 #include "common.h"
+#include "encode_row.h"
 
 namespace pqhsa {
-
-constexpr int kEncThreads = 256;
-constexpr int kCoarseChunk = 32;
-
-struct EncodeArgs {
-    KvView kv;
-    int H, L, sink;
-    const int32_t *slot0;  // [B]
-    const int32_t *count;  // [B]
-    const float *coarse;   // [BH, L, 128]
-    const float *codebooks;
-    float eps;
-    uint32_t *codes;
-    uint16_t *list_ids;
-    float *norms;
-    int32_t *pos;
-    int64_t n_cap;
-    float *vsum, *vcount, *vbar;
-    const int32_t *n_idx;
-};
 
 // One thread per key row; coarse centroids pass through LDS in chunks shared by the block.
 template <int DT>
@@ -125,119 +106,26 @@ __global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) 
     if (a.pos) a.pos[o] = slot;
 }
 
-__device__ inline unsigned long long wave_min_u64(unsigned long long v, int width) {
-    for (int off = width / 2; off > 0; off >>= 1) {
-        const unsigned int lo = (unsigned int)__shfl_xor((int)(v & 0xffffffffull), off, width);
-        const unsigned int hi = (unsigned int)__shfl_xor((int)(v >> 32), off, width);
-        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
-        v = o < v ? o : v;
-    }
-    return v;
-}
-
 // One workgroup per key row: the latency-bound form used for the per-step append.
 template <int DT>
 __global__ __launch_bounds__(kEncThreads) void encode_row_kernel(EncodeArgs a) {
-    __shared__ float xs[kD];
-    __shared__ float nrm_s;
-    __shared__ unsigned long long best_s[kEncThreads / kWave];
-    __shared__ int code_s[kM];
-    const int tid = threadIdx.x;
     const int bh = blockIdx.y;
     const int b = bh / a.H, h = bh % a.H;
     const int j = blockIdx.x;
     if (j >= a.count[b]) return;
-    const int slot = a.slot0[b] + j;
-    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
-    const char *row = a.kv.k_base + row_offset(a.kv, b, h, (int64_t)a.sink + slot) * esz;
-    if (tid < kD) xs[tid] = load1<DT>(row, tid);
-    __syncthreads();
-    if (tid == 0) {
-        float ss = 0.0f;
-        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(xs[d], xs[d], ss);
-        float n = sqrtf(ss);
-        nrm_s = n < a.eps ? a.eps : n;
-    }
-    __syncthreads();
-    if (tid < kD) xs[tid] = xs[tid] / nrm_s;
-    __syncthreads();
-
-    const float *cbase = a.coarse + (size_t)bh * a.L * kD;
-    unsigned long long best = ~0ull;
-    for (int l = tid; l < a.L; l += kEncThreads) {
-        const float4 *c4 = reinterpret_cast<const float4 *>(cbase + (size_t)l * kD);
-        float d2 = 0.0f;
-#pragma unroll 8
-        for (int d4 = 0; d4 < kD / 4; ++d4) {
-            const float4 c = c4[d4];
-            float t;
-            t = xs[4 * d4] - c.x; d2 = __builtin_fmaf(t, t, d2);
-            t = xs[4 * d4 + 1] - c.y; d2 = __builtin_fmaf(t, t, d2);
-            t = xs[4 * d4 + 2] - c.z; d2 = __builtin_fmaf(t, t, d2);
-            t = xs[4 * d4 + 3] - c.w; d2 = __builtin_fmaf(t, t, d2);
-        }
-        // d2 >= 0, so its bit pattern orders like the value; the list id breaks ties low
-        const unsigned long long key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)l;
-        best = key < best ? key : best;
-    }
-    best = wave_min_u64(best, kWave);
-    if ((tid & (kWave - 1)) == 0) best_s[tid / kWave] = best;
-    __syncthreads();
-    best = best_s[0];
-#pragma unroll
-    for (int w = 1; w < kEncThreads / kWave; ++w) best = best_s[w] < best ? best_s[w] : best;
-    const int list = (int)(best & 0xffffffffull);
-    __syncthreads();
-    if (tid < kD) xs[tid] = xs[tid] - cbase[(size_t)list * kD + tid];
-    __syncthreads();
-    if (tid < kM * kCodes) {
-        const int m = tid / kCodes, c = tid % kCodes;
-        const float *w = a.codebooks + ((size_t)bh * kM * kCodes + tid) * kSub;
-        float d2 = 0.0f;
-#pragma unroll
-        for (int e = 0; e < kSub; ++e) {
-            const float t = xs[m * kSub + e] - w[e];
-            d2 = __builtin_fmaf(t, t, d2);
-        }
-        unsigned long long key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)c;
-        key = wave_min_u64(key, kCodes);
-        if (c == 0) code_s[m] = (int)(key & 0xffffffffull);
-    }
-    __syncthreads();
-    if (tid == 0) {
-        uint32_t word = 0;
-#pragma unroll
-        for (int m = 0; m < kM; ++m) word |= (uint32_t)code_s[m] << (4 * m);
-        const size_t o = (size_t)bh * a.n_cap + slot;
-        a.codes[o] = word;
-        a.list_ids[o] = (uint16_t)list;
-        a.norms[o] = nrm_s;
-        if (a.pos) a.pos[o] = slot;
-    }
+    encode_one_row<DT>(a, bh, b, h, a.slot0[b] + j);
 }
 
 // Add the values of freshly encoded rows to their lists, in insertion order, then refresh the
 // touched list means.  One workgroup per stream, one thread per value channel.
 template <int DT>
 __global__ __launch_bounds__(kD) void value_append_kernel(EncodeArgs a) {
-    const int d = threadIdx.x;
     const int bh = blockIdx.x;
     const int b = bh / a.H, h = bh % a.H;
     const int cnt = a.count[b];
     const int s0 = a.slot0[b];
-    const size_t esz = DT == PQHSA_F32 ? 4 : 2;
-    float *vsum = a.vsum + (size_t)bh * a.L * kD;
-    float *vcount = a.vcount + (size_t)bh * a.L;
-    float *vbar = a.vbar + (size_t)bh * a.L * kD;
-    for (int j = 0; j < cnt; ++j) {
-        const int l = a.list_ids[(size_t)bh * a.n_cap + s0 + j];
-        const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + s0 + j) * esz;
-        vsum[(size_t)l * kD + d] += load1<DT>(row, d);
-        __syncthreads();
-        if (d == 0) vcount[l] += 1.0f;
-        __syncthreads();
-        vbar[(size_t)l * kD + d] = vsum[(size_t)l * kD + d] / vcount[l];
-    }
+    for (int j = 0; j < cnt; ++j)
+        value_append_one<DT>(a, bh, b, h, s0 + j, a.list_ids[(size_t)bh * a.n_cap + s0 + j]);
 }
 
 // Rebuild per-list value sums / counts / means.  One workgroup per (stream, 8 lists); every
@@ -304,7 +192,7 @@ __global__ __launch_bounds__(256) void paged_gather_kernel(KvView kv, int seq, i
     reinterpret_cast<uint4 *>(out_v + dst)[lane] = reinterpret_cast<const uint4 *>(kv.v_base + off)[lane];
 }
 
-static int fill_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *index, int sink, const int32_t *slot0,
+int fill_encode_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *index, int sink, const int32_t *slot0,
                      const int32_t *count, float eps) {
     PQHSA_REQUIRE(index != nullptr, "index is NULL");
     int rc = validate_view(kv);
@@ -340,7 +228,7 @@ using namespace pqhsa;
 extern "C" int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink, const int32_t *slot0,
                             const int32_t *count, int32_t count_max, float eps, void *stream) {
     EncodeArgs a = {};
-    int rc = fill_args(a, kv, index, sink, slot0, count, eps);
+    int rc = fill_encode_args(a, kv, index, sink, slot0, count, eps);
     if (rc) return rc;
     PQHSA_REQUIRE(slot0 && count, "encode: NULL slot0/count");
     return launch_encode(a, kv->dtype, index->batch * index->kv_heads, count_max, static_cast<hipStream_t>(stream));
@@ -350,7 +238,7 @@ extern "C" int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *i
                                    const int32_t *slot0, const int32_t *count, int32_t count_max, float eps,
                                    void *stream_v) {
     EncodeArgs a = {};
-    int rc = fill_args(a, kv, index, sink, slot0, count, eps);
+    int rc = fill_encode_args(a, kv, index, sink, slot0, count, eps);
     if (rc) return rc;
     PQHSA_REQUIRE(slot0 && count, "encode_append: NULL slot0/count");
     PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar, "encode_append: index has no value summaries");
@@ -365,7 +253,7 @@ extern "C" int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *i
 extern "C" int pqhsa_value_summaries(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink, int32_t n_max,
                                      void *stream) {
     EncodeArgs a = {};
-    int rc = fill_args(a, kv, index, sink, nullptr, nullptr, 0.0f);
+    int rc = fill_encode_args(a, kv, index, sink, nullptr, nullptr, 0.0f);
     if (rc) return rc;
     PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar && index->n_idx, "value_summaries: NULL arrays");
     (void)n_max;

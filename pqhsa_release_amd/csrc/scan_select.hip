@@ -441,14 +441,14 @@ __device__ inline void find_from_top(const uint32_t *hist, int nbins, uint32_t w
 // One wave per row: exact first-digit threshold from a full histogram (logit-matrix top-k).
 __global__ __launch_bounds__(kWave) void thresh_kernel(const uint32_t *__restrict__ hist,
                                                        const int32_t *__restrict__ n_arr,
-                                                       const int32_t *__restrict__ k_arr,
+                                                       const int32_t *__restrict__ k_arr, int k_cap,
                                                        uint32_t *__restrict__ thr_key, int32_t *__restrict__ k_row,
                                                        float *__restrict__ ref_val) {
     __shared__ uint32_t res[2];
     const int row = blockIdx.x;
     const int lane = threadIdx.x;
     const int n = n_arr[row];
-    const int k = min(max(k_arr[row], 0), n);
+    const int k = min(min(max(k_arr[row], 0), n), k_cap);
     if (lane == 0) {
         res[0] = (uint32_t)kHistBins;  // nothing reaches this bin: keeps no key
         res[1] = 0u;
@@ -554,6 +554,7 @@ struct SampleArgs {
     int L, GP, G;
     double fraction;
     int topk;
+    int k_cap;                 // room of the caller's top-k arrays: k never exceeds it
     uint32_t *thr_key;         // [BH * GP]
     int32_t *k_row;
     float *ref_val;
@@ -602,7 +603,8 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
     for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
     const float qn = a.qnorm[row];
-    const int k = resolve_k(n, a.fraction, a.topk);
+    // (the device-side count may have moved past what the host sized k_cap for: stay inside it)
+    const int k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
     // expected sampled keys among the top max(k, 1), plus the margin
     const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
     const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
@@ -1131,6 +1133,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     sa.n_arr = index->n_idx; sa.ns_arr = index->s_n; sa.n_div = index->kv_heads;
     sa.qnorm = qnorm; sa.lut = lut; sa.list_scores = list_scores; sa.scale = scale;
     sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
+    sa.k_cap = select->k_cap;
     sa.thr_key = thr_key; sa.k_row = k_row; sa.ref_val = ref_val;
     int rc = launch_sample_thresh(sa, streams, stream);
     if (rc) return rc;
@@ -1226,7 +1229,7 @@ extern "C" int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t row
     a.hist = hist;
     rc = launch_scan(a, kHist, kLogits, 1, rows, n_max, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(thresh_kernel, dim3(rows), dim3(kWave), 0, stream, hist, n, k, thr_key, k_row, ref_val);
+    hipLaunchKernelGGL(thresh_kernel, dim3(rows), dim3(kWave), 0, stream, hist, n, k, k_cap, thr_key, k_row, ref_val);
     rc = check_launch("thresh");
     if (rc) return rc;
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count; a.emit_pairs = pairs; a.emit_cap = cap;

@@ -162,7 +162,9 @@ class DeviceIndex:
 
     @classmethod
     def sample_size(cls, n: int) -> int:
-        return min(n, cls.SAMPLE_MAX, max((n + cls.SAMPLE_RATE - 1) // cls.SAMPLE_RATE, cls.SAMPLE_MIN))
+        want = max(n // cls.SAMPLE_RATE, cls.SAMPLE_MIN)
+        want = want // 1024 * 1024  # the threshold kernel holds the sample in registers, 1024 keys per slot
+        return min(n, cls.SAMPLE_MAX, want)
 
     @property
     def n_max(self) -> int:
@@ -177,6 +179,13 @@ class DeviceIndex:
         self.n_sorted_host = [min(s, n) for s, n in zip(self.n_sorted_host, self.n_host)]
         self.n_idx.copy_(torch.tensor(self.n_host, dtype=torch.int32))
         self.n_sorted.copy_(torch.tensor(self.n_sorted_host, dtype=torch.int32))
+
+    def note_appended(self, counts) -> None:
+        """Host-side bookkeeping after a fused append + decode step: the device already holds the
+        new counts (the step stored them), only the host mirror moves."""
+        self.n_host = [n + int(c) for n, c in zip(self.n_host, counts)]
+        if max(self.n_host, default=0) > self.n_cap:
+            raise ValueError("index capacity exceeded")
 
     def reset_layout(self) -> None:
         """Declare the stored keys to be in insertion order again (after a bulk re-encode)."""
@@ -405,29 +414,41 @@ class DecodeCall:
 
     def __init__(self, q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int,
                  full_max: int, fraction: float | None, topk: int, scale: float, workspace: DecodeWorkspace,
-                 eps: float = EPS, n_max: int | None = None) -> None:
+                 eps: float = EPS, n_max: int | None = None, append_count: torch.Tensor | None = None) -> None:
         _need_cuda(q, out, seq_lens)
+        if append_count is not None and (append_count.dtype != torch.int32 or append_count.numel() != index.batch
+                                         or not append_count.is_cuda):
+            raise ValueError("append_count must be a device int32 [B] tensor")
         if tuple(q.shape) != (index.batch, index.kv_heads * groups, HEAD_DIM) or not q.is_contiguous():
             raise ValueError(f"q must be contiguous [B, H*G, {HEAD_DIM}], got {tuple(q.shape)}")
         if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
             raise ValueError("out must match q in shape and dtype")
-        self._fn = _lib.load().pqhsa_decode_step
+        lib = _lib.load()
+        self._fn = lib.pqhsa_decode_step if append_count is None else lib.pqhsa_append_decode_step
+        self._append = () if append_count is None else (append_count.data_ptr(),)
+        self._index = index
         self._sel = Select()
         self._sel.fraction = float(fraction) if fraction else 0.0
         self._sel.topk = int(topk)
         self._sel.k_cap = workspace.k_cap
-        self._keep = (q, out, kv, index, seq_lens, workspace)
+        self._keep = (q, out, kv, index, seq_lens, workspace, append_count)
         self.n_max = index.n_max if n_max is None else int(n_max)
         self.full_max = int(full_max)
-        self._head = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups,
-                      seq_lens.data_ptr(), int(sink))
+        self._head = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups)
+        self._seq_lens = seq_lens.data_ptr()
+        self._sink = int(sink)
         self._tail = (ctypes.byref(self._sel), float(scale), eps, workspace.topk_idx.data_ptr(),
                       workspace.topk_val.data_ptr(), workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(),
                       workspace.bytes)
         self.out = out
 
-    def run(self, stream: int | None = None) -> None:
-        rc = self._fn(*self._head, self.n_max, self.full_max, *self._tail, _stream() if stream is None else stream)
+    def run(self, stream: int | None = None, seq_lens_ptr: int | None = None) -> None:
+        """One step.  With ``append_count`` set at construction this is the fused append + decode
+        step: ``n_max`` must already count the appended key, and the caller records the append in
+        the index's host-side mirror afterwards (``DeviceIndex.note_appended``).  ``seq_lens_ptr``
+        overrides the sequence-length array for this step (an int32 [B] device pointer)."""
+        rc = self._fn(*self._head, self._seq_lens if seq_lens_ptr is None else seq_lens_ptr, self._sink, self.n_max,
+                      self.full_max, *self._tail, *self._append, _stream() if stream is None else stream)
         if rc:
             _lib.check(rc, "pqhsa_decode_step")
 

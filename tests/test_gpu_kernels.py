@@ -407,3 +407,75 @@ def test_decode_step_graph_replays_match_eager_runs():
         assert torch.equal(ws.topk_idx.sort(dim=1).values, want_idx), round_
         np.testing.assert_allclose(out.cpu().numpy(), want_out.cpu().numpy(), atol=1e-5, err_msg=str(round_))
         assert torch.isfinite(junk)
+
+
+def test_fused_append_decode_steps_match_oracle_and_separate_append():
+    """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
+    the launch that builds the tables, attends over the grown index, and leaves the new count in
+    device memory.  Checked against the oracle on the same prefix of the context."""
+    dev = _cuda()
+    steps, len0 = 5, 1800
+    p = Problem(lens=[len0 + steps, len0 + steps - 300], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=47)
+    lens0 = [ln - steps for ln in p.lens]
+    n0 = [p.n(b) - steps for b in range(p.B)]
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    idx = p.device_index(dev, finalize=False)          # every key's codes are there, only the first n0 count
+    idx.set_counts(n0)
+    ops.value_summaries(kv, idx, p.sink)
+    idx.finalize_layout()
+    frac = 0.04
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, frac, 0))
+    q = p.q_tensor().float()
+    out = torch.empty_like(q)
+    one = torch.ones(p.B, dtype=torch.int32, device=dev)
+    seq = torch.tensor(lens0, dtype=torch.int32, device=dev)
+    call = ops.DecodeCall(q, out, kv, idx, p.G, seq, sink=p.sink, full_max=p.sink + p.local, fraction=frac, topk=0,
+                          scale=SCALE, workspace=ws, append_count=one)
+    for t in range(1, steps + 1):
+        seq.add_(1)
+        call.n_max = max(n0) + t
+        call.run()
+        idx.note_appended([1] * p.B)
+        torch.cuda.synchronize()
+        assert idx.n_idx.cpu().tolist() == [n + t for n in n0]          # the step advanced the device-side counts
+        tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        for (b, h), ix in p.index.items():
+            n, ln = n0[b] + t, lens0[b] + t
+            bh = b * p.H + h
+            codes, lists, norms = idx.by_key(bh, n)
+            assert np.array_equal(u32(codes), ix["codes"][:n]) and np.array_equal(u16(lists), ix["list_ids"][:n])
+            assert np.array_equal(norms.cpu().numpy(), ix["norms"][:n])
+            _, _, vbar = fixed.value_summaries(p.values[b, h][p.sink : p.sink + n].numpy(), ix["list_ids"][:n], p.L)
+            np.testing.assert_allclose(idx.vbar[bh].cpu().numpy(), vbar, rtol=1e-6, atol=1e-6)
+            part = {"coarse": ix["coarse"], "codebooks": ix["codebooks"], "codes": ix["codes"][:n],
+                    "list_ids": ix["list_ids"][:n], "norms": ix["norms"][:n], "vbar": vbar}
+            want_out, want_idx, _ = fixed.decode_step(p.queries[b, h].numpy(), p.keys[b, h][:ln].numpy(),
+                                                      p.values[b, h][:ln].numpy(), part, sink=p.sink, local=p.local,
+                                                      fraction=frac, scale=SCALE)
+            for g in range(p.G):
+                assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (t, b, h, g)
+            assert np.abs(o[b, h] - want_out).max() <= 2e-3, (t, b, h)
+    assert idx.tail_max() == steps and ws.rescans() == 0
+
+
+def test_device_counts_ahead_of_the_host_stay_inside_k_cap():
+    """If the device-side key count has moved past what the caller sized k_cap and n_max for (an
+    append the host has not accounted for yet), the step selects k_cap keys instead of reading or
+    writing past the top-k arrays."""
+    dev = _cuda()
+    p = Problem(lens=[3000], heads=1, groups=2, lists=16, seed=53)
+    idx = p.device_index(dev)
+    n = p.n(0)
+    small = n - 400
+    k_cap = ops.resolve_topk(small, 0.05, 0)                 # sized for fewer keys than the device holds
+    assert ops.resolve_topk(n, 0.05, 0) > k_cap
+    ws = ops.DecodeWorkspace(idx, p.G, k_cap)
+    q = p.q_tensor()
+    out = torch.empty_like(q)
+    ops.decode_step(q, out, ops.kv_contiguous(*p.dense_kv()), idx, p.G, p.seq_lens(), sink=p.sink,
+                    full_max=p.sink + p.local, fraction=0.05, topk=0, scale=SCALE, workspace=ws, n_max=small)
+    torch.cuda.synchronize()
+    assert ws.topk_cnt.cpu().tolist() == [k_cap] * p.G
+    got = ws.topk_idx.cpu().numpy()
+    assert ((got >= 0) & (got < n)).all() and bool(torch.isfinite(out).all())
