@@ -7,14 +7,14 @@ namespace pqhsa {
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps, float *qnorm,
                      float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words,
-                     const EncodeArgs *append, int kv_dtype, const int32_t *append_count, int32_t *n_after,
-                     hipStream_t stream);
+                     const AppendFinish *append, int32_t *n_after, unsigned long long *nearest, hipStream_t stream);
+int lut_list_blocks(int num_lists);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select,
                        uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra,
                        void *pairs, uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans,
                        int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
-                       hipStream_t stream);
+                       const AppendFinish *append, hipStream_t stream);
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
@@ -40,6 +40,7 @@ struct Carve {
     int32_t *topk_cnt;
     float *partials;
     int32_t *n_after;  // [B] keys per sequence after this step's append
+    unsigned long long *nearest;  // [BH, list blocks] nearest centroid to the appended key, per list block
     size_t total;
     int tile_keys;
 };
@@ -76,6 +77,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.topk_cnt = reinterpret_cast<int32_t *>(take(BH * G * 4));
     c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G))));
     c.n_after = reinterpret_cast<int32_t *>(take((size_t)B * 4));
+    c.nearest = reinterpret_cast<unsigned long long *>(take(BH * (size_t)lut_list_blocks(L) * 8));
     c.total = off;
     return c;
 }
@@ -137,25 +139,29 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
 
     // with an append, the first launch also encodes the new keys and publishes the new counts;
     // every later kernel of the step reads those, and the last one stores them into the index
-    EncodeArgs enc = {};
+    AppendFinish ap = {};
     pqhsa_index after = *index;
     if (append_count) {
         PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar && index->pos,
                       "append_decode_step: the index has no value summaries / position map");
-        rc = fill_encode_args(enc, kv, index, sink, nullptr, nullptr, eps);
+        rc = fill_encode_args(ap.enc, kv, index, sink, nullptr, nullptr, eps);
         if (rc) return rc;
+        ap.count = append_count;
+        ap.nearest = c.nearest;
+        ap.blocks = lut_list_blocks(index->num_lists);
+        ap.kv_dtype = kv->dtype;
         after.n_idx = c.n_after;
     }
     const pqhsa_index *index_in = index;
     index = &after;
     profile_mark(kProfLut, stream);
     rc = launch_lut_build(q, q_dtype, index_in, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words,
-                          append_count ? &enc : nullptr, kv->dtype, append_count, c.n_after, stream);
+                          append_count ? &ap : nullptr, c.n_after, c.nearest, stream);
     if (rc) return rc;
     profile_mark(kProfSample, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
                             c.k_row, c.ref_val, c.ref_extra, c.pairs, c.aux, c.mass, c.mass_extra, c.rescans,
-                            c.tile_keys, topk_idx, topk_val, topk_cnt, stream);
+                            c.tile_keys, topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.mass_extra, c.ref_val, c.ref_extra, scale, c.partials,

@@ -132,6 +132,112 @@ __device__ inline void value_append_one(const EncodeArgs &a, int bh, int b, int 
     if (d < kD) vbar[(size_t)l * kD + d] = vsum[(size_t)l * kD + d] / vcount[l];
 }
 
+// one element of a row whose element type is only known at run time
+__device__ inline float load1_any(int dtype, const char *row, int d) {
+    if (dtype == PQHSA_F32) return load1<PQHSA_F32>(row, d);
+    if (dtype == PQHSA_BF16) return load1<PQHSA_BF16>(row, d);
+    return load1<PQHSA_F16>(row, d);
+}
+
+// The decode step's fused append is split over two launches so that it adds no latency of its own.
+// First half (inside the table-building launch, whose list blocks hold 64 coarse centroids each
+// in LDS anyway): every list block writes the nearest of ITS centroids to the new key as
+// (distance bits << 32 | list id).  Second half (this function, one extra workgroup per stream in
+// the threshold launch): pick the nearest list over the blocks' answers, PQ-encode the residual,
+// store norm / list id / codes at the end of the stream's keys and add the value row to the
+// list's sum, count and mean.  Same arithmetic as encode_one_row, so the same bits.
+// True when sequence b appends a key in this step and the key fits: there is room in the index
+// and, for a paged cache, its token lies inside the block table.
+__device__ inline bool append_wanted(const EncodeArgs &a, const int32_t *count, int b) {
+    if (count == nullptr || count[b] <= 0) return false;
+    const int64_t slot = a.n_idx[b];
+    if (slot < 0 || slot >= a.n_cap) return false;
+    if (a.kv.paged && (a.sink + slot) / a.kv.block_size >= a.kv.max_blocks) return false;
+    return true;
+}
+
+struct AppendFinish {
+    EncodeArgs enc;
+    const int32_t *count;                // [B] > 0: the sequence appends one key (NULL: no append in this step)
+    const unsigned long long *nearest;   // [BH, blocks]
+    int blocks;
+    int kv_dtype;
+};
+
+__device__ inline void append_finish(const AppendFinish &f, int bh) {
+    __shared__ float xs[kD];
+    __shared__ float nrm_s;
+    __shared__ int list_s;
+    __shared__ int code_s[kM];
+    const EncodeArgs &a = f.enc;
+    const int tid = threadIdx.x;
+    const int b = bh / a.H, h = bh % a.H;
+    if (!append_wanted(a, f.count, b)) return;
+    const int slot = a.n_idx[b];  // the index still holds the count from before this step
+    const size_t esz = f.kv_dtype == PQHSA_F32 ? 4 : 2;
+    const int64_t tok_off = row_offset(a.kv, b, h, (int64_t)a.sink + slot) * (int64_t)esz;
+    float vnew = 0.0f;
+    float4 cw[kSub / 4];
+    if (tid < kD) {
+        xs[tid] = load1_any(f.kv_dtype, a.kv.k_base + tok_off, tid);
+        vnew = load1_any(f.kv_dtype, a.kv.v_base + tok_off, tid);
+        const float4 *w4 = reinterpret_cast<const float4 *>(a.codebooks + ((size_t)bh * kM * kCodes + tid) * kSub);
+#pragma unroll
+        for (int e = 0; e < kSub / 4; ++e) cw[e] = w4[e];
+    }
+    unsigned long long part = ~0ull;
+    if (tid < f.blocks) part = f.nearest[(size_t)bh * f.blocks + tid];
+    part = wave_min_u64(part, kWave);  // at most 64 list blocks
+    __syncthreads();
+    if (tid == 0) {
+        float ss = 0.0f;
+        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(xs[d], xs[d], ss);
+        float n = sqrtf(ss);
+        nrm_s = n < a.eps ? a.eps : n;
+        list_s = min((int)(part & 0xffffffffull), a.L - 1);
+    }
+    __syncthreads();
+    const int list = list_s;
+    float sum = 0.0f, cnt = 1.0f;
+    if (tid < kD) {
+        const float c = a.coarse[((size_t)bh * a.L + list) * kD + tid];
+        sum = a.vsum[((size_t)bh * a.L + list) * kD + tid];
+        cnt = a.vcount[(size_t)bh * a.L + list];
+        xs[tid] = xs[tid] / nrm_s - c;
+    }
+    __syncthreads();
+    if (tid < kM * kCodes) {
+        const int m = tid / kCodes, c = tid % kCodes;
+        const float w[kSub] = {cw[0].x, cw[0].y, cw[0].z, cw[0].w, cw[1].x, cw[1].y, cw[1].z, cw[1].w,
+                               cw[2].x, cw[2].y, cw[2].z, cw[2].w, cw[3].x, cw[3].y, cw[3].z, cw[3].w};
+        float d2 = 0.0f;
+#pragma unroll
+        for (int e = 0; e < kSub; ++e) {
+            const float t = xs[m * kSub + e] - w[e];
+            d2 = __builtin_fmaf(t, t, d2);
+        }
+        unsigned long long key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)c;
+        key = wave_min_u64(key, kCodes);
+        if (c == 0) code_s[m] = (int)(key & 0xffffffffull);
+        // value summaries of the list: every thread has read the old count above
+        sum += vnew;
+        a.vsum[((size_t)bh * a.L + list) * kD + tid] = sum;
+        a.vbar[((size_t)bh * a.L + list) * kD + tid] = sum / (cnt + 1.0f);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int m = 0; m < kM; ++m) word |= (uint32_t)code_s[m] << (4 * m);
+        const size_t o = (size_t)bh * a.n_cap + slot;
+        a.codes[o] = word;
+        a.list_ids[o] = (uint16_t)list;
+        a.norms[o] = nrm_s;
+        if (a.pos) a.pos[o] = slot;
+        a.vcount[(size_t)bh * a.L + list] = cnt + 1.0f;
+    }
+}
+
 int fill_encode_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *index, int sink, const int32_t *slot0,
                      const int32_t *count, float eps);
 

@@ -5,10 +5,10 @@
 // query-to-IVF-centroid dot products.  All reductions are left-to-right fused multiply-add
 // chains so the results are bit-identical to the scalar CPU oracle.
 //
-// A serving step that appends one key per sequence before it attends gives this launch one more
-// block per stream: it encodes the new key (norm, list, PQ codes), adds its value row to the
-// list's sum and mean, and publishes the new key count for the kernels that follow, so the
-// append costs no launch of its own.
+// A serving step that appends one key per sequence before it attends starts the append here:
+// each list block also finds, among the 64 centroids it holds, the one nearest to the new key,
+// and the new key counts are published for the kernels that follow (encode_row.h: append_finish
+// completes the append inside the next launch).
 #include "common.h"
 #include "encode_row.h"
 
@@ -18,12 +18,16 @@ constexpr int kLutThreads = 256;
 constexpr int kListsPerBlock = 64;
 constexpr int kMaxG = 16;
 
-template <int DT, int KDT>
+int lut_list_blocks(int num_lists);
+
+template <int DT>
 __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
     const char *__restrict__ q, int H, int G, int Gp, const float *__restrict__ coarse,
     const float *__restrict__ codebooks, int L, float eps, float *__restrict__ qnorm,
     float *__restrict__ lut, float *__restrict__ list_scores, uint32_t *__restrict__ zero_base,
-    size_t zero_words, EncodeArgs enc, const int32_t *__restrict__ append_count, int32_t *__restrict__ n_after) {
+    size_t zero_words, AppendFinish ap, int32_t *__restrict__ n_after, unsigned long long *__restrict__ nearest) {
+    __shared__ float kx[kD];
+    __shared__ float kn_s;
     __shared__ float qh[kMaxG][kD];
     __shared__ float qn[kMaxG];
     __shared__ float cs[kListsPerBlock][kD + 1];
@@ -34,11 +38,10 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
 
     // list blocks: their 64 x 128 centroid tile (2048 float4, 8 per thread) is requested before
     // anything else, so the loads are all in flight while the query rows are normalised
-    const bool append_block = append_count != nullptr && blockIdx.x == gridDim.x - 1;
     const int l0 = ((int)blockIdx.x - 1) * kListsPerBlock;
-    const int nl = (blockIdx.x == 0 || append_block) ? 0 : min(kListsPerBlock, L - l0);
+    const int nl = blockIdx.x == 0 ? 0 : min(kListsPerBlock, L - l0);
     float4 tile[8];
-    if (blockIdx.x != 0 && !append_block) {
+    if (blockIdx.x != 0) {
         const float4 *c4 = reinterpret_cast<const float4 *>(coarse + ((size_t)bh * L + l0) * kD);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -54,16 +57,13 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         for (size_t i = me; i < zero_words; i += nthreads) zero_base[i] = 0u;
     }
 
-    if (append_block) {
-        // the sequence's new key sits at retrieval-local index n_idx[b], the end of the stored keys
-        const int cnt = append_count[b] > 0 ? 1 : 0;
-        const int slot = enc.n_idx[b];
-        if (h == 0 && tid == 0) n_after[b] = slot + cnt;
-        if (cnt) {
-            const int list = encode_one_row<KDT>(enc, bh, b, h, slot);
-            value_append_one<KDT>(enc, bh, b, h, slot, list);
-        }
-        return;
+    // the sequence's new key (if any) sits at retrieval-local index n_idx[b], the end of the stored keys
+    const bool appending = append_wanted(ap.enc, ap.count, b);
+    if (ap.count != nullptr && blockIdx.x == 0 && h == 0 && tid == 0) n_after[b] = ap.enc.n_idx[b] + (appending ? 1 : 0);
+    if (appending && tid < kD) {
+        const size_t kesz = ap.kv_dtype == PQHSA_F32 ? 4 : 2;
+        const char *krow = ap.enc.kv.k_base + row_offset(ap.enc.kv, b, h, (int64_t)ap.enc.sink + ap.enc.n_idx[b]) * (int64_t)kesz;
+        kx[tid] = load1_any(ap.kv_dtype, krow, tid);
     }
 
     // query rows of this stream: q[b, h*G + g, :]
@@ -80,11 +80,18 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         float n = sqrtf(ss);
         qn[tid] = n < eps ? eps : n;
     }
+    if (appending && tid == kMaxG) {  // one more thread: the new key's norm, same chain as the encode kernels
+        float ss = 0.0f;
+        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(kx[d], kx[d], ss);
+        float n = sqrtf(ss);
+        kn_s = n < ap.enc.eps ? ap.enc.eps : n;
+    }
     __syncthreads();
     for (int i = tid; i < G * kD; i += kLutThreads) {
         int g = i / kD, d = i % kD;
         qh[g][d] = qh[g][d] / qn[g];
     }
+    if (appending && tid < kD) kx[tid] = kx[tid] / kn_s;
     __syncthreads();
 
     if (blockIdx.x == 0) {
@@ -125,48 +132,55 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         }
         out[(size_t)lane * Gp + g] = acc;
     }
+    if (appending && wave == 0) {
+        // nearest of this block's centroids to the new key: squared distance chain as in the encode
+        // kernels; its bit pattern orders like the value (>= 0) and the list id breaks ties low
+        unsigned long long key = ~0ull;
+        if (lane < nl) {
+            float d2 = 0.0f;
+#pragma unroll 8
+            for (int d = 0; d < kD; ++d) {
+                const float t = kx[d] - cs[lane][d];
+                d2 = __builtin_fmaf(t, t, d2);
+            }
+            key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)(l0 + lane);
+        }
+        key = wave_min_u64(key, kWave);
+        if (lane == 0) nearest[(size_t)bh * (gridDim.x - 1) + (blockIdx.x - 1)] = key;
+    }
 }
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps,
                      float *qnorm, float *lut, float *list_scores, uint32_t *zero_base,
-                     size_t zero_words, const EncodeArgs *append, int kv_dtype, const int32_t *append_count,
-                     int32_t *n_after, hipStream_t stream) {
+                     size_t zero_words, const AppendFinish *append, int32_t *n_after,
+                     unsigned long long *nearest, hipStream_t stream) {
     PQHSA_REQUIRE(q && index && qnorm && lut && list_scores, "lut_build: NULL argument");
     PQHSA_REQUIRE(G >= 1 && G <= kMaxG, "lut_build: G=%d outside [1, %d]", G, kMaxG);
     PQHSA_REQUIRE(index->num_lists >= 1 && index->num_lists <= 4096, "lut_build: num_lists=%d", index->num_lists);
     const int BH = index->batch * index->kv_heads;
     if (BH == 0) return PQHSA_OK;
     const int Gp = padded_groups(G);
-    const bool with_append = append != nullptr && append_count != nullptr;
-    PQHSA_REQUIRE(!with_append || n_after != nullptr, "lut_build: the fused append needs the new-count array");
-    dim3 grid(1 + (index->num_lists + kListsPerBlock - 1) / kListsPerBlock + (with_append ? 1 : 0), BH);
-    EncodeArgs enc = {};
-    if (with_append) enc = *append;
-#define PQHSA_LUT(QD, KD)                                                                                      \
-    hipLaunchKernelGGL((lut_build_kernel<QD, KD>), grid, dim3(kLutThreads), 0, stream,                          \
-                       static_cast<const char *>(q), index->kv_heads, G, Gp, index->coarse, index->codebooks,   \
-                       index->num_lists, eps, qnorm, lut, list_scores, zero_base, zero_words, enc,              \
-                       with_append ? append_count : nullptr, n_after)
-    const int kd = with_append ? kv_dtype : PQHSA_F32;  // without an append the key type is not used
-    if (q_dtype == PQHSA_F32 && kd == PQHSA_F32) PQHSA_LUT(PQHSA_F32, PQHSA_F32);
-    else if (q_dtype == PQHSA_F32 && kd == PQHSA_BF16) PQHSA_LUT(PQHSA_F32, PQHSA_BF16);
-    else if (q_dtype == PQHSA_F32 && kd == PQHSA_F16) PQHSA_LUT(PQHSA_F32, PQHSA_F16);
-    else if (q_dtype == PQHSA_BF16 && kd == PQHSA_F32) PQHSA_LUT(PQHSA_BF16, PQHSA_F32);
-    else if (q_dtype == PQHSA_BF16 && kd == PQHSA_BF16) PQHSA_LUT(PQHSA_BF16, PQHSA_BF16);
-    else if (q_dtype == PQHSA_F16 && kd == PQHSA_F32) PQHSA_LUT(PQHSA_F16, PQHSA_F32);
-    else if (q_dtype == PQHSA_F16 && kd == PQHSA_F16) PQHSA_LUT(PQHSA_F16, PQHSA_F16);
-    else {
-        set_error("lut_build: unsupported dtype pair (q %d, kv %d)", q_dtype, kv_dtype);
-        return PQHSA_EINVAL;
+    AppendFinish ap = {};
+    if (append && append->count) {
+        PQHSA_REQUIRE(n_after && nearest, "lut_build: the fused append needs its scratch arrays");
+        ap = *append;
     }
-#undef PQHSA_LUT
+    dim3 grid(1 + lut_list_blocks(index->num_lists), BH);
+    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(lut_build_kernel<DT>, grid, dim3(kLutThreads), 0, stream,
+                                                     static_cast<const char *>(q), index->kv_heads, G, Gp,
+                                                     index->coarse, index->codebooks, index->num_lists, eps,
+                                                     qnorm, lut, list_scores, zero_base, zero_words, ap, n_after,
+                                                     nearest));
     return check_launch("lut_build");
 }
+
+// list blocks of one stream in the table-building launch (each takes 64 coarse lists)
+int lut_list_blocks(int num_lists) { return (num_lists + kListsPerBlock - 1) / kListsPerBlock; }
 
 }  // namespace pqhsa
 
 extern "C" int pqhsa_lut_build(const void *q, int32_t q_dtype, const pqhsa_index *index, int32_t G,
                                float eps, float *qnorm, float *lut, float *list_scores, void *stream) {
-    return pqhsa::launch_lut_build(q, q_dtype, index, G, eps, qnorm, lut, list_scores, nullptr, 0, nullptr, 0,
-                                   nullptr, nullptr, static_cast<hipStream_t>(stream));
+    return pqhsa::launch_lut_build(q, q_dtype, index, G, eps, qnorm, lut, list_scores, nullptr, 0, nullptr, nullptr,
+                                   nullptr, static_cast<hipStream_t>(stream));
 }

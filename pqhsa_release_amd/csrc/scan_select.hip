@@ -21,6 +21,7 @@
 #include <cstdlib>
 
 #include "common.h"
+#include "encode_row.h"
 
 namespace pqhsa {
 
@@ -558,6 +559,7 @@ struct SampleArgs {
     uint32_t *thr_key;         // [BH * GP]
     int32_t *k_row;
     float *ref_val;
+    AppendFinish append;       // count != NULL: one more workgroup per stream completes the step's append
 };
 
 constexpr int kSampleRegsMax = 32;  // sampled keys per thread: at most 32768 per row
@@ -572,6 +574,10 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
     const int bh = blockIdx.y;
+    if (g == a.GP) {  // the extra workgroup of a step that appends: it shares this launch, nothing else
+        append_finish(a.append, bh);
+        return;
+    }
     const size_t row = (size_t)bh * a.GP + g;
     if (g >= a.G) {
         if (tid == 0) {
@@ -1087,7 +1093,7 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
     PQHSA_REQUIRE(a.s_cap <= (int64_t)kSampleRegsMax * kSelThreads, "sample_thresh: at most %d sampled keys per row, got %lld",
                   kSampleRegsMax * kSelThreads, (long long)a.s_cap);
     const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
-    const dim3 grid(a.GP, streams), block(kSelThreads);
+    const dim3 grid(a.GP + (a.append.count ? 1 : 0), streams), block(kSelThreads);
     if (a.s_cap <= 4 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<4>, grid, block, lds, stream, a);
     else if (a.s_cap <= 8 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<8>, grid, block, lds, stream, a);
     else if (a.s_cap <= 16 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<16>, grid, block, lds, stream, a);
@@ -1125,15 +1131,17 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
                        uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra, void *pairs,
                        uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans, int emit_tile_keys,
-                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, hipStream_t stream) {
+                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
+                       hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
-    // 1. threshold per row from the sampled keys
+    // 1. threshold per row from the sampled keys (and, in a step that appends, the rest of the append)
     SampleArgs sa = {};
     sa.codes = index->s_codes; sa.list_ids = index->s_list_ids; sa.norms = index->s_norms; sa.s_cap = index->s_cap;
     sa.n_arr = index->n_idx; sa.ns_arr = index->s_n; sa.n_div = index->kv_heads;
     sa.qnorm = qnorm; sa.lut = lut; sa.list_scores = list_scores; sa.scale = scale;
     sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
     sa.k_cap = select->k_cap;
+    if (append) sa.append = *append;
     sa.thr_key = thr_key; sa.k_row = k_row; sa.ref_val = ref_val;
     int rc = launch_sample_thresh(sa, streams, stream);
     if (rc) return rc;
