@@ -41,6 +41,8 @@ class PQHSAEngine:
         self.indexed_len = [0] * self.B             # tokens visible to the index bookkeeping
         self.pending = [0] * self.B                 # appended since the last index update
         self.deferred_pending = False
+        self._fused_append = False                  # one token was appended; the next forward() encodes it
+        self._append_counts: dict[tuple, torch.Tensor] = {}
         self.seq_lens = torch.zeros(self.B, dtype=torch.int32, device=self.device)
         self._ws: dict[int, ops.DecodeWorkspace] = {}
         self.index_adds = self.index_rebuilds = self.online_codebook_updates = self.deferred_index_updates = 0
@@ -144,6 +146,7 @@ class PQHSAEngine:
         self.indexed_len = list(self.lens)
         self.pending = [0] * self.B
         self.deferred_pending = False
+        self._fused_append = False
         counts = [self.n(b) for b in range(self.B)]
         lists = self._effective_lists() if coarse is None else int(coarse.shape[-2])
         self.index = None
@@ -190,6 +193,17 @@ class PQHSAEngine:
             self.lens[b] += count
             self.pending[b] += count
         self.seq_lens += count
+        if self._fused_append:
+            # a second append before the step that would have carried the first: settle the first now
+            self._fused_append = False
+            self._refresh_index_now()
+            return
+        if (count == 1 and ac.index_update_strategy == "incremental" and ac.index_update_interval == 1
+                and self.index is not None and self.index.n_max > 0):
+            # the usual serving step (one token, then attend): the next forward() appends and attends
+            # in the same launches
+            self._fused_append = True
+            return
         if max(self.pending) >= ac.index_update_interval:
             if ac.index_update_strategy == "deferred":
                 if not self.deferred_pending:
@@ -198,7 +212,14 @@ class PQHSAEngine:
             else:
                 self._refresh_index_now()
 
+    def _settle(self) -> None:
+        """Bring the index up to date if an append is still waiting for the next forward()."""
+        if self._fused_append:
+            self._fused_append = False
+            self._refresh_index_now()
+
     def apply_pending_index_update(self) -> bool:
+        self._settle()
         if not self.deferred_pending:
             return False
         self._refresh_index_now()
@@ -283,10 +304,35 @@ class PQHSAEngine:
         if ws is None or ws.k_cap < k_cap:
             ws = self._ws[groups] = ops.DecodeWorkspace(self.index, groups, k_cap)
         scale = (1.0 / math.sqrt(D)) if ac.scale is None else float(ac.scale)
+        append_count, added = None, None
+        if self._fused_append:
+            self._fused_append = False
+            old = [self.n(b) for b in range(self.B)]
+            self.indexed_len = list(self.lens)
+            self.pending = [0] * self.B
+            added = [self.n(b) - n0 for b, n0 in enumerate(old)]
+            if max(added) > 1 or max(self.n(b) for b in range(self.B)) > self.index.n_cap:
+                # not the one-key case after all (or the index must grow first): the separate path
+                self.indexed_len = [ln - 1 for ln in self.lens]
+                self._refresh_index_now()
+                added = None
+            elif max(added) == 1:
+                key = tuple(added)
+                if key not in self._append_counts:
+                    self._append_counts[key] = torch.tensor(added, dtype=torch.int32, device=self.device)
+                append_count = self._append_counts[key]
+            else:
+                added = None
         full_max = max(self.full_count(b) for b in range(self.B))
+        n_max = self.index.n_max + (1 if append_count is not None else 0)
         ops.decode_step(q, out, self.kv, self.index, groups, self.seq_lens, sink=self.sink, full_max=full_max,
                         fraction=ac.retrieval_top_fraction, topk=ac.retrieval_topk, scale=scale, workspace=ws,
-                        eps=self.index_config.eps)
+                        eps=self.index_config.eps, n_max=n_max, append_count=append_count)
+        if append_count is not None:
+            self.index.note_appended(added)
+            self.index_adds += 1
+            if self.index.tail_max() >= self.resort_tail:
+                self.index.finalize_layout(seed=self.index_config.seed)
         return out
 
     def last_topk(self, groups: int):
@@ -296,6 +342,7 @@ class PQHSAEngine:
 
     # ------------------------------------------------------------------ checkpoint
     def state_dict(self) -> dict[str, object]:
+        self._settle()
         idx = self.index
         state: dict[str, object] = {
             "lens": list(self.lens), "indexed_len": list(self.indexed_len), "pending": list(self.pending),

@@ -381,8 +381,12 @@ class DecodeWorkspace:
 
 def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
                 seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
-                scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None) -> torch.Tensor:
-    """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``."""
+                scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None,
+                append_count: torch.Tensor | None = None) -> torch.Tensor:
+    """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``.
+    With ``append_count`` (device int32 [B]) the step first appends one key to every sequence whose
+    entry is positive (``pqhsa_append_decode_step``): ``n_max`` must count the appended key and the
+    caller calls ``index.note_appended`` afterwards."""
     _need_cuda(q, out, seq_lens)
     lib = _lib.load()
     if tuple(q.shape) != (index.batch, index.kv_heads * groups, HEAD_DIM) or not q.is_contiguous():
@@ -396,10 +400,15 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     sel.topk = int(topk)
     sel.k_cap = workspace.k_cap
     n_max = index.n_max if n_max is None else int(n_max)
-    rc = lib.pqhsa_decode_step(q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups,
-                               seq_lens.data_ptr(), int(sink), n_max, int(full_max), ctypes.byref(sel), float(scale),
-                               eps, workspace.topk_idx.data_ptr(), workspace.topk_val.data_ptr(),
-                               workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(), workspace.bytes, _stream())
+    args = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups, seq_lens.data_ptr(),
+            int(sink), n_max, int(full_max), ctypes.byref(sel), float(scale), eps, workspace.topk_idx.data_ptr(),
+            workspace.topk_val.data_ptr(), workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(), workspace.bytes)
+    if append_count is None:
+        rc = lib.pqhsa_decode_step(*args, _stream())
+    else:
+        if append_count.dtype != torch.int32 or append_count.numel() != index.batch or not append_count.is_cuda:
+            raise ValueError("append_count must be a device int32 [B] tensor")
+        rc = lib.pqhsa_append_decode_step(*args, append_count.data_ptr(), _stream())
     _lib.check(rc, "pqhsa_decode_step")
     return out
 
