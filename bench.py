@@ -79,7 +79,10 @@ def make_stream(ctx, groups, seed, device, dtype):
 class Layer:
     """One layer's resident state: K/V (paged or dense), trained + encoded index, queries."""
 
-    def __init__(self, cfg_id, seed0, device):
+    def __init__(self, cfg_id, seed0, device, room=0):
+        """``room`` > 0 prepares the layer for that many append + decode steps: the cache holds
+        ``room`` more tokens per sequence (already written, as a serving engine writes a token's K/V
+        before attention runs), and each step makes one of them visible."""
         from pqhsa_release_amd import ops
         from pqhsa_release_amd.index.train import train_ivfpq
 
@@ -92,9 +95,10 @@ class Layer:
             self.lens = [ctx] * B
         self.n = [max(SINK, ln - LOCAL) - SINK for ln in self.lens]
         n_max = max(self.n)
-        self.index = ops.DeviceIndex(B, H, LISTS, n_max + 256, device)
+        self.index = ops.DeviceIndex(B, H, LISTS, n_max + room + 256, device)
+        self.room, self.t = room, 0
         if paged:
-            blocks_per = [(ln + BLOCK - 1) // BLOCK for ln in self.lens]
+            blocks_per = [(ln + room + BLOCK - 1) // BLOCK for ln in self.lens]
             total = sum(blocks_per)
             order = torch.randperm(total, generator=gen) if shuffled else torch.arange(total)
             table = torch.zeros(B, max(blocks_per), dtype=torch.int32)
@@ -106,11 +110,12 @@ class Layer:
             self.cache = torch.zeros(2, total, BLOCK, H, 128, dtype=dtype, device=device)
             self.kv = ops.kv_paged(self.cache, self.block_table)
         else:
-            self.keys = torch.zeros(B, H, max(self.lens), 128, dtype=dtype, device=device)
+            self.keys = torch.zeros(B, H, max(self.lens) + room, 128, dtype=dtype, device=device)
             self.values = torch.zeros_like(self.keys)
             self.kv = ops.kv_contiguous(self.keys, self.values)
         q = torch.empty(B, H * G, 128, dtype=dtype, device=device)
-        for b, ln in enumerate(self.lens):
+        for b, ln0 in enumerate(self.lens):
+            ln = ln0 + room
             pos = torch.arange(ln, device=device)
             for h in range(H):
                 k, v, qq = make_stream(ln, G, seed0 + 1000 * b + h, device, dtype)
@@ -134,12 +139,30 @@ class Layer:
         ops.value_summaries(self.kv, self.index, SINK)
         self.index.finalize_layout()
         self.seq_lens = torch.tensor(self.lens, dtype=torch.int32, device=device)
-        k_cap = ops.resolve_topk(n_max, FRACTION, 0)
+        k_cap = ops.resolve_topk(n_max + room, FRACTION, 0)
         self.ws = ops.DecodeWorkspace(self.index, G, k_cap)
         self.call = ops.DecodeCall(self.q, self.out, self.kv, self.index, G, self.seq_lens, sink=SINK,
                                    full_max=SINK + LOCAL, fraction=FRACTION, topk=0, scale=1.0 / math.sqrt(128),
                                    workspace=self.ws)
+        if room:
+            # step t sees lens + t tokens; the key that leaves the local window is appended by the step
+            steps = torch.arange(room + 1, dtype=torch.int32).unsqueeze(1)
+            self.seq_steps = (torch.tensor(self.lens, dtype=torch.int32).unsqueeze(0) + steps).to(device).contiguous()
+            self.ones = torch.ones(B, dtype=torch.int32, device=device)
+            self.append_call = ops.DecodeCall(self.q, self.out, self.kv, self.index, G, self.seq_lens, sink=SINK,
+                                              full_max=SINK + LOCAL, fraction=FRACTION, topk=0,
+                                              scale=1.0 / math.sqrt(128), workspace=self.ws, append_count=self.ones)
         torch.cuda.synchronize()
+
+    def append_step(self, stream):
+        """One serving step: the next token becomes visible, its predecessor that leaves the local
+        window is encoded into the index, then attention runs (one fused call)."""
+        if self.t >= self.room:
+            raise RuntimeError("bench layer: no room left for another append step")
+        self.t += 1
+        self.append_call.n_max = max(self.n) + self.t
+        self.append_call.run(stream, seq_lens_ptr=self.seq_steps[self.t].data_ptr())
+        self.index.note_appended([1] * self.B)
 
     def algorithmic_bytes(self):
         """Bytes each kernel must touch per launch (10 B per indexed key-head, tables, selected and
@@ -185,7 +208,7 @@ def cpu_baseline(layer, seconds=12.0):
             break
     per_stream = (time.perf_counter() - t0) / reps
     got = layer.out[b, h * G : (h + 1) * G].float().cpu()
-    err = float((got - out).abs().max())
+    err = None if layer.t else float((got - out).abs().max())  # after append steps the device result is for a longer context
     streams = sum(1 for _ in range(layer.B * layer.H))
     scale_factor = sum(layer.n) * layer.H / max(n, 1)  # streams weighted by their indexed length
     return {
@@ -209,6 +232,8 @@ def main():
     ap.add_argument("--layers", type=int, default=3, help="distinct resident layers rotated through (defeats cache reuse)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--append", action="store_true",
+                    help="every step appends one key per sequence before it attends (always on for config 4)")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one device copy of this many MiB after the warm-up (a kernel of known HBM "
                          "traffic, the yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
@@ -225,13 +250,20 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     t_setup = time.perf_counter()
-    layers = [Layer(args.config, 100 + 7919 * i, device) for i in range(max(1, args.layers))]
+    appending = args.append or args.config == 4
+    nl = max(1, args.layers)
+    room = (3 * args.steps + 4 * args.warmup + 60 + nl - 1) // nl + 8 if appending else 0
+    layers = [Layer(args.config, 100 + 7919 * i, device, room=room) for i in range(nl)]
     log(f"setup {time.perf_counter() - t_setup:.1f}s: {CONFIGS[args.config][0]}, {len(layers)} resident layers")
     stream = torch.cuda.current_stream().cuda_stream
 
     def run_steps(count, offset=0):
         for i in range(count):
-            layers[(i + offset) % len(layers)].call.run(stream)
+            layer = layers[(i + offset) % len(layers)]
+            if appending:
+                layer.append_step(stream)
+            else:
+                layer.call.run(stream)
 
     run_steps(args.warmup)
     torch.cuda.synchronize()
@@ -275,16 +307,18 @@ def main():
 
     # the same steps replayed from HIP graphs (one per resident layer): what a serving loop that
     # captures its steady state would see
-    for l in layers:
-        l.call.capture()
-    for i in range(args.warmup):
-        layers[i % len(layers)].call.replay()
-    torch.cuda.synchronize()
-    t3 = time.perf_counter()
-    for i in range(args.steps):
-        layers[i % len(layers)].call.replay()
-    torch.cuda.synchronize()
-    ms_graph = (time.perf_counter() - t3) * 1000.0 / args.steps
+    ms_graph = None
+    if not appending:  # (a captured graph has the key count of its capture baked into its launch shapes)
+        for l in layers:
+            l.call.capture()
+        for i in range(args.warmup):
+            layers[i % len(layers)].call.replay()
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        for i in range(args.steps):
+            layers[i % len(layers)].call.replay()
+        torch.cuda.synchronize()
+        ms_graph = (time.perf_counter() - t3) * 1000.0 / args.steps
 
     layer = layers[0]
     ab = layer.algorithmic_bytes()
@@ -337,7 +371,8 @@ def main():
         "kernels": kernels,
         "kernel_sum_us": round(sum(kus.values()), 3),
         "ms_per_step_without_event_log": round(ms_plain, 6),
-        "ms_per_step_graph_replay": round(ms_graph, 6),
+        "ms_per_step_graph_replay": None if ms_graph is None else round(ms_graph, 6),
+        "append_per_step": appending,
         "selection": {"k": math.ceil(layer.n[0] * FRACTION), "rescanned_rows": sum(l.ws.rescans() for l in layers),
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},

@@ -162,8 +162,9 @@ class DeviceIndex:
 
     @classmethod
     def sample_size(cls, n: int) -> int:
-        want = max(n // cls.SAMPLE_RATE, cls.SAMPLE_MIN)
-        want = want // 1024 * 1024  # the threshold kernel holds the sample in registers, 1024 keys per slot
+        # a whole number of 1024-key slots (the threshold kernel holds the sample in registers, one
+        # slot per thread), as close to n / SAMPLE_RATE as that allows
+        want = max((n // cls.SAMPLE_RATE + 512) // 1024 * 1024, cls.SAMPLE_MIN)
         return min(n, cls.SAMPLE_MAX, want)
 
     @property
