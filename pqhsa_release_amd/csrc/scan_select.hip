@@ -278,55 +278,59 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
                 any |= emit_mask[g] != 0u;
             }
             if (__ballot(any) != 0ull) {  // wave-uniform
+                // slot of every candidate inside its wave, per row: prefix sums of the lanes' counts,
+                // two rows to a 32-bit word
+                uint32_t excl[GP], tot[GP];
 #pragma unroll
                 for (int g2 = 0; g2 < GP; g2 += 2) {
                     uint32_t packed = __popc(emit_mask[g2]);
                     if constexpr (GP > 1) packed |= (uint32_t)__popc(emit_mask[g2 + 1 < GP ? g2 + 1 : g2]) << 16;
                     const uint32_t incl = wave_prefix_u32(packed);
                     const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
-                    if (total == 0u) continue;
-                    const uint32_t excl = incl - packed;
+                    const uint32_t ex = incl - packed;
+                    excl[g2] = ex & 0xffffu;
+                    tot[g2] = total & 0xffffu;
+                    if (g2 + 1 < GP) {
+                        excl[g2 + 1 < GP ? g2 + 1 : g2] = ex >> 16;
+                        tot[g2 + 1 < GP ? g2 + 1 : g2] = total >> 16;
+                    }
+                }
+                // A window whose candidates do not fit the row's staging area (a list close to the
+                // query: most of its keys are candidates) writes them straight to memory.  Lane g
+                // reserves the space of row g, so all rows share one round trip to memory.
+                uint32_t direct = 0u, want_res = 0u;
 #pragma unroll
-                    for (int gg = 0; gg < 2; ++gg) {
-                        const int g = g2 + gg;
-                        if (g < GP) {
-                            const uint32_t tot = (total >> (16 * gg)) & 0xffffu;
-                            if (tot == 0u) continue;  // wave-uniform
-                            const size_t srow = ((size_t)wave * GP + g) * cap_w;
-                            if (wcnt[g] != 0u && wcnt[g] + tot > (uint32_t)cap_w) {
-                                // staging area full: the wave moves it to memory (wave-uniform branch)
-                                const uint32_t c = min(wcnt[g], (uint32_t)cap_w);
-                                uint32_t at = 0u;
-                                if (lane == 0) at = atomicAdd(&a.emit_count[(size_t)bh * GP + g], c);
-                                at = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
-                                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                                __builtin_amdgcn_wave_barrier();
-                                const size_t o = ((size_t)bh * GP + g) * a.emit_cap + at;
-                                for (uint32_t i = lane; i < c; i += kWave) {
-                                    a.emit_pairs[o + i] = stage_s[srow + i];
-                                    if (a.emit_aux) a.emit_aux[o + i] = stage_aux[srow + i];
-                                }
-                                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                                __builtin_amdgcn_wave_barrier();
-                                wcnt[g] = 0u;
-                            }
-                            uint32_t slot = wcnt[g] + ((excl >> (16 * gg)) & 0xffffu);
-                            wcnt[g] += tot;
-                            if (emit_mask[g] == 0u) continue;
+                for (int g = 0; g < GP; ++g) {
+                    if (tot[g] != 0u && wcnt[g] + tot[g] > (uint32_t)cap_w) {
+                        direct |= 1u << g;
+                        if (lane == g) want_res = tot[g];
+                    }
+                }
+                uint32_t at = 0u;
+                if (direct != 0u && want_res != 0u) at = atomicAdd(&a.emit_count[(size_t)bh * GP + lane], want_res);
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                if (!((emit_mask[g] >> j) & 1u)) continue;
-                                const uint2 pr = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
-                                if (slot < (uint32_t)cap_w) {
-                                    stage_s[srow + slot] = pr;
-                                    if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
-                                } else {  // staging full: reserve one slot in memory directly
-                                    const uint32_t p = atomicAdd(&a.emit_count[(size_t)bh * GP + g], 1u);
-                                    a.emit_pairs[((size_t)bh * GP + g) * a.emit_cap + p] = pr;
-                                    if (a.emit_aux) a.emit_aux[((size_t)bh * GP + g) * a.emit_cap + p] = (uint16_t)lid[j];
-                                }
-                                ++slot;
-                            }
+                for (int g = 0; g < GP; ++g) {
+                    if (tot[g] == 0u) continue;  // wave-uniform
+                    if ((direct >> g) & 1u) {
+                        const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)at, g);
+                        size_t o = ((size_t)bh * GP + g) * a.emit_cap + first + excl[g];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            if (!((emit_mask[g] >> j) & 1u)) continue;
+                            a.emit_pairs[o] = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
+                            if (a.emit_aux) a.emit_aux[o] = (uint16_t)lid[j];
+                            ++o;
+                        }
+                    } else {
+                        const size_t srow = ((size_t)wave * GP + g) * cap_w;
+                        uint32_t slot = wcnt[g] + excl[g];
+                        wcnt[g] += tot[g];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            if (!((emit_mask[g] >> j) & 1u)) continue;
+                            stage_s[srow + slot] = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
+                            if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
+                            ++slot;
                         }
                     }
                 }
@@ -378,7 +382,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         // one reservation per (workgroup, row); every wave then copies its own staging area out
         if (lane == 0) {
 #pragma unroll
-            for (int g = 0; g < GP; ++g) wcnt_s[wave * GP + g] = min(wcnt[g], (uint32_t)cap_w);
+            for (int g = 0; g < GP; ++g) wcnt_s[wave * GP + g] = wcnt[g];
         }
         __syncthreads();
         if (tid < GP) {
@@ -395,7 +399,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         __syncthreads();
 #pragma unroll
         for (int g = 0; g < GP; ++g) {
-            const uint32_t c = min(wcnt[g], (uint32_t)cap_w);
+            const uint32_t c = wcnt[g];
             const size_t o = ((size_t)bh * GP + g) * a.emit_cap + base_s[wave * GP + g];
             const size_t srow = ((size_t)wave * GP + g) * cap_w;
             for (uint32_t i = lane; i < c; i += kWave) {
