@@ -1039,9 +1039,10 @@ int pick_tile_keys(int64_t n_max, int streams) {
     return (int)keys;
 }
 
-// per-wave, per-row staging capacity of the candidate scan
+// per-wave, per-row staging capacity of the candidate scan; sparse windows are staged, a window
+// that does not fit writes straight to memory, so a small area is enough
 int stage_cap_for(int GP, int tile_keys) {
-    int cap = 512 / GP;
+    int cap = 256 / GP;
     const int wave_keys = tile_keys / kScanWaves;
     if (cap > wave_keys) cap = wave_keys;
     if (cap < 32) cap = 32;
@@ -1118,9 +1119,10 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     return check_launch("select_final");
 }
 
-// Tile of the full scan of a decode step.
+// Tile of the full scan of a decode step: whole 1024-key iterations, sized so that the launch has
+// about four workgroups per compute unit (256 units; PQHSA_EMIT_WGS overrides the target).
 int emit_tile_keys_for(int64_t n_cap, int streams) {
-    static const int target = env_int("PQHSA_EMIT_WGS", 1024);
+    static const int target = env_int("PQHSA_EMIT_WGS", 1280);
     int64_t tiles_per_stream = (target + streams - 1) / (streams > 0 ? streams : 1);
     if (tiles_per_stream < 1) tiles_per_stream = 1;
     int64_t keys = (n_cap + tiles_per_stream - 1) / tiles_per_stream;
