@@ -104,8 +104,8 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     __shared__ float red[kGroups][kD];
     __shared__ float red_m[kGroups];
     __shared__ float red_l[kGroups];
-    __shared__ float bg_s[2][2][kD];
-    __shared__ float ms_s[2][kAttThreads / kWave];
+    __shared__ __align__(16) float bg_s[2][kAttThreads / (kD / 4)][kD];
+    __shared__ float ms_s[2][kAttThreads / (kD / 4)];
     const int tid = threadIdx.x;
     const int split = blockIdx.x, g = blockIdx.y, bh = blockIdx.z;
     const int b = bh / a.H, h = bh % a.H;
@@ -123,6 +123,37 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int cnt = end - start;
     float *part = a.partials + (orow * a.splits + split) * kPartWidth;
 
+    // ---- background slice: lists [l_lo, l_hi) -------------------------------------------
+    // 32 lanes cover one list mean (four elements each), eight lists per pass.  The first passes
+    // are requested here, before anything depends on memory, and used only after the first K/V
+    // rows have been requested, so that neither waits for the other.
+    constexpr int kBgLanes = kD / 4;
+    constexpr int kBgRows = kAttThreads / kBgLanes;
+    constexpr int kBgU = 8;
+    const int per = (a.L + a.splits - 1) / a.splits;
+    const int l_lo = min(split * per, a.L), l_hi = n > 0 ? min(l_lo + per, a.L) : l_lo;
+    const int bl = tid / kBgLanes, bd = (tid % kBgLanes) * 4;
+    const float *vb = a.vbar + (size_t)bh * a.L * kD;
+    const float *m0 = a.mass0 ? a.mass0 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
+    const float *m1 = a.mass1 ? a.mass1 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
+    float4 bv[kBgU];
+    float bw0[kBgU], bw1[kBgU];
+    auto bg_fetch = [&](int first) {
+#pragma unroll
+        for (int u = 0; u < kBgU; ++u) {
+            const int l = first + bl + u * kBgRows;
+            bv[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            bw0[u] = 0.0f;
+            bw1[u] = 0.0f;
+            if (l < l_hi) {
+                bv[u] = *reinterpret_cast<const float4 *>(vb + (size_t)l * kD + bd);
+                if (m0) bw0[u] = m0[(size_t)l * a.mass_l];
+                if (m1) bw1[u] = m1[(size_t)l * a.mass_l];
+            }
+        }
+    };
+    bg_fetch(l_lo);
+
     // ---- row addresses of this chunk (block-table lookups happen here, once) ---------------
     int64_t *off_s = reinterpret_cast<int64_t *>(smem);  // [chunk] element offsets of the rows
     {
@@ -136,49 +167,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
             off_s[i] = row_offset(a.kv, b, h, pos);
         }
     }
-
-    // ---- background slice: lists [l_lo, l_hi) -------------------------------------------
-    {
-        const int per = (a.L + a.splits - 1) / a.splits;
-        const int l_lo = min(split * per, a.L), l_hi = min(l_lo + per, a.L);
-        const int d = tid & (kD - 1);
-        const int half = tid / kD;
-        const float *vb = a.vbar + (size_t)bh * a.L * kD;
-        const float *m0 = a.mass0 ? a.mass0 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
-        const float *m1 = a.mass1 ? a.mass1 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
-        float bg0 = 0.0f, bg1 = 0.0f, s0 = 0.0f, s1 = 0.0f;
-        if (n > 0) {
-#pragma unroll 8
-            for (int l = l_lo + half; l < l_hi; l += 2) {
-                const float v = vb[(size_t)l * kD + d];
-                const float w0 = m0 ? m0[(size_t)l * a.mass_l] : 0.0f;
-                const float w1 = m1 ? m1[(size_t)l * a.mass_l] : 0.0f;
-                bg0 = __builtin_fmaf(w0, v, bg0);
-                bg1 = __builtin_fmaf(w1, v, bg1);
-                if (d == 0) { s0 += w0; s1 += w1; }
-            }
-        }
-        bg_s[0][half][d] = bg0;
-        bg_s[1][half][d] = bg1;
-        s0 = wave_sum(s0);
-        s1 = wave_sum(s1);
-        if ((tid & (kWave - 1)) == 0) { ms_s[0][tid / kWave] = s0; ms_s[1][tid / kWave] = s1; }
-        __syncthreads();  // also publishes off_s
-        if (tid < kD) {
-            part[4 + kD + tid] = bg_s[0][0][tid] + bg_s[0][1][tid];
-            part[4 + 2 * kD + tid] = bg_s[1][0][tid] + bg_s[1][1][tid];
-        }
-        if (tid == 0) {
-            part[2] = ms_s[0][0] + ms_s[0][1] + ms_s[0][2] + ms_s[0][3];
-            part[3] = ms_s[1][0] + ms_s[1][1] + ms_s[1][2] + ms_s[1][3];
-        }
-    }
-
-    if (cnt <= 0) {
-        if (tid == 0) { part[0] = -INFINITY; part[1] = 0.0f; }
-        if (tid < kD) part[4 + tid] = 0.0f;
-        return;
-    }
+    __syncthreads();
 
     // ---- exact rows: K and V of a row travel together, softmax kept online per row group -----
     // Each group of 16 lanes owns rows grp, grp + 16, ...; U rows per batch, and the loads of the
@@ -196,20 +185,65 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     using Raw = RawSlice<KDT>;
     const int my_rows = cnt > grp ? (cnt - grp + kGroups - 1) / kGroups : 0;
     const int batches = (my_rows + U - 1) / U;
-    auto fetch = [&](Raw (&kb)[U], Raw (&vb)[U], int t) {
+    auto fetch = [&](Raw (&kb)[U], Raw (&vb_)[U], int t) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ii = grp + kGroups * (t * U + u);
             if (ii < cnt) {
                 const int64_t off = off_s[ii] * (int64_t)kesz;
                 kb[u].load(a.kv.k_base + off, lane16);
-                vb[u].load(a.kv.v_base + off, lane16);
+                vb_[u].load(a.kv.v_base + off, lane16);
             } else {
                 kb[u].zero();
-                vb[u].zero();
+                vb_[u].zero();
             }
         }
     };
+    Raw k0[U], v0[U], k1[U], v1[U];
+    if (batches > 0) fetch(k0, v0, 0);
+
+    // ---- background arithmetic, while the first K/V rows are on their way ---------------------
+    {
+        float4 b0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), b1 = b0;
+        float s0 = 0.0f, s1 = 0.0f;
+        for (int first = l_lo; first < l_hi; first += kBgU * kBgRows) {
+            if (first != l_lo) bg_fetch(first);
+#pragma unroll
+            for (int u = 0; u < kBgU; ++u) {
+                b0.x = __builtin_fmaf(bw0[u], bv[u].x, b0.x); b0.y = __builtin_fmaf(bw0[u], bv[u].y, b0.y);
+                b0.z = __builtin_fmaf(bw0[u], bv[u].z, b0.z); b0.w = __builtin_fmaf(bw0[u], bv[u].w, b0.w);
+                b1.x = __builtin_fmaf(bw1[u], bv[u].x, b1.x); b1.y = __builtin_fmaf(bw1[u], bv[u].y, b1.y);
+                b1.z = __builtin_fmaf(bw1[u], bv[u].z, b1.z); b1.w = __builtin_fmaf(bw1[u], bv[u].w, b1.w);
+                s0 += bw0[u];
+                s1 += bw1[u];
+            }
+        }
+        *reinterpret_cast<float4 *>(&bg_s[0][bl][bd]) = b0;
+        *reinterpret_cast<float4 *>(&bg_s[1][bl][bd]) = b1;
+        if (bd == 0) { ms_s[0][bl] = s0; ms_s[1][bl] = s1; }
+        __syncthreads();
+        if (tid < kD) {
+            float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < kBgRows; ++r) { t0 += bg_s[0][r][tid]; t1 += bg_s[1][r][tid]; }
+            part[4 + kD + tid] = t0;
+            part[4 + 2 * kD + tid] = t1;
+        }
+        if (tid == 0) {
+            float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < kBgRows; ++r) { t0 += ms_s[0][r]; t1 += ms_s[1][r]; }
+            part[2] = t0;
+            part[3] = t1;
+        }
+    }
+
+    if (cnt <= 0) {
+        if (tid == 0) { part[0] = -INFINITY; part[1] = 0.0f; }
+        if (tid < kD) part[4 + tid] = 0.0f;
+        return;
+    }
+
     float m_g = -INFINITY, l_g = 0.0f;
     float acc[8];
 #pragma unroll
@@ -246,8 +280,6 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         m_g = m_new;
     };
     {
-        Raw k0[U], v0[U], k1[U], v1[U];
-        if (batches > 0) fetch(k0, v0, 0);
         for (int t = 0; t < batches; t += 2) {
             if (t + 1 < batches) fetch(k1, v1, t + 1);
             consume(k0, v0, t);
