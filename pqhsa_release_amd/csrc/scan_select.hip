@@ -494,12 +494,15 @@ __device__ inline uint32_t wave_count_if(bool pred) { return (uint32_t)__popcll(
 // want-th largest key); padding keys are 0 and never counted (T >= 1).  Stops early at a prefix T
 // whose count is within [want, want + slack]; `exact` is set when that count is exactly want:
 // then {key >= T} is the answer set.
+// The search starts from prefix t0 at bit bit0: the caller knows that every key that counts has
+// t0's bits above bit0 (t0 = 0, bit0 = 31: nothing known).
 template <int R>
 __device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, uint32_t slack,
-                                       uint32_t (*red)[kSelWaves], int &step, bool &exact) {
-    uint32_t t = 0u;
+                                       uint32_t (*red)[kSelWaves], int &step, bool &exact, uint32_t t0 = 0u,
+                                       int bit0 = 31) {
+    uint32_t t = t0;
     exact = false;
-    for (int bit = 31; bit >= 0; --bit) {
+    for (int bit = bit0; bit >= 0; --bit) {
         const uint32_t trial = t | (1u << bit);
         uint32_t c = 0;
 #pragma unroll
@@ -514,6 +517,38 @@ __device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, 
         }
     }
     return t;
+}
+
+// The leading bits that all keys of the workgroup share, keys equal to PAD aside: returns the
+// shared prefix and, in bit0, the highest bit in which two keys differ (-1: all equal, or none).
+// One barrier; `span` holds 2 * kSelWaves words that nothing else uses until the next barrier.
+template <uint32_t PAD, int R>
+__device__ inline uint32_t shared_prefix(const uint32_t (&key)[R], uint32_t *span, int &bit0) {
+    uint32_t hi = 0u, lo = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        hi = max(hi, key[r] != PAD ? key[r] : 0u);
+        lo = min(lo, key[r] != PAD ? key[r] : 0xffffffffu);
+    }
+    hi = wave_max_u32(hi);
+    lo = ~wave_max_u32(~lo);
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        span[threadIdx.x / kWave] = hi;
+        span[kSelWaves + threadIdx.x / kWave] = lo;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) {
+        hi = max(hi, span[w]);
+        lo = min(lo, span[kSelWaves + w]);
+    }
+    if (lo >= hi) {  // all equal, or no keys at all
+        bit0 = -1;
+        return hi;
+    }
+    bit0 = 31 - __clz(hi ^ lo);
+    return bit0 == 31 ? 0u : hi & ~((2u << bit0) - 1u);
 }
 
 // The same search over keys in memory (any count).
@@ -727,7 +762,11 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
     bool exact = false;
     uint32_t tkey = 0u;
     if (k > 0) {
-        tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact);
+        // candidates all lie between the threshold and the row maximum: their keys share the leading
+        // bits, which the search need not visit
+        int bit0;
+        const uint32_t t0 = shared_prefix<0u>(key, wsum, bit0);
+        tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact, t0, bit0);
     } else {  // nothing is selected: the reference of the losers' weights is the largest key
         uint32_t kmax = 0u;
 #pragma unroll
@@ -758,8 +797,9 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 tidx[r] = key[r] == tkey ? (pos_row ? (uint32_t)pos_row[where[r]] : where[r]) : 0xffffffffu;
-            uint32_t lo = 0u;
-            for (int bit = 31; bit >= 0; --bit) {
+            int bit1;
+            uint32_t lo = shared_prefix<0xffffffffu>(tidx, wsum, bit1);  // the tied indices' common leading bits
+            for (int bit = bit1; bit >= 0; --bit) {
                 const uint32_t trial = lo | (1u << bit);
                 uint32_t c = 0;
 #pragma unroll
@@ -889,7 +929,7 @@ template <int RS>
 __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
-    __shared__ uint32_t wsum[kSelWaves];
+    __shared__ uint32_t wsum[2 * kSelWaves];
     float *mx = reinterpret_cast<float *>(smem);  // [L] (the re-scan parks its [128 + L] tables here first)
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
