@@ -819,15 +819,29 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
 #pragma unroll
     for (int r = 0; r < R; ++r) mine += (k > 0 && key[r] >= tkey) ? 1u : 0u;
     uint32_t at = block_exclusive_u32(mine, wsum);
+    const int lane = tid & (kWave - 1);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const uint32_t p = (uint32_t)r * kSelThreads + tid;
-        if (p >= cnt) continue;
-        if (k > 0 && key[r] >= tkey) {
-            out.winner(at++, key[r], where[r]);
-        } else {
+        const bool real = p < cnt;
+        const bool wins = real && k > 0 && key[r] >= tkey;
+        if (wins) out.winner(at++, key[r], where[r]);
+        if (out.mx) {
+            // Losers return their weight to their list.  Candidates arrive in runs of equal list
+            // (the scan emits them in stored order), so the lanes of a wave add one sum per run:
+            // the run's last lane adds its prefix sum, the first takes back the prefix before it.
             const bool tie_loser = ties && (where[r] & 0x80000000u);
-            out.loser(tie_loser ? tkey : key[r], list[r]);
+            const float w = (real && !wins) ? __expf(key_to_float(tie_loser ? tkey : key[r]) - out.ref1) : 0.0f;
+            const int l = (int)list[r];
+            const int prev = dpp_move<kDppWaveShr1>(l);
+            const int next = dpp_move<kDppWaveShl1>(l);
+            const bool is_start = lane == 0 || prev != l;
+            const bool is_end = lane == kWave - 1 || next != l;
+            const float pre = wave_prefix_f32(w);
+            if (is_start || is_end) {
+                const float add = is_start ? (is_end ? w : w - pre) : pre;
+                if (add != 0.0f) atomicAdd(&out.mx[l], add);
+            }
         }
     }
 }
