@@ -63,7 +63,7 @@ struct ScanArgs {
     const uint32_t *thr_key;  // [rows] keys at or above it are candidates
     const float *ref_val;     // [rows] reference logit of the background sums
     uint32_t *emit_count;     // [rows]
-    uint2 *emit_pairs;        // [rows, emit_cap] (key, stored position)
+    uint2 *emit_pairs;        // [rows, emit_cap] (key, retrieval-local index)
     uint16_t *emit_aux;       // [rows, emit_cap] list id of the candidate (NULL: none)
     int64_t emit_cap;
     float *mass;              // [BH, L, GP] accumulated with atomics (NULL: none)
@@ -176,6 +176,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     for (int i0 = tile0 + tid * kKeysPerThread; i0 - lane * kKeysPerThread < tile_end; i0 += kKeysPerIter) {
         float s[kKeysPerThread][GP];
         uint32_t lid[kKeysPerThread];
+        uint32_t ridx[kKeysPerThread] = {(uint32_t)i0, (uint32_t)i0 + 1u, (uint32_t)i0 + 2u, (uint32_t)i0 + 3u};
         const bool in_range = i0 < tile_end;
         if constexpr (SRC == kIndex) {
             uint4 cw = make_uint4(0, 0, 0, 0);
@@ -185,6 +186,12 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
                 cw = *reinterpret_cast<const uint4 *>(a.codes + base + i0);
                 lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + i0);
                 nw = *reinterpret_cast<const float4 *>(a.norms + base + i0);
+                if constexpr (MODE == kEmit) {  // candidates are recorded under their retrieval-local index
+                    if (a.pos) {
+                        const int4 pw = *reinterpret_cast<const int4 *>(a.pos + base + i0);
+                        ridx[0] = (uint32_t)pw.x; ridx[1] = (uint32_t)pw.y; ridx[2] = (uint32_t)pw.z; ridx[3] = (uint32_t)pw.w;
+                    }
+                }
             }
             const uint32_t c[4] = {cw.x, cw.y, cw.z, cw.w};
             const float kn[4] = {nw.x, nw.y, nw.z, nw.w};
@@ -317,7 +324,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             if (!((emit_mask[g] >> j) & 1u)) continue;
-                            a.emit_pairs[o] = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
+                            a.emit_pairs[o] = make_uint2(order_key(s[j][g]), ridx[j]);
                             if (a.emit_aux) a.emit_aux[o] = (uint16_t)lid[j];
                             ++o;
                         }
@@ -328,7 +335,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             if (!((emit_mask[g] >> j) & 1u)) continue;
-                            stage_s[srow + slot] = make_uint2(order_key(s[j][g]), (uint32_t)(i0 + j));
+                            stage_s[srow + slot] = make_uint2(order_key(s[j][g]), ridx[j]);
                             if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
                             ++slot;
                         }
@@ -689,7 +696,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
 
 // ---- exact selection among the candidates -----------------------------------------------
 struct SelectArgs {
-    uint2 *pairs;          // [rows, emit_cap] (key, stored position)
+    uint2 *pairs;          // [rows, emit_cap] (key, retrieval-local index)
     uint16_t *aux;         // [rows, emit_cap] list ids (NULL: none)
     int64_t emit_cap;
     uint32_t *emit_count;  // [rows]
@@ -737,12 +744,11 @@ struct SelectOut {
     int32_t *out_idx;
     float *out_val;
     uint32_t k_cap;
-    const int32_t *pos_row;  // NULL: identity
     float *mx;               // LDS [L] (NULL: no background)
     float ref1;
     __device__ inline void winner(uint32_t at, uint32_t key, uint32_t where) const {
         if (at < k_cap) {
-            out_idx[at] = pos_row ? pos_row[where] : (int32_t)where;
+            out_idx[at] = (int32_t)where;
             if (out_val) out_val[at] = key_to_float(key);
         }
     }
@@ -755,7 +761,7 @@ struct SelectOut {
 // tid; slots at or past cnt hold key 0.
 template <int R>
 __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
-                                     int k, const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                     int k, SelectOut out, uint32_t (*red)[kSelWaves],
                                      uint32_t *wsum, float *ref1_out) {
     const int tid = threadIdx.x;
     int step = 0;
@@ -796,7 +802,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
             uint32_t tidx[R];
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                tidx[r] = key[r] == tkey ? (pos_row ? (uint32_t)pos_row[where[r]] : where[r]) : 0xffffffffu;
+                tidx[r] = key[r] == tkey ? where[r] : 0xffffffffu;
             int bit1;
             uint32_t lo = shared_prefix<0xffffffffu>(tidx, wsum, bit1);  // the tied indices' common leading bits
             for (int bit = bit1; bit >= 0; --bit) {
@@ -848,7 +854,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
 
 template <int R>
 __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
-                                   const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                   SelectOut out, uint32_t (*red)[kSelWaves],
                                    uint32_t *wsum, float *ref1_out) {
     uint32_t key[R], where[R], list[R];
 #pragma unroll
@@ -859,17 +865,16 @@ __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, cons
         where[r] = pr.y;
         list[r] = (aux && p < cnt) ? aux[p] : 0u;
     }
-    select_loaded<R>(key, where, list, cnt, k, pos_row, out, red, wsum, ref1_out);
+    select_loaded<R>(key, where, list, cnt, k, out, red, wsum, ref1_out);
 }
 
 // Candidates in memory (any count): the same selection, streaming the pairs on every pass.
 __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
-                                  const int32_t *pos_row, SelectOut out, uint32_t (*red)[kSelWaves],
+                                  SelectOut out, uint32_t (*red)[kSelWaves],
                                   uint32_t *wsum, float *ref1_out) {
     const int tid = threadIdx.x;
     const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
     auto key_at = [=](uint32_t p) { return pairs[p].x; };
-    auto index_of = [=](uint32_t where) { return pos_row ? (uint32_t)pos_row[where] : where; };
     int step = 0;
     bool exact = false;
     uint32_t tkey = 0u;
@@ -907,7 +912,7 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
                     bool hit = false;
                     if (p < cnt) {
                         const uint2 pr = pairs[p];
-                        hit = pr.x == tkey && index_of(pr.y) < trial;
+                        hit = pr.x == tkey && pr.y < trial;
                     }
                     c += wave_count_if(hit);
                 }
@@ -920,7 +925,7 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
     auto selected = [=](uint2 pr) {
         if (k <= 0) return false;
         if (pr.x != tkey || idx_thr == 0xffffffffu) return pr.x >= tkey;
-        return index_of(pr.y) <= idx_thr;
+        return pr.y <= idx_thr;
     };
     out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
     *ref1_out = out.ref1;
@@ -954,7 +959,6 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     const int k = a.k_row[row];
     uint2 *pairs = a.pairs + row * a.emit_cap;
     uint16_t *aux = a.aux ? a.aux + row * a.emit_cap : nullptr;
-    const int32_t *pos_row = a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr;
     constexpr int RA = RS > 0 ? RS : 1;
     uint32_t skey[RA], swhere[RA], slist[RA];
     if constexpr (RS > 0) {
@@ -990,7 +994,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             uint32_t lid = a.list_ids[base + p];
             if (lid >= (uint32_t)a.L) lid = 0u;
             const float s = score_one(lut_s, ls_s, a.codes[base + p], lid, qn, a.norms[base + p], a.scale);
-            pairs[p] = make_uint2(order_key(s), (uint32_t)p);
+            pairs[p] = make_uint2(order_key(s), a.pos ? (uint32_t)a.pos[base + p] : (uint32_t)p);
             if (aux) aux[p] = (uint16_t)lid;
         }
         cnt = (uint32_t)n;
@@ -1005,7 +1009,6 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     out.out_idx = a.topk_idx + orow * a.k_cap;
     out.out_val = a.topk_val ? a.topk_val + orow * a.k_cap : nullptr;
     out.k_cap = (uint32_t)a.k_cap;
-    out.pos_row = pos_row;
     out.mx = mass_out ? mx : nullptr;
     out.ref1 = 0.0f;
     float ref1;
@@ -1016,18 +1019,18 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             for (int r = 0; r < RS; ++r) {
                 if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, swhere[r] = 0u, slist[r] = 0u;
             }
-            select_loaded<RS>(skey, swhere, slist, cnt, k, pos_row, out, red, wsum, &ref1);
+            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ref1);
             done = true;
         }
     }
     if (!done) {
         if constexpr (RS == 0) {  // no estimate: pick the register variant from the count
-            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
-            else select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, out, red, wsum, &ref1);
+            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, out, red, wsum, &ref1);
+            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, out, red, wsum, &ref1);
+            else select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
         } else {  // the estimate was exceeded, or the row was re-scanned (rare): stream from memory
-            select_mem(a, cnt, k, pairs, aux, pos_row, out, red, wsum, &ref1);
+            select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
         }
     }
     __syncthreads();
