@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     // rows have been requested, so that neither waits for the other.
     constexpr int kBgLanes = kD / 4;
     constexpr int kBgRows = kAttThreads / kBgLanes;
-    constexpr int kBgU = 8;
+    constexpr int kBgU = 4;
     const int per = (a.L + a.splits - 1) / a.splits;
     const int l_lo = min(split * per, a.L), l_hi = n > 0 ? min(l_lo + per, a.L) : l_lo;
     const int bl = tid / kBgLanes, bd = (tid % kBgLanes) * 4;
@@ -201,6 +201,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     };
     Raw k0[U], v0[U], k1[U], v1[U];
     if (batches > 0) fetch(k0, v0, 0);
+    if (batches > 1) fetch(k1, v1, 1);
 
     // ---- background arithmetic, while the first K/V rows are on their way ---------------------
     {
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     };
     {
         for (int t = 0; t < batches; t += 2) {
-            if (t + 1 < batches) fetch(k1, v1, t + 1);
+            if (t > 0 && t + 1 < batches) fetch(k1, v1, t + 1);  // batch 1 is already on its way
             consume(k0, v0, t);
             if (t + 1 < batches) {
                 if (t + 2 < batches) fetch(k0, v0, t + 2);
