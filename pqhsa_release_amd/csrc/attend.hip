@@ -388,7 +388,9 @@ __global__ __launch_bounds__(kAttThreads) void subtract_selected_kernel(const fl
 int pick_splits(int streams_rows, int rows_max) {
     static const int target = getenv("PQHSA_ATT_WGS") ? atoi(getenv("PQHSA_ATT_WGS")) : 1024;
     int s = (target + streams_rows - 1) / (streams_rows > 0 ? streams_rows : 1);
-    const int need = (rows_max + kMaxChunk - 1) / kMaxChunk;
+    // chunks of at most 384 rows: short enough that a ragged batch (rows of very different
+    // lengths) still spreads evenly over the compute units
+    const int need = (rows_max + 383) / 384;
     if (s < need) s = need;
     if (s < 1) s = 1;
     if (s > kMaxSplits) s = kMaxSplits;

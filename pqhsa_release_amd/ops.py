@@ -131,7 +131,7 @@ class DeviceIndex:
     """
 
     SAMPLE_RATE = 32
-    SAMPLE_MIN = 1024
+    SAMPLE_MIN = 4096
     SAMPLE_MAX = 32768   # the threshold kernel keeps the sampled keys of one row in LDS
 
     def __init__(self, batch: int, kv_heads: int, num_lists: int, n_cap: int, device) -> None:

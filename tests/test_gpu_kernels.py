@@ -257,7 +257,7 @@ def test_decode_step_rescans_rows_when_the_sampled_threshold_keeps_too_few():
     keeps fewer than k candidates, is re-scored in full by its selection workgroup, and the
     result is still the exact top-k with the right background."""
     dev = _cuda()
-    p = Problem(lens=[6000], heads=1, groups=2, lists=32, seed=29)
+    p = Problem(lens=[20000], heads=1, groups=2, lists=32, seed=29)
     idx = p.device_index(dev)
     _, _, logits = p.oracle_step(0, 0, 0.02)
     ns = int(idx.s_n[0])
