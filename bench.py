@@ -178,6 +178,22 @@ class Layer:
                 "total": scan + tables + exact + full + bg}
 
 
+def copy_bandwidth(device, mib=1024, reps=10):
+    """HBM bandwidth a plain device-to-device copy reaches on this box (bytes read + written per
+    second), the practical ceiling the roofline fraction can also be read against."""
+    src = torch.empty(mib * 262144, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * src.numel() * 4 * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+
 def cpu_baseline(layer, seconds=12.0):
     """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
     the same inputs and trained index, and scale to the whole layer."""
@@ -207,6 +223,15 @@ def cpu_baseline(layer, seconds=12.0):
         if time.perf_counter() - t0 > seconds and reps >= 3:
             break
     per_stream = (time.perf_counter() - t0) / reps
+    torch.set_num_threads(1)  # the same sample on one core, for a quarter of the time budget
+    t1, reps1 = time.perf_counter(), 0
+    while True:
+        tr.hybrid_forward_many(q, keys, values, **args)
+        reps1 += 1
+        if time.perf_counter() - t1 > seconds / 4 and reps1 >= 2:
+            break
+    per_stream_1 = (time.perf_counter() - t1) / reps1
+    torch.set_num_threads(cores)
     got = layer.out[b, h * G : (h + 1) * G].float().cpu()
     err = None if layer.t else float((got - out).abs().max())  # after append steps the device result is for a longer context
     streams = sum(1 for _ in range(layer.B * layer.H))
@@ -218,6 +243,7 @@ def cpu_baseline(layer, seconds=12.0):
         "kind": "port",
         "sample": f"torch-CPU restatement of forward_many on 1 of {streams} (sequence, KV head) streams "
                   f"(n={n}, G={G}), {reps} reps, scaled by indexed keys to the whole layer",
+        "single_core_value": per_stream_1 * scale_factor * 1e6,
         "max_abs_diff_vs_gpu": err,
         "gpu_out_dtype": str(layer.out.dtype).replace("torch.", ""),  # a bf16 output carries 2^-9 relative rounding
     }
@@ -377,6 +403,9 @@ def main():
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},
     }
+    copy_gbps = copy_bandwidth(device)
+    result["hbm_copy_GBps"] = round(copy_gbps, 1)
+    result["roofline"]["frac_of_copy"] = round(result["roofline"]["achieved"] / copy_gbps, 4)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(layer, args.cpu_seconds)
     print(json.dumps(result), flush=True)
