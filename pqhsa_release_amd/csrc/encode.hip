@@ -11,7 +11,7 @@ namespace pqhsa {
 
 // One thread per key row; coarse centroids pass through LDS in chunks shared by the block.
 template <int DT>
-__global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) {
+__global__ __launch_bounds__(kEncThreads, 3) void encode_bulk_kernel(EncodeArgs a) {
     __shared__ __align__(16) float cs[kCoarseChunk][kD];
     __shared__ __align__(16) float cb_s[kM * kCodes * kSub];
     const int tid = threadIdx.x;
@@ -43,7 +43,10 @@ __global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) 
         nrm = sqrtf(ss);
         if (nrm < a.eps) nrm = a.eps;
 #pragma unroll
-        for (int d = 0; d < kD; ++d) x[d] = x[d] / nrm;
+        for (int d = 0; d < kD; ++d) {
+            x[d] = x[d] / nrm;
+            if (d % 8 == 7) __builtin_amdgcn_sched_barrier(0);  // keeps the divisions' temporaries few
+        }
     } else {
 #pragma unroll
         for (int d = 0; d < kD; ++d) x[d] = 0.0f;
@@ -59,16 +62,26 @@ __global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) 
             reinterpret_cast<float4 *>(&cs[0][0])[i] = reinterpret_cast<const float4 *>(cbase + (size_t)l0 * kD)[i];
         __syncthreads();
         if (valid) {
+#pragma unroll 1
             for (int l = 0; l < nl; ++l) {
                 float d2 = 0.0f;
+                // the centroid passes through registers in pieces of 16 elements: the key row already
+                // takes 128 registers, and three waves per SIMD need the rest to stay small
 #pragma unroll
-                for (int d4 = 0; d4 < kD / 4; ++d4) {
-                    const float4 c = reinterpret_cast<const float4 *>(&cs[l][0])[d4];
-                    float t;
-                    t = x[4 * d4] - c.x; d2 = __builtin_fmaf(t, t, d2);
-                    t = x[4 * d4 + 1] - c.y; d2 = __builtin_fmaf(t, t, d2);
-                    t = x[4 * d4 + 2] - c.z; d2 = __builtin_fmaf(t, t, d2);
-                    t = x[4 * d4 + 3] - c.w; d2 = __builtin_fmaf(t, t, d2);
+                for (int d16 = 0; d16 < kD / 16; ++d16) {
+                    float4 c[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) c[u] = reinterpret_cast<const float4 *>(&cs[l][0])[4 * d16 + u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int d = 16 * d16 + 4 * u;
+                        float t;
+                        t = x[d] - c[u].x; d2 = __builtin_fmaf(t, t, d2);
+                        t = x[d + 1] - c[u].y; d2 = __builtin_fmaf(t, t, d2);
+                        t = x[d + 2] - c[u].z; d2 = __builtin_fmaf(t, t, d2);
+                        t = x[d + 3] - c[u].w; d2 = __builtin_fmaf(t, t, d2);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 if (d2 < bestd) { bestd = d2; best = l0 + l; }
             }
@@ -81,12 +94,14 @@ __global__ __launch_bounds__(kEncThreads) void encode_bulk_kernel(EncodeArgs a) 
     for (int d4 = 0; d4 < kD / 4; ++d4) {
         const float4 c = reinterpret_cast<const float4 *>(cbest)[d4];
         x[4 * d4] -= c.x; x[4 * d4 + 1] -= c.y; x[4 * d4 + 2] -= c.z; x[4 * d4 + 3] -= c.w;
+        if (d4 % 4 == 3) __builtin_amdgcn_sched_barrier(0);  // a few loads in flight, not all 32
     }
     uint32_t word = 0;
 #pragma unroll
     for (int m = 0; m < kM; ++m) {
         int bc = 0;
         float bd = INFINITY;
+#pragma unroll 1
         for (int c = 0; c < kCodes; ++c) {
             const float *w = &cb_s[(m * kCodes + c) * kSub];
             float d2 = 0.0f;

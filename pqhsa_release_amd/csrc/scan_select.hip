@@ -8,14 +8,17 @@
 //           matrices only: the first digit of the stand-alone radix top-k)
 //   kEmit   keep every key whose order-preserving key reaches the row's threshold as a
 //           (key, index, list) candidate, and sum exp(logit - reference) of all other keys per
-//           IVF list.  Candidate slots come from a wave prefix sum into wave-private staging
-//           (no atomics in the loop); stored keys are ordered by list, so the per-list sums are
+//           IVF list.  Candidate slots come from a wave prefix sum: sparse 256-key windows go to
+//           wave-private LDS staging (one reservation in memory per workgroup and row, at the
+//           end), a window too dense for the staging area reserves once per row and writes
+//           straight to memory.  Stored keys are ordered by list, so the per-list sums are
 //           wave-level segment sums with one LDS update per (wave, list) instead of one per key.
 // sample_thresh_kernel scores a fixed random subset of the stored keys and takes, as the
 // threshold, the sampled key whose rank keeps, with a wide safety margin, more than k keys of the
 // full row; select_final_kernel finds the exact k-th largest key among the candidates by
-// bisection on the 32-bit key (ties at the boundary go to the lowest index), compacts the
-// winners, and returns the losers' weights to their lists.  A row whose estimate kept fewer than
+// bisection on the 32-bit key, below the leading bits that all candidates share (ties at the
+// boundary go to the lowest index), compacts the winners, and returns the losers' weights to
+// their lists.  A row whose estimate kept fewer than
 // k candidates is re-scanned in full by its select workgroup, so the result is always the exact
 // top-k.
 #include <cstdlib>
