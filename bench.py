@@ -84,7 +84,7 @@ class Layer:
         ``room`` more tokens per sequence (already written, as a serving engine writes a token's K/V
         before attention runs), and each step makes one of them visible."""
         from pqhsa_release_amd import ops
-        from pqhsa_release_amd.index.train import train_ivfpq
+        from pqhsa_release_amd.index.train import train_ivfpq_batched
 
         desc, B, H, G, ctx, dtype, paged, shuffled = CONFIGS[cfg_id]
         self.B, self.H, self.G, self.dtype = B, H, G, dtype
@@ -117,6 +117,7 @@ class Layer:
         for b, ln0 in enumerate(self.lens):
             ln = ln0 + room
             pos = torch.arange(ln, device=device)
+            head_keys = []
             for h in range(H):
                 k, v, qq = make_stream(ln, G, seed0 + 1000 * b + h, device, dtype)
                 if paged:
@@ -127,17 +128,20 @@ class Layer:
                     self.keys[b, h, :ln] = k
                     self.values[b, h, :ln] = v
                 q[b, h * G : (h + 1) * G] = qq
-                coarse, books = train_ivfpq(k[SINK : SINK + self.n[b]], num_lists=LISTS, coarse_iter=1, pq_iter=2,
-                                            seed=0)
-                self.index.coarse[b * H + h, : coarse.shape[0]] = coarse
-                self.index.codebooks[b * H + h] = books
+                head_keys.append(k[SINK : SINK + self.n[b]])
                 del k, v
+            # the sequence's KV heads have one length: their indexes train together
+            coarse, books = train_ivfpq_batched(torch.stack(head_keys), num_lists=LISTS, coarse_iter=1, pq_iter=2,
+                                                seed=0)
+            self.index.coarse[b * H : (b + 1) * H, : coarse.shape[1]] = coarse
+            self.index.codebooks[b * H : (b + 1) * H] = books
+            del head_keys
         self.q = q
         self.out = torch.empty_like(q)
         self.index.set_counts(self.n)
         ops.encode(self.kv, self.index, SINK, [0] * B, self.n)
-        ops.value_summaries(self.kv, self.index, SINK)
         self.index.finalize_layout()
+        ops.value_summaries(self.kv, self.index, SINK)
         self.seq_lens = torch.tensor(self.lens, dtype=torch.int32, device=device)
         k_cap = ops.resolve_topk(n_max + room, FRACTION, 0)
         self.ws = ops.DecodeWorkspace(self.index, G, k_cap)

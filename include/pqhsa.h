@@ -130,7 +130,9 @@ int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink
 /*
  * Rebuild vsum / vcount / vbar from the values of all indexed keys
  * (SparseKVCache._build_retrieval_value_summaries, pq_hsa/attention/kv_cache.py:688-728).
- * n_max >= max_b n_idx[b].
+ * n_max >= max_b n_idx[b] sizes the launch (<= 0: n_cap).  Three launches: clear, accumulate
+ * with float atomics, divide; fastest on a list-ordered layout, where a run of keys of one list
+ * costs one atomic add per channel.
  */
 int pqhsa_value_summaries(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
                           int32_t n_max, void *stream);

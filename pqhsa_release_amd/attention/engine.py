@@ -17,7 +17,7 @@ import torch
 
 from .. import ops
 from ..config import IVFPQConfig, SparseAttentionConfig, validate_for_kernels
-from ..index.train import train_ivfpq
+from ..index.train import train_ivfpq_batched
 
 D = ops.HEAD_DIM
 
@@ -128,6 +128,13 @@ class PQHSAEngine:
                 getattr(self.index, name).copy_(getattr(old, name))
             self.index.n_sorted_host = list(old.n_sorted_host)
 
+    def _retrieval_block(self, b: int, count: int) -> torch.Tensor:
+        """The first ``count`` retrieval-region keys of every KV head of sequence b, ``[H, count, 128]``."""
+        s = self._sink_end(b)
+        if self.keys_buf is not None:
+            return self.keys_buf[b, :, s : s + count]
+        return ops.paged_gather_range(self.kv, b, s, s + count)[0]
+
     def _retrieval_keys(self, b: int, h: int, start: int, count: int) -> torch.Tensor:
         s = self._sink_end(b)
         if self.keys_buf is not None:
@@ -153,29 +160,31 @@ class PQHSAEngine:
         self._alloc_index(max(counts), lists)
         ic = self.index_config
         if coarse is None:
-            paged_cache = {}
+            # sequences of one length train together, all their KV heads at once
+            by_count: dict[int, list[int]] = {}
             for b in range(self.B):
-                if counts[b] == 0:
-                    continue
-                if self.keys_buf is None:
-                    s = self._sink_end(b)
-                    paged_cache[b], _ = ops.paged_gather_range(self.kv, b, s, s + counts[b])
-                for h in range(self.H):
-                    rows = (self.keys_buf[b, h, self._sink_end(b) : self._sink_end(b) + counts[b]]
-                            if self.keys_buf is not None else paged_cache[b][h])
-                    c, cb = train_ivfpq(rows, num_lists=lists, coarse_iter=ic.coarse_max_iter,
-                                        pq_iter=ic.pq_max_iter, seed=ic.seed, eps=ic.eps)
-                    self.index.coarse[b * self.H + h, : c.shape[0]].copy_(c)
-                    self.index.codebooks[b * self.H + h].copy_(cb)
-                paged_cache.pop(b, None)
+                if counts[b] > 0:
+                    by_count.setdefault(counts[b], []).append(b)
+            for n, seqs in by_count.items():
+                step = max(1, ((1 << 31) // (n * ops.HEAD_DIM * 4)) // self.H)  # about 2 GB of fp32 keys per batch
+                for i in range(0, len(seqs), step):
+                    part = seqs[i : i + step]
+                    rows = torch.stack([self._retrieval_block(b, n) for b in part]).reshape(-1, n, ops.HEAD_DIM)
+                    c, cb = train_ivfpq_batched(rows, num_lists=lists, coarse_iter=ic.coarse_max_iter,
+                                                pq_iter=ic.pq_max_iter, seed=ic.seed, eps=ic.eps)
+                    del rows
+                    for j, b in enumerate(part):
+                        sl = slice(b * self.H, (b + 1) * self.H)
+                        self.index.coarse[sl, : c.shape[1]].copy_(c[j * self.H : (j + 1) * self.H])
+                        self.index.codebooks[sl].copy_(cb[j * self.H : (j + 1) * self.H])
         else:
             self.index.coarse.copy_(coarse.to(self.device, torch.float32).expand_as(self.index.coarse))
             self.index.codebooks.copy_(codebooks.to(self.device, torch.float32).expand_as(self.index.codebooks))
         self.index.set_counts(counts)
         if max(counts) > 0:
             ops.encode(self.kv, self.index, self.sink, [0] * self.B, counts, eps=ic.eps)
-            ops.value_summaries(self.kv, self.index, self.sink)
             self.index.finalize_layout(seed=ic.seed)
+            ops.value_summaries(self.kv, self.index, self.sink)   # after the sort: one atomic per run of a list
         self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
         self.index_rebuilds += 1
 
@@ -285,8 +294,8 @@ class PQHSAEngine:
         idx.reset_layout()
         idx.set_counts(new)
         ops.encode(self.kv, idx, self.sink, [0] * self.B, new, eps=ic.eps)
-        ops.value_summaries(self.kv, idx, self.sink)
         idx.finalize_layout(seed=ic.seed)
+        ops.value_summaries(self.kv, idx, self.sink)
 
     # ------------------------------------------------------------------ forward
     def forward(self, q: torch.Tensor, groups: int, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -143,51 +143,79 @@ __global__ __launch_bounds__(kD) void value_append_kernel(EncodeArgs a) {
         value_append_one<DT>(a, bh, b, h, s0 + j, a.list_ids[(size_t)bh * a.n_cap + s0 + j]);
 }
 
-// Rebuild per-list value sums / counts / means.  One workgroup per (stream, 8 lists); every
-// workgroup walks the list ids in insertion order and accumulates the rows of its lists.
-constexpr int kListsPerWg = 8;
+// Rebuild per-list value sums / counts / means in three launches: clear, accumulate, divide.
+// Accumulate: 16 lanes own one value row (8 channels each); every 16-lane group walks 16
+// consecutive stored keys and hands a run of equal list ids to the list's sum with one atomic
+// add per channel, so on a list-ordered layout most keys cost no atomic at all (an unordered
+// layout pays one set per key).  The sums are exact up to the order of fp32 additions.
+constexpr int kSumThreads = 256;
+constexpr int kSumGroups = kSumThreads / 16;
+constexpr int kSumRun = 16;
 
 template <int DT>
-__global__ __launch_bounds__(kD) void value_summaries_kernel(EncodeArgs a) {
-    __shared__ float acc[kListsPerWg][kD];
-    __shared__ float cnt_s[kListsPerWg];
-    const int d = threadIdx.x;
+__global__ __launch_bounds__(kSumThreads) void value_sums_kernel(EncodeArgs a) {
+    const int lane16 = threadIdx.x & 15, grp = threadIdx.x >> 4;
     const int bh = blockIdx.y;
     const int b = bh / a.H, h = bh % a.H;
-    const int l0 = blockIdx.x * kListsPerWg;
     const int n = a.n_idx[b];
+    const int first = (blockIdx.x * kSumGroups + grp) * kSumRun;
+    if (first >= n) return;
     const size_t esz = DT == PQHSA_F32 ? 4 : 2;
+    // lane r of the group fetches list id and token of the group's r-th key
+    int my_list = -1, my_tok = 0;
+    if (first + lane16 < n) {
+        const size_t o = (size_t)bh * a.n_cap + first + lane16;
+        my_list = a.list_ids[o];
+        my_tok = a.pos ? a.pos[o] : first + lane16;  // retrieval-local index of the stored key
+        if (my_list >= a.L) my_list = -1;
+    }
+    float *vsum = a.vsum + (size_t)bh * a.L * kD;
+    float *vcount = a.vcount + (size_t)bh * a.L;
+    float acc[8];
+    int cur = -1;
+    float run = 0.0f;
+    auto flush = [&]() {
+        if (cur < 0) return;
 #pragma unroll
-    for (int l = 0; l < kListsPerWg; ++l) acc[l][d] = 0.0f;
-    if (d < kListsPerWg) cnt_s[d] = 0.0f;
-    __syncthreads();
-    __shared__ int rel[kD];
-    __shared__ int tok[kD];
-    const uint16_t *lids = a.list_ids + (size_t)bh * a.n_cap;
-    const int32_t *pos = a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr;
-    for (int i0 = 0; i0 < n; i0 += kD) {
-        __syncthreads();
-        rel[d] = (i0 + d < n) ? (int)lids[i0 + d] - l0 : -1;
-        tok[d] = (i0 + d < n && pos) ? pos[i0 + d] : i0 + d;  // retrieval-local index of the stored key
-        __syncthreads();
-        const int lim = min(kD, n - i0);
-        for (int t = 0; t < lim; ++t) {
-            const int l = rel[t];
-            if (l < 0 || l >= kListsPerWg) continue;
-            const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + tok[t]) * esz;
-            acc[l][d] += load1<DT>(row, d);
-            if (d == 0) cnt_s[l] += 1.0f;
+        for (int e = 0; e < 8; ++e) unsafeAtomicAdd(&vsum[(size_t)cur * kD + lane16 * 8 + e], acc[e]);
+        if (lane16 == 0) unsafeAtomicAdd(&vcount[cur], run);
+    };
+    for (int r0 = 0; r0 < kSumRun; r0 += 4) {
+        int l[4];
+        float f[4][8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {  // four rows on their way at once
+            l[u] = __shfl(my_list, r0 + u, 16);
+            const int tok = __shfl(my_tok, r0 + u, 16);
+            if (l[u] >= 0) {
+                const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + tok) * esz;
+                load8<DT>(row, lane16, f[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (l[u] < 0) continue;  // past the end of the stream (uniform in the group)
+            if (l[u] != cur) {
+                flush();
+                cur = l[u];
+                run = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += f[u][e];
+            run += 1.0f;
         }
     }
-    __syncthreads();
-    for (int l = 0; l < kListsPerWg; ++l) {
-        if (l0 + l >= a.L) break;
-        const size_t o = ((size_t)bh * a.L + l0 + l) * kD + d;
-        const float c = cnt_s[l];
-        a.vsum[o] = acc[l][d];
-        a.vbar[o] = c > 0.0f ? acc[l][d] / c : 0.0f;
-        if (d == 0) a.vcount[(size_t)bh * a.L + l0 + l] = c;
-    }
+    flush();
+}
+
+__global__ __launch_bounds__(256) void value_means_kernel(const float *vsum, const float *vcount, float *vbar,
+                                                          size_t elems) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= elems) return;
+    const float c = vcount[i / kD];
+    vbar[i] = c > 0.0f ? vsum[i] / c : 0.0f;
 }
 
 // ---- paged readers ----------------------------------------------------------------------
@@ -271,12 +299,21 @@ extern "C" int pqhsa_value_summaries(const pqhsa_kv_view *kv, const pqhsa_index 
     int rc = fill_encode_args(a, kv, index, sink, nullptr, nullptr, 0.0f);
     if (rc) return rc;
     PQHSA_REQUIRE(index->vsum && index->vcount && index->vbar && index->n_idx, "value_summaries: NULL arrays");
-    (void)n_max;
     const int BH = index->batch * index->kv_heads;
     if (BH == 0) return PQHSA_OK;
-    dim3 grid((index->num_lists + kListsPerWg - 1) / kListsPerWg, BH);
-    PQHSA_DISPATCH_DTYPE(kv->dtype, hipLaunchKernelGGL(value_summaries_kernel<DT>, grid, dim3(kD), 0,
-                                                       static_cast<hipStream_t>(stream), a));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t elems = (size_t)BH * index->num_lists * kD;
+    rc = launch_fill_zero(index->vsum, elems * sizeof(float), s);
+    if (rc) return rc;
+    rc = launch_fill_zero(index->vcount, (size_t)BH * index->num_lists * sizeof(float), s);
+    if (rc) return rc;
+    const int64_t keys = n_max > 0 && n_max <= index->n_cap ? n_max : index->n_cap;  // n_max <= 0: not known
+    dim3 grid((unsigned)((keys + kSumGroups * kSumRun - 1) / (kSumGroups * kSumRun)), BH);
+    PQHSA_DISPATCH_DTYPE(kv->dtype, hipLaunchKernelGGL(value_sums_kernel<DT>, grid, dim3(kSumThreads), 0, s, a));
+    rc = check_launch("value_sums");
+    if (rc) return rc;
+    hipLaunchKernelGGL(value_means_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, s, index->vsum,
+                       index->vcount, index->vbar, elems);
     return check_launch("value_summaries");
 }
 

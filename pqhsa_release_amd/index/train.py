@@ -85,3 +85,114 @@ def train_ivfpq(keys: torch.Tensor, *, num_lists: int, num_subspaces: int = 8, n
         c, _ = kmeans_l2(chunks[:, m].contiguous(), num_codes, max_iter=pq_iter, seed=seed + 10_000 + m, eps=eps)
         books.append(c)
     return coarse.float().contiguous(), torch.stack(books, dim=0).float().contiguous()
+
+
+# ---- all streams of equal length at once --------------------------------------------------------
+# The per-stream procedure above issues a few hundred small launches per stream.  Streams of the
+# same length (all KV heads of a sequence, and every sequence of the same context) share the seeded
+# draws, so they train together as batched matrix products: the reference's own answer to the
+# build time (pq_hsa/index/batched_build.py:82-167).
+
+
+class _LazyGenerators:
+    """One generator per stream, all seeded alike, created only for a stream that needs a draw of
+    its own (an empty cluster) and first advanced past the draws every stream shares."""
+
+    def __init__(self, streams: int, seed: int, device, n: int, shared_perm: bool) -> None:
+        self.gens = [None] * streams
+        self.seed, self.device, self.n, self.shared_perm = int(seed), device, n, shared_perm
+
+    def get(self, s: int) -> torch.Generator:
+        if self.gens[s] is None:
+            g = torch.Generator(device=self.device)
+            g.manual_seed(self.seed)
+            if self.shared_perm:
+                torch.randperm(self.n, generator=g, device=self.device)
+            self.gens[s] = g
+        return self.gens[s]
+
+
+def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int = 1 << 27) -> torch.Tensor:
+    """``vectors [S, N, D]``, ``centroids [S, K, D]`` -> nearest centroid per vector ``[S, N]``."""
+    s, n, _ = vectors.shape
+    cf = centroids.float()
+    half_sq = (cf * cf).sum(dim=2).unsqueeze(1)
+    chunk = max(1024, budget // max(1, s * cf.shape[1]))
+    out = torch.empty(s, n, dtype=torch.long, device=vectors.device)
+    for i in range(0, n, chunk):
+        v = vectors[:, i : i + chunk].float()
+        out[:, i : i + chunk] = (half_sq - 2.0 * torch.bmm(v, cf.transpose(1, 2))).argmin(dim=2)
+    return out
+
+
+def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed: int = 0, eps: float = 1e-12):
+    """``kmeans_l2`` for ``S`` independent problems of one size, ``vectors [S, N, D]``: the seeded
+    start (one permutation, the same for every problem, as S separate calls with one seed would
+    draw) and the Lloyd iterations run as batched products; a problem whose assignment stops
+    changing keeps its centroids, as the early exit of the per-stream loop does."""
+    if vectors.ndim != 3:
+        raise ValueError(f"vectors must be [S, N, D], got {tuple(vectors.shape)}")
+    s, n, dim = vectors.shape
+    if n == 0:
+        raise ValueError("cannot train k-means with zero vectors")
+    dev = vectors.device
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(int(seed))
+    lazy = _LazyGenerators(s, seed, dev, n, shared_perm=n >= num_clusters)
+    if n >= num_clusters:
+        centroids = vectors[:, torch.randperm(n, generator=gen, device=dev)[:num_clusters]].clone()
+    else:
+        extra = torch.randint(0, n, (num_clusters - n,), generator=gen, device=dev)
+        centroids = torch.cat([vectors, vectors[:, extra]], dim=1).clone()
+        for i in range(s):  # every stream's own generator has made this draw too
+            torch.randint(0, n, (num_clusters - n,), generator=lazy.get(i), device=dev)
+    assign = torch.zeros(s, n, dtype=torch.long, device=dev)
+    live = torch.ones(s, dtype=torch.bool, device=dev)
+    offsets = (torch.arange(s, device=dev) * num_clusters).unsqueeze(1)
+    flat = vectors.reshape(s * n, dim).float()
+    for _ in range(max_iter):
+        nxt = _nearest_batched(vectors, centroids)
+        same = (assign == nxt).all(dim=1)
+        assign = torch.where(live.unsqueeze(1), nxt, assign)
+        live = live & ~same
+        if not bool(live.any()):
+            break
+        sums = torch.zeros(s * num_clusters, dim, dtype=torch.float32, device=dev)
+        sums.index_add_(0, (assign + offsets).reshape(-1), flat)
+        counts = torch.bincount((assign + offsets).reshape(-1), minlength=s * num_clusters).float()
+        filled = counts > 0
+        sums[filled] /= counts[filled].unsqueeze(1).clamp_min(eps)
+        sums = sums.reshape(s, num_clusters, dim)
+        empty = (~filled).reshape(s, num_clusters)
+        if bool(empty.any()):
+            for i in torch.nonzero(empty.any(dim=1)).flatten().tolist():
+                if not bool(live[i]):
+                    continue
+                pick = torch.randint(0, n, (int(empty[i].sum().item()),), generator=lazy.get(i), device=dev)
+                sums[i][empty[i]] = vectors[i][pick].float()
+        centroids = torch.where(live.view(s, 1, 1), sums.to(vectors.dtype), centroids)
+    return centroids, _nearest_batched(vectors, centroids)
+
+
+def train_ivfpq_batched(keys: torch.Tensor, *, num_lists: int, num_subspaces: int = 8, num_codes: int = 16,
+                        coarse_iter: int = 1, pq_iter: int = 2, seed: int = 0, eps: float = 1e-12):
+    """``train_ivfpq`` for ``S`` streams of one length at once: ``keys [S, N, D]`` ->
+    ``(coarse [S, L', D], codebooks [S, M, num_codes, D/M])``, fp32."""
+    if keys.ndim != 3 or keys.shape[1] == 0:
+        raise ValueError("cannot build IVF-PQ index with zero keys")
+    if keys.shape[2] % num_subspaces != 0:
+        raise ValueError(f"dim={keys.shape[2]} must be divisible by num_subspaces={num_subspaces}")
+    k32 = keys.float()
+    norms = torch.linalg.vector_norm(k32, dim=-1).clamp_min(eps)
+    dirs = k32 / norms.unsqueeze(-1)
+    lists = min(int(num_lists), dirs.shape[1])
+    coarse, assign = kmeans_l2_batched(dirs, lists, max_iter=coarse_iter, seed=seed, eps=eps)
+    resid = dirs - torch.gather(coarse, 1, assign.unsqueeze(-1).expand(-1, -1, dirs.shape[2]))
+    sub = keys.shape[2] // num_subspaces
+    chunks = resid.reshape(resid.shape[0], resid.shape[1], num_subspaces, sub)
+    books = []
+    for m in range(num_subspaces):
+        c, _ = kmeans_l2_batched(chunks[:, :, m].contiguous(), num_codes, max_iter=pq_iter,
+                                 seed=seed + 10_000 + m, eps=eps)
+        books.append(c)
+    return coarse.float().contiguous(), torch.stack(books, dim=1).float().contiguous()

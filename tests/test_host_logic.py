@@ -285,3 +285,24 @@ def test_plugin_is_a_noop_unless_enabled_and_config_env_round_trip(clean_runtime
     cfg.apply_env_defaults()
     back = PQHSAConfig.from_env()
     assert (back.top_fraction, back.local_window, back.batch) == (0.05, 64, True)
+
+
+def test_batched_index_training_equals_the_per_stream_procedure():
+    """Streams of one length train together (batched matrix products); with the shared seed the
+    result is what one train_ivfpq call per stream gives, including the paths for fewer vectors
+    than clusters and for clusters left empty (each stream then draws from its own generator)."""
+    from pqhsa_release_amd.index.train import train_ivfpq, train_ivfpq_batched
+
+    gen = torch.Generator().manual_seed(5)
+    centers = torch.randn(4, 24, 128, generator=gen)
+    pick = torch.randint(0, 24, (4, 1500), generator=gen)
+    keys = centers[torch.arange(4)[:, None], pick] + 0.3 * torch.randn(4, 1500, 128, generator=gen)
+    for k, lists in ((keys, 32), (keys[:, :12], 32)):   # 12 keys: fewer than the 16 codewords
+        coarse, books = train_ivfpq_batched(k, num_lists=lists, coarse_iter=2, pq_iter=3, seed=11)
+        assert coarse.shape == (4, min(lists, k.shape[1]), 128) and books.shape == (4, 8, 16, 16)
+        for s in range(4):
+            c1, b1 = train_ivfpq(k[s], num_lists=lists, coarse_iter=2, pq_iter=3, seed=11)
+            torch.testing.assert_close(coarse[s], c1, rtol=0, atol=1e-6)
+            torch.testing.assert_close(books[s], b1, rtol=0, atol=1e-6)
+    with pytest.raises(ValueError):
+        train_ivfpq_batched(keys[:, :0], num_lists=8)
