@@ -39,10 +39,22 @@ class MultiHeadAttentionOutput:
     leading_shape: tuple[int, ...]
 
 
-@dataclass(slots=True)
 class DecodeAttentionOutput:
-    context: torch.Tensor
-    per_query: tuple[MultiHeadAttentionOutput, ...]
+    """``context`` plus the reference's per-query / per-stream records.  The records are host
+    bookkeeping (one small object per query row and stream); they are built when ``per_query`` is
+    first read, so a serving loop that only takes ``context`` does not pay for them."""
+
+    __slots__ = ("context", "_per_query")
+
+    def __init__(self, context: torch.Tensor, per_query) -> None:
+        self.context = context
+        self._per_query = per_query   # the records, or a function that builds them
+
+    @property
+    def per_query(self) -> tuple[MultiHeadAttentionOutput, ...]:
+        if callable(self._per_query):
+            self._per_query = self._per_query()
+        return self._per_query
 
 
 def _normalize_queries(queries: torch.Tensor) -> tuple[torch.Tensor, bool]:
@@ -121,24 +133,31 @@ class _AdapterBase:
         eng = self._check_built()
         return eng.B * eng.H if eng.apply_pending_index_update() else 0
 
-    def _per_query(self, context: torch.Tensor, groups: int) -> tuple[MultiHeadAttentionOutput, ...]:
-        """context [B, H, Q, D] -> the reference's per-query / per-stream records (host numbers
-        only; nothing is read back from the device)."""
+    def _per_query_later(self, context: torch.Tensor, groups: int):
+        """context [B, H, Q, D] -> a function that builds the reference's per-query / per-stream
+        records (host numbers only; nothing is read back from the device).  The counts are taken
+        now, so later appends do not change what the records say about this step."""
         eng = self.engine
         from .. import ops
 
-        records = []
-        for qpos in range(context.shape[2]):
-            per_stream = []
-            for b in range(eng.B):
-                n, full = eng.n(b), eng.full_count(b)
-                k = ops.resolve_topk(n, self.attention_config.retrieval_top_fraction,
-                                     self.attention_config.retrieval_topk)
-                for h in range(context.shape[1]):
-                    per_stream.append(StreamOutput(context[b, h, qpos], full + k, full + n, n, k, n))
-            records.append(MultiHeadAttentionOutput(context[:, :, qpos], tuple(per_stream),
-                                                    (context.shape[0], context.shape[1])))
-        return tuple(records)
+        ac = self.attention_config
+        counts = []
+        for b in range(eng.B):
+            n, full = eng.n(b), eng.full_count(b)
+            counts.append((n, full, ops.resolve_topk(n, ac.retrieval_top_fraction, ac.retrieval_topk)))
+
+        def build() -> tuple[MultiHeadAttentionOutput, ...]:
+            records = []
+            for qpos in range(context.shape[2]):
+                per_stream = []
+                for b, (n, full, k) in enumerate(counts):
+                    for h in range(context.shape[1]):
+                        per_stream.append(StreamOutput(context[b, h, qpos], full + k, full + n, n, k, n))
+                records.append(MultiHeadAttentionOutput(context[:, :, qpos], tuple(per_stream),
+                                                        (context.shape[0], context.shape[1])))
+            return tuple(records)
+
+        return build
 
     def state_dict(self) -> dict[str, object]:
         eng = self._check_built()
@@ -192,7 +211,7 @@ class IVFPQDecodeAttentionAdapter(_AdapterBase):
             raise ValueError(f"queries must have shape ({b}, {h}, query_len, 128), got {tuple(q.shape)}")
         qlen = q.shape[2]
         ctx = eng.forward(q.reshape(b, h * qlen, 128), qlen).reshape(b, h, qlen, 128).to(queries.dtype)
-        per_query = self._per_query(ctx, qlen)
+        per_query = self._per_query_later(ctx, qlen)
         return DecodeAttentionOutput(context=ctx if had_len else ctx.squeeze(-2), per_query=per_query)
 
     def decode_step(self, queries, keys=None, values=None, *, append_kv: bool = True) -> DecodeAttentionOutput:
@@ -239,7 +258,7 @@ class GQAIVFPQDecodeAttentionAdapter(_AdapterBase):
             raise ValueError(f"queries must be [{b}, {self.num_query_heads}, (1,) 128], got {tuple(queries.shape)}")
         ctx = eng.forward(q, self.num_key_value_groups).to(queries.dtype)
         g = self.num_key_value_groups
-        per_query = self._per_query(ctx.reshape(b, self.num_key_value_heads, g, 128), g)
+        per_query = self._per_query_later(ctx.reshape(b, self.num_key_value_heads, g, 128), g)
         return DecodeAttentionOutput(context=ctx.unsqueeze(2) if had_len else ctx, per_query=per_query)
 
     def forward_context_fast(self, queries: torch.Tensor) -> torch.Tensor:

@@ -128,19 +128,13 @@ class PQHSAEngine:
                 getattr(self.index, name).copy_(getattr(old, name))
             self.index.n_sorted_host = list(old.n_sorted_host)
 
-    def _retrieval_block(self, b: int, count: int) -> torch.Tensor:
-        """The first ``count`` retrieval-region keys of every KV head of sequence b, ``[H, count, 128]``."""
-        s = self._sink_end(b)
+    def _retrieval_block(self, b: int, count: int, start: int = 0) -> torch.Tensor:
+        """``count`` retrieval-region keys of every KV head of sequence b from retrieval-local index
+        ``start`` on, ``[H, count, 128]``."""
+        s = self._sink_end(b) + start
         if self.keys_buf is not None:
             return self.keys_buf[b, :, s : s + count]
         return ops.paged_gather_range(self.kv, b, s, s + count)[0]
-
-    def _retrieval_keys(self, b: int, h: int, start: int, count: int) -> torch.Tensor:
-        s = self._sink_end(b)
-        if self.keys_buf is not None:
-            return self.keys_buf[b, h, s + start : s + start + count]
-        k, _ = ops.paged_gather_range(self.kv, b, s + start, s + start + count)
-        return k[h]
 
     def build(self, lens, *, coarse: torch.Tensor | None = None, codebooks: torch.Tensor | None = None) -> None:
         """(Re)build the index over the retrieval region of every sequence.  Without
@@ -266,30 +260,35 @@ class PQHSAEngine:
         from the HIP encode kernel; the small per-list means are torch ops on the device."""
         ic, idx = self.index_config, self.index
         lr = ic.online_codebook_lr
+        H, L = self.H, idx.num_lists
+        head = torch.arange(H, device=self.device).unsqueeze(1)
+
+        def new_dirs(b: int) -> torch.Tensor:  # [H, added, 128] directions of sequence b's new keys
+            rows = self._retrieval_block(b, added[b], start=old[b]).float()
+            return rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
+
         ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # lists of the new rows
-        for b in range(self.B):
+        for b in range(self.B):  # all KV heads of a sequence move their tables in one go
             if added[b] <= 0:
                 continue
-            for h in range(self.H):
-                bh = b * self.H + h
-                rows = self._retrieval_keys(b, h, old[b], added[b]).float()
-                dirs = rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
-                lids = idx.list_ids_long()[bh, old[b] : old[b] + added[b]]
-                _ema_rows(idx.coarse[bh], dirs, lids, lr, ic.eps)
+            sl = slice(old[b], old[b] + added[b])
+            lids = idx.list_ids[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFF
+            _ema_rows(idx.coarse[b * H : (b + 1) * H].view(H * L, D), new_dirs(b).reshape(-1, D),
+                      (lids + head * L).reshape(-1), lr, ic.eps)
         ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # re-assign with moved lists
         for b in range(self.B):
             if added[b] <= 0:
                 continue
-            for h in range(self.H):
-                bh = b * self.H + h
-                rows = self._retrieval_keys(b, h, old[b], added[b]).float()
-                dirs = rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
-                sl = slice(old[b], old[b] + added[b])
-                lids = idx.list_ids_long()[bh, sl]
-                resid = (dirs - idx.coarse[bh][lids]).reshape(-1, ops.SUBSPACES, ops.SUBDIM)
-                words = idx.codes[bh, sl].to(torch.int64) & 0xFFFFFFFF
-                for m in range(ops.SUBSPACES):
-                    _ema_rows(idx.codebooks[bh, m], resid[:, m], (words >> (4 * m)) & 15, lr, ic.eps)
+            sl = slice(old[b], old[b] + added[b])
+            lids = idx.list_ids[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFF
+            coarse = idx.coarse[b * H : (b + 1) * H]
+            resid = new_dirs(b) - torch.gather(coarse, 1, lids.unsqueeze(-1).expand(-1, -1, D))
+            words = idx.codes[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFFFFFF
+            shifts = 4 * torch.arange(ops.SUBSPACES, device=self.device)
+            code = (words.unsqueeze(-1) >> shifts) & 15                           # [H, added, 8]
+            book = (head.unsqueeze(-1) * ops.SUBSPACES + torch.arange(ops.SUBSPACES, device=self.device)) * 16
+            _ema_rows(idx.codebooks[b * H : (b + 1) * H].view(H * ops.SUBSPACES * 16, ops.SUBDIM),
+                      resid.reshape(-1, ops.SUBDIM), (code + book).reshape(-1), lr, ic.eps)
         new = [o + a for o, a in zip(old, added)]
         idx.reset_layout()
         idx.set_counts(new)
