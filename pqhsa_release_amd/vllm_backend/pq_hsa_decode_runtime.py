@@ -52,6 +52,8 @@ STATS: dict[str, Any] = {
     "reject": {},
     "pq_batch_steps": 0,
     "pq_batch_reqs_total": 0,
+    "pq_batch_fused_steps": 0,
+    "pq_batch_group_builds": 0,
     "batch_mode": False,
 }
 
@@ -162,6 +164,24 @@ def reject(reason: str) -> bool:
     return False
 
 
+def host_seq_lens(attn_metadata) -> list[int]:
+    """The batch's sequence lengths as host integers.  Reading them from the device waits for the
+    GPU, so the list is taken from a host copy when the metadata carries one and is kept on the
+    metadata object: every layer of a step gets the same object."""
+    cached = getattr(attn_metadata, "_pq_host_seq_lens", None)
+    if cached is not None:
+        return cached
+    src = getattr(attn_metadata, "seq_lens_cpu", None)
+    if src is None:
+        src = attn_metadata.seq_lens
+    lens = [int(x) for x in src.tolist()]
+    try:
+        attn_metadata._pq_host_seq_lens = lens
+    except Exception:
+        pass
+    return lens
+
+
 def should_pq_decode(attn_metadata) -> bool:
     if attn_metadata is None:
         return reject("no_metadata")
@@ -175,7 +195,7 @@ def should_pq_decode(attn_metadata) -> bool:
             return reject("num_reqs<1")
         if int(getattr(attn_metadata, "num_actual_tokens", 0)) != int(seq_lens.shape[0]):
             return reject("num_actual_tokens!=num_reqs")
-        if int(seq_lens.min().item()) < min_pq_seq():
+        if min(host_seq_lens(attn_metadata)) < min_pq_seq():
             return reject("seq_too_short")
         return True
     if int(getattr(attn_metadata, "num_actual_tokens", 0)) != 1:
@@ -329,13 +349,76 @@ def run_pq_decode(impl, layer, query, key, value, kv_cache, attn_metadata) -> to
     return ctx
 
 
+def batch_fused() -> bool:
+    """``PQ_HSA_BATCH_FUSED`` (default on): the requests of a decode batch share one engine and one
+    kernel sequence per layer; ``0`` keeps one sidecar per request, as the reference does."""
+    return os.environ.get("PQ_HSA_BATCH_FUSED", "1") == "1"
+
+
+def _int32_table(attn_metadata, num_reqs: int) -> torch.Tensor:
+    table = attn_metadata.block_table[:num_reqs]
+    if table.dtype != torch.int32 or not table.is_contiguous():
+        table = table.to(torch.int32).contiguous()
+    return table
+
+
+def run_pq_decode_group(impl, layer, query, key, value, kv_cache, attn_metadata, output) -> torch.Tensor:
+    """All requests of the decode batch through one engine: the step's appends ride on the decode
+    launches and every sequence, KV head and query row is served by the same six kernels.  The
+    group is rebuilt whenever the batch is not the previous one advanced by one token each."""
+    from ..attention.engine import PQHSAEngine
+
+    st = state_for(impl, layer)
+    num_reqs = int(attn_metadata.seq_lens.shape[0])
+    lens = list(host_seq_lens(attn_metadata))
+    grp = st.get("group")
+    sequential = (grp is not None and len(grp["lens"]) == num_reqs
+                  and all(now == before + 1 for now, before in zip(lens, grp["lens"])))
+    table = _int32_table(attn_metadata, num_reqs)
+    if not sequential:
+        t0 = time.perf_counter()
+        eng = PQHSAEngine(paper_index_config(), paper_attention_config(impl.scale), batch=num_reqs,
+                          kv_heads=impl.num_kv_heads, device=kv_cache.device)
+        eng.bind_paged(kv_cache, table)
+        eng.build(lens)
+        grp = st["group"] = {"engine": eng, "lens": lens, "appends": 0}
+        STATS["pq_build_s_total"] += time.perf_counter() - t0
+        STATS["pq_batch_group_builds"] += 1
+        STATS["sidecar"] = "PQHSAEngine"
+    else:
+        eng = grp["engine"]
+        eng.bind_paged(kv_cache, table)      # the block table may have grown
+        eng.advance(1)
+        grp["lens"], grp["appends"] = lens, grp["appends"] + 1
+        STATS["pq_append_calls"] += 1
+    q, dst = query[:num_reqs], output[:num_reqs]
+    groups = impl.num_heads // impl.num_kv_heads
+    if dst.shape == q.shape and dst.dtype == q.dtype == kv_cache.dtype and dst.is_contiguous():
+        eng.forward(q, groups, out=dst)                      # straight into vLLM's output buffer
+    else:
+        copy_ctx(output, eng.forward(q, groups), num_reqs)
+    if sequential and flush_interval() > 0 and grp["appends"] % flush_interval() == 0:
+        t1 = time.perf_counter()
+        eng.apply_pending_index_update()
+        STATS["pq_flush_s_total"] += time.perf_counter() - t1
+        STATS["pq_flush_calls"] += 1
+    STATS["pq_batch_steps"] += 1
+    STATS["pq_batch_fused_steps"] += 1
+    STATS["pq_batch_reqs_total"] += num_reqs
+    STATS["pq_decode_calls"] += 1
+    return output
+
+
 def run_pq_decode_batch(impl, layer, query, key, value, kv_cache, attn_metadata, output) -> torch.Tensor:
     """``PQ_HSA_BATCH=1``: one sidecar per request of the decode batch
-    (benchmarks/vllm_backend/pq_hsa_batch_decode.py:383-432 of the reference)."""
+    (benchmarks/vllm_backend/pq_hsa_batch_decode.py:383-432 of the reference), or, by default,
+    one engine for the whole batch (``batch_fused``)."""
+    if batch_fused():
+        return run_pq_decode_group(impl, layer, query, key, value, kv_cache, attn_metadata, output)
     st = state_for(impl, layer)
     per_req = st.setdefault("batch", {})
     num_reqs = int(attn_metadata.seq_lens.shape[0])
-    lens = [int(x) for x in attn_metadata.seq_lens.tolist()]
+    lens = list(host_seq_lens(attn_metadata))
     for r in range(num_reqs):
         rs = per_req.get(r)
         sequential = rs is not None and lens[r] == rs["seq_len"] + 1

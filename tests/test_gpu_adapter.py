@@ -328,3 +328,84 @@ def test_vllm_hook_single_token_decode_over_a_paged_cache(layout, monkeypatch):
     finally:
         wrap.unwrap_forward(Impl)
         rt.reset_pq_hsa_layer_state()
+
+
+def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
+    """PQ_HSA_BATCH=1: a ragged decode batch through the hook, once with one engine for the whole
+    batch (the default: appends ride on the decode launches) and once with one sidecar per
+    request (the reference's form); both must agree with each other step by step, and the
+    batch must be rebuilt when a request leaves."""
+    dev = _cuda()
+    from pqhsa_release_amd.vllm_backend import pq_hsa_decode_runtime as rt
+    from pqhsa_release_amd.vllm_backend import pq_hsa_flashattn_wrap as wrap
+
+    H, G, bs, steps = 2, 4, 16, 6
+    ctxs = [1500, 900, 1203]
+    B = len(ctxs)
+    probs = [_problem(dev, heads=H, groups=G, ctx=c, extra=steps, seed=50 + i) for i, c in enumerate(ctxs)]
+    per_seq = (max(ctxs) + steps + bs - 1) // bs
+    perm = torch.randperm(B * per_seq, generator=torch.Generator().manual_seed(3)).to(torch.int32).to(dev)
+    table = perm.reshape(B, per_seq).contiguous()
+    cache = torch.zeros(2, B * per_seq, bs, H, DIM, dtype=torch.bfloat16, device=dev)
+    for b, (keys, values, _) in enumerate(probs):
+        pos = torch.arange(ctxs[b], device=dev)
+        cache[0][table[b, pos // bs].long(), pos % bs] = keys[0, :, : ctxs[b]].transpose(0, 1)
+        cache[1][table[b, pos // bs].long(), pos % bs] = values[0, :, : ctxs[b]].transpose(0, 1)
+
+    class Impl:
+        scale, num_heads, num_kv_heads, kv_cache_dtype = SCALE, H * G, H, "auto"
+
+        def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None, **extra):
+            output.fill_(-7.0)
+            return output
+
+    def run(fused, reqs_at):
+        for k in list(os.environ):
+            if k.startswith("PQ_HSA_"):
+                monkeypatch.delenv(k)
+        for k, v in {"PQ_HSA_ENABLE": "1", "PQ_HSA_BATCH": "1", "PQ_HSA_BATCH_FUSED": fused, "PQ_HSA_NUM_LISTS": "64",
+                     "PQ_HSA_TOP_FRAC": "0.02", "PQ_HSA_LOCAL": "64", "PQ_HSA_UPD_INTERVAL": "1",
+                     "PQ_HSA_FLUSH_INTERVAL": "0"}.items():
+            monkeypatch.setenv(k, v)
+        rt.reset_pq_hsa_runtime_stats()
+        rt.reset_pq_hsa_layer_state()
+        kvc = cache.clone()
+        wrap.wrap_forward(Impl)
+        impl, layer = Impl(), types.SimpleNamespace(layer_name="layers.0.attn")
+        outs = []
+        try:
+            for s in range(steps + 1):
+                reqs = reqs_at(s)
+                lens = [ctxs[b] + s for b in reqs]
+                last = torch.tensor([ln - 1 for ln in lens], device=dev)
+                tb = table[reqs].contiguous()
+                slots = tb[torch.arange(len(reqs), device=dev), last // bs].long() * bs + last % bs
+                md = types.SimpleNamespace(max_query_len=1, num_actual_tokens=len(reqs), use_cascade=False,
+                                           max_seq_len=max(lens), block_table=tb, slot_mapping=slots,
+                                           seq_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
+                k_new = torch.cat([probs[b][0][:, :, ctxs[b] + s - 1] for b in reqs])      # [R, H, D]
+                v_new = torch.cat([probs[b][1][:, :, ctxs[b] + s - 1] for b in reqs])
+                query = torch.cat([probs[b][2][0, :, s].reshape(1, H * G, DIM) for b in reqs])
+                out = torch.zeros(len(reqs), H * G, DIM, dtype=torch.bfloat16, device=dev)
+                res = impl.forward(layer, query, k_new, v_new, kvc, md, output=out)
+                assert res is out and float(out.float().abs().max()) != 7.0
+                outs.append(out.float().cpu().numpy())
+            return outs, dict(rt.STATS)
+        finally:
+            wrap.unwrap_forward(Impl)
+            rt.reset_pq_hsa_layer_state()
+
+    everyone = lambda s: [0, 1, 2]
+    one_leaves = lambda s: [0, 1, 2] if s < 4 else [0, 2]
+    for reqs_at, builds in ((everyone, 1), (one_leaves, 2)):
+        fused, st_f = run("1", reqs_at)
+        single, st_s = run("0", reqs_at)
+        assert st_f["pq_batch_fused_steps"] == steps + 1 and st_f["pq_batch_group_builds"] == builds
+        assert st_s["pq_batch_fused_steps"] == 0 and st_s["pq_build_calls"] >= 3
+        for s, (a, b) in enumerate(zip(fused, single)):
+            if len(reqs_at(s)) < B:
+                # the group was rebuilt for everyone, the per-request form rebuilt only the request
+                # that moved up a row: only that row still runs on an index trained on the same keys
+                a, b = a[1:], b[1:]
+            # the same kernels on the same trained indexes: only bf16 rounding of the output differs
+            assert np.abs(a - b).max() <= 2e-3 + 2.0 ** -7 * np.abs(b).max(), (s, np.abs(a - b).max())

@@ -306,3 +306,33 @@ def test_batched_index_training_equals_the_per_stream_procedure():
             torch.testing.assert_close(books[s], b1, rtol=0, atol=1e-6)
     with pytest.raises(ValueError):
         train_ivfpq_batched(keys[:, :0], num_lists=8)
+
+
+def test_batch_mode_per_request_sidecars(fake_stack, monkeypatch):
+    """PQ_HSA_BATCH=1 with PQ_HSA_BATCH_FUSED=0: one sidecar per request, built on first sight,
+    appended to while the request advances by one token, rebuilt when it does not."""
+    impl, layer, kv_cache = fake_stack
+    monkeypatch.setenv("PQ_HSA_ENABLE", "1")
+    monkeypatch.setenv("PQ_HSA_BATCH", "1")
+    monkeypatch.setenv("PQ_HSA_BATCH_FUSED", "0")
+
+    def batch_step(lens):
+        n = len(lens)
+        md = meta(seq_len=max(lens), reqs=n, tokens=n)
+        md.seq_lens = torch.tensor(lens, dtype=torch.int32)
+        out = torch.zeros(n, 8, 128)
+        q, k, v = torch.zeros(n, 8, 128), torch.zeros(n, 2, 128), torch.zeros(n, 2, 128)
+        return rt.pq_or_dense_forward(impl, layer, q, k, v, kv_cache, md, out, lambda: torch.full((n, 8, 128), -1.0))
+
+    monkeypatch.setattr(rt, "gather_flashattn_kv",
+                        lambda kv, md, i=0: (torch.zeros(1, 2, int(md.seq_lens[i]), 128),
+                                             torch.zeros(1, 2, int(md.seq_lens[i]), 128), int(md.seq_lens[i])))
+    res = batch_step([500, 300, 400])
+    assert [float(res[r, 0, 0]) for r in range(3)] == [500.0, 300.0, 400.0] and FakeSidecar.built == 3
+    res = batch_step([501, 301, 401])
+    assert [float(res[r, 0, 0]) for r in range(3)] == [501.0, 301.0, 401.0] and FakeSidecar.built == 3
+    res = batch_step([502, 350])                      # request 1 is a different one now, request 2 left
+    assert [float(res[r, 0, 0]) for r in range(2)] == [502.0, 350.0] and FakeSidecar.built == 4
+    assert sorted(rt.state_for(impl, layer)["batch"]) == [0, 1]
+    assert rt.STATS["pq_batch_steps"] == 3 and rt.STATS["pq_batch_reqs_total"] == 8
+    assert rt.STATS["pq_batch_fused_steps"] == 0
