@@ -316,45 +316,68 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     }
 }
 
+constexpr int kRedLanes = 4;  // split partials are folded four at a time (512 threads)
+
 template <int QDT>
-__global__ __launch_bounds__(kD) void attend_reduce_kernel(AttendArgs a) {
-    const int d = threadIdx.x;
+__global__ __launch_bounds__(kD * kRedLanes) void attend_reduce_kernel(AttendArgs a) {
+    __shared__ float head_s[3];                 // row maximum, mass sums of the two background parts
+    __shared__ float acc_s[kRedLanes][kD];
+    __shared__ float den_s[kRedLanes];
+    const int tid = threadIdx.x;
+    const int d = tid & (kD - 1), sl = tid / kD;
     const int g = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.H, h = bh % a.H;
     const size_t orow = (size_t)bh * a.G + g;
     const int n = a.n_idx[b];
-    if (a.n_commit_dst && g == 0 && h == 0 && d == 0) a.n_commit_dst[b] = a.n_commit_src[b];
+    if (a.n_commit_dst && g == 0 && h == 0 && tid == 0) a.n_commit_dst[b] = a.n_commit_src[b];
     const float *part = a.partials + orow * a.splits * kPartWidth;
     const float r0 = (n > 0 && a.mass0) ? a.ref0[(size_t)bh * a.ref_stride + g] : -INFINITY;
     const float r1 = (n > 0 && a.mass1) ? a.ref1[(size_t)bh * a.ref_stride + g] : -INFINITY;
-    float ms0 = 0.0f, ms1 = 0.0f;
-    float m = -INFINITY;
-#pragma unroll 8
-    for (int s = 0; s < a.splits; ++s) {  // independent loads: several splits in flight at once
-        m = fmaxf(m, part[s * kPartWidth]);
-        ms0 += part[s * kPartWidth + 2];
-        ms1 += part[s * kPartWidth + 3];
+    // the first wave takes one split per lane (at most 64 splits): maximum and mass sums
+    if (tid < kWave) {
+        float m = -INFINITY, ms0 = 0.0f, ms1 = 0.0f;
+        if (tid < a.splits) {
+            m = part[tid * kPartWidth];
+            ms0 = part[tid * kPartWidth + 2];
+            ms1 = part[tid * kPartWidth + 3];
+        }
+        m = wave_max(m);
+        ms0 = wave_sum(ms0);
+        ms1 = wave_sum(ms1);
+        if (tid == 0) { head_s[0] = m; head_s[1] = ms0; head_s[2] = ms1; }
     }
+    __syncthreads();
+    float m = head_s[0];
+    const float ms0 = head_s[1], ms1 = head_s[2];
     // a background part only matters (and only bounds the maximum) when it holds any weight
     if (ms0 != 0.0f && r0 > -INFINITY) m = fmaxf(m, r0);
     if (ms1 != 0.0f && r1 > -INFINITY) m = fmaxf(m, r1);
     const size_t qesz = QDT == PQHSA_F32 ? 4 : 2;
     char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
     if (m == -INFINITY) {  // nothing to attend to
-        store1<QDT>(orow_p, d, 0.0f);
+        if (sl == 0) store1<QDT>(orow_p, d, 0.0f);
         return;
     }
     const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
     const float f1 = (ms1 != 0.0f && r1 > -INFINITY) ? __expf(r1 - m) : 0.0f;
     float acc = 0.0f, den = 0.0f;
-#pragma unroll 8
-    for (int s = 0; s < a.splits; ++s) {
+#pragma unroll 4
+    for (int s = sl; s < a.splits; s += kRedLanes) {  // independent loads: several splits in flight at once
         const float *p = part + s * kPartWidth;
         const float w = p[0] == -INFINITY ? 0.0f : __expf(p[0] - m);
         den = __builtin_fmaf(p[1], w, den);
         acc = __builtin_fmaf(p[4 + d], w, acc);
         acc = __builtin_fmaf(p[4 + kD + d], f0, acc);
         acc = __builtin_fmaf(p[4 + 2 * kD + d], f1, acc);
+    }
+    acc_s[sl][d] = acc;
+    if (d == 0) den_s[sl] = den;
+    __syncthreads();
+    if (sl != 0) return;
+#pragma unroll
+    for (int r = 1; r < kRedLanes; ++r) {
+        acc += acc_s[r][d];
+        den += den_s[r];
     }
     den += ms0 * f0 + ms1 * f1;
     den = fmaxf(den, FLT_MIN);
@@ -435,7 +458,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     int rc = check_launch("attend_partial");
     if (rc) return rc;
     if (mark) profile_mark(kProfReduce, stream);
-    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kD), 0, stream, a));
+    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kD * kRedLanes), 0, stream, a));
     if (mark) profile_mark(kProfKernels, stream);
     return check_launch("attend_reduce");
 }
