@@ -14,14 +14,14 @@
 
 namespace pqhsa {
 
-constexpr int kLutThreads = 256;
+constexpr int kLutThreads = 256;  // at least; one wave per padded query row when the group is wider than 4
 constexpr int kListsPerBlock = 64;
 constexpr int kMaxG = 16;
 
 int lut_list_blocks(int num_lists);
 
 template <int DT>
-__global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
+__global__ __launch_bounds__(1024) void lut_build_kernel(
     const char *__restrict__ q, int H, int G, int Gp, const float *__restrict__ coarse,
     const float *__restrict__ codebooks, int L, float eps, float *__restrict__ qnorm,
     float *__restrict__ lut, float *__restrict__ list_scores, uint32_t *__restrict__ zero_base,
@@ -33,6 +33,7 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
     __shared__ float cs[kListsPerBlock][kD + 1];
 
     const int tid = threadIdx.x;
+    const int nthr = blockDim.x;
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
 
@@ -45,15 +46,15 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         const float4 *c4 = reinterpret_cast<const float4 *>(coarse + ((size_t)bh * L + l0) * kD);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const int i = tid + u * kLutThreads;
+            const int i = tid + u * nthr;
             tile[u] = i < nl * (kD / 4) ? c4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
     }
 
     // scratch that the later kernels of a decode step accumulate into starts at zero
     if (zero_words) {
-        const size_t nthreads = (size_t)gridDim.x * gridDim.y * kLutThreads;
-        const size_t me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kLutThreads + tid;
+        const size_t nthreads = (size_t)gridDim.x * gridDim.y * nthr;
+        const size_t me = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * nthr + tid;
         for (size_t i = me; i < zero_words; i += nthreads) zero_base[i] = 0u;
     }
 
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
     // query rows of this stream: q[b, h*G + g, :]
     const size_t esz = DT == PQHSA_F32 ? 4 : 2;
     const char *qrow0 = q + ((size_t)b * H * G + (size_t)h * G) * kD * esz;
-    for (int i = tid; i < G * kD; i += kLutThreads) {
+    for (int i = tid; i < G * kD; i += nthr) {
         int g = i / kD, d = i % kD;
         qh[g][d] = load1<DT>(qrow0 + (size_t)g * kD * esz, d);
     }
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         kn_s = n < ap.enc.eps ? ap.enc.eps : n;
     }
     __syncthreads();
-    for (int i = tid; i < G * kD; i += kLutThreads) {
+    for (int i = tid; i < G * kD; i += nthr) {
         int g = i / kD, d = i % kD;
         qh[g][d] = qh[g][d] / qn[g];
     }
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
         if (tid < Gp) qnorm[(size_t)bh * Gp + tid] = tid < G ? qn[tid] : 0.0f;
         const float *cb = codebooks + (size_t)bh * kM * kCodes * kSub;
         float *out = lut + (size_t)bh * kM * kCodes * Gp;
-        for (int e = tid; e < kM * kCodes * Gp; e += kLutThreads) {
+        for (int e = tid; e < kM * kCodes * Gp; e += nthr) {
             int g = e % Gp;
             int mc = e / Gp;  // m * 16 + c
             float acc = 0.0f;
@@ -115,7 +116,8 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
 
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        const int i = tid + u * kLutThreads;
+        const int i = tid + u * nthr;
+        if (i >= kListsPerBlock * (kD / 4)) break;  // wider workgroups need fewer rounds
         float *dst = &cs[i / (kD / 4)][(i % (kD / 4)) * 4];
         dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
     }
@@ -123,7 +125,7 @@ __global__ __launch_bounds__(kLutThreads) void lut_build_kernel(
     const int lane = tid % kListsPerBlock;
     const int wave = tid / kListsPerBlock;
     float *out = list_scores + ((size_t)bh * L + l0) * Gp;
-    for (int g = wave; g < Gp; g += kLutThreads / kListsPerBlock) {
+    for (int g = wave; g < Gp; g += nthr / kListsPerBlock) {
         if (lane >= nl) continue;
         float acc = 0.0f;
         if (g < G) {
@@ -166,7 +168,8 @@ int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G
         ap = *append;
     }
     dim3 grid(1 + lut_list_blocks(index->num_lists), BH);
-    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(lut_build_kernel<DT>, grid, dim3(kLutThreads), 0, stream,
+    const int threads = Gp * kWave > kLutThreads ? Gp * kWave : kLutThreads;  // a wave per padded query row
+    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(lut_build_kernel<DT>, grid, dim3(threads), 0, stream,
                                                      static_cast<const char *>(q), index->kv_heads, G, Gp,
                                                      index->coarse, index->codebooks, index->num_lists, eps,
                                                      qnorm, lut, list_scores, zero_base, zero_words, ap, n_after,
