@@ -479,3 +479,43 @@ def test_device_counts_ahead_of_the_host_stay_inside_k_cap():
     assert ws.topk_cnt.cpu().tolist() == [k_cap] * p.G
     got = ws.topk_idx.cpu().numpy()
     assert ((got >= 0) & (got < n)).all() and bool(torch.isfinite(out).all())
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_decode_step_random_shapes_match_oracle(seed):
+    """A seeded sweep over batch sizes, ragged lengths, group widths, list counts, dtypes, page
+    layouts, selection fractions and sorted / insertion-order layouts: top-k sets bit-exact,
+    outputs within the stated bound (plus the output's own rounding for 16-bit queries)."""
+    import random
+
+    dev = _cuda()
+    rng = random.Random(seed)
+    for case in range(6):
+        lens = [rng.randint(300, rng.choice([3000, 12000, 30000])) for _ in range(rng.choice([1, 2, 3]))]
+        heads, groups = rng.choice([1, 2]), rng.choice([1, 2, 3, 4, 5, 7, 8])
+        lists = rng.choice([16, 32, 64, 128])
+        dtype = rng.choice([torch.float32, torch.bfloat16, torch.float16])
+        fraction = rng.choice([0.01, 0.02, 0.05, 0.1, 0.3])
+        layout = rng.choice(["dense", "5d", "4d"])
+        finalize = rng.random() < 0.75
+        what = (seed, case, lens, heads, groups, lists, dtype, fraction, layout, finalize)
+        p = Problem(lens=lens, heads=heads, groups=groups, lists=lists, dtype=dtype, seed=500 + 10 * seed + case)
+        idx = p.device_index(dev, finalize=finalize)
+        kv = ops.kv_contiguous(*p.dense_kv()) if layout == "dense" else ops.kv_paged(*p.paged_kv(layout))
+        ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, fraction, 0))
+        q = p.q_tensor()
+        out = torch.empty_like(q)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
+                        fraction=fraction, topk=0, scale=SCALE, workspace=ws)
+        torch.cuda.synchronize()
+        tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        tol = 1e-4 if dtype == torch.float32 else 2e-3
+        rel = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+        for (b, h) in p.index:
+            want_out, want_idx, _ = p.oracle_step(b, h, fraction)
+            k = want_idx.shape[1]
+            for g in range(p.G):
+                assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (what, b, h, g)
+            assert (np.abs(o[b, h] - want_out) <= tol + rel * np.abs(want_out)).all(), (what, b, h)
+        assert ws.rescans() == 0, what
