@@ -519,3 +519,27 @@ def test_decode_step_random_shapes_match_oracle(seed):
                 assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (what, b, h, g)
             assert (np.abs(o[b, h] - want_out) <= tol + rel * np.abs(want_out)).all(), (what, b, h)
         assert ws.rescans() == 0, what
+
+
+@pytest.mark.parametrize("groups,lists,lens", [(16, 64, [2600]), (12, 256, [5000, 1700]), (9, 512, [7000])])
+def test_decode_step_wide_groups_and_many_lists(groups, lists, lens):
+    """Query groups of 9 to 16 rows (padded to 16 in the kernels) and list counts up to the
+    headline configuration's 512, against the oracle."""
+    dev = _cuda()
+    p = Problem(lens=lens, heads=1, groups=groups, lists=lists, dtype=torch.bfloat16, seed=61)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.05, 0))
+    q = p.q_tensor().float()
+    out = torch.empty_like(q)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.05,
+                    topk=0, scale=SCALE, workspace=ws)
+    torch.cuda.synchronize()
+    tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+    o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    for (b, h) in p.index:
+        want_out, want_idx, _ = p.oracle_step(b, h, 0.05)
+        k = want_idx.shape[1]
+        for g in range(p.G):
+            assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (b, h, g)
+        assert np.abs(o[b, h] - want_out).max() <= 2e-3, (b, h)
