@@ -529,12 +529,12 @@ __device__ inline uint32_t bisect_regs(const uint32_t (&key)[R], uint32_t want, 
     return t;
 }
 
-// The leading bits that all keys of the workgroup share, keys equal to PAD aside: returns the
-// shared prefix and, in bit0, the highest bit in which two keys differ (-1: all equal, or none).
+// Smallest and largest key of the workgroup, keys equal to PAD aside (lo > hi: there are none).
 // One barrier; `span` holds 2 * kSelWaves words that nothing else uses until the next barrier.
 template <uint32_t PAD, int R>
-__device__ inline uint32_t shared_prefix(const uint32_t (&key)[R], uint32_t *span, int &bit0) {
-    uint32_t hi = 0u, lo = 0xffffffffu;
+__device__ inline void block_min_max(const uint32_t (&key)[R], uint32_t *span, uint32_t &lo, uint32_t &hi) {
+    hi = 0u;
+    lo = 0xffffffffu;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         hi = max(hi, key[r] != PAD ? key[r] : 0u);
@@ -553,13 +553,31 @@ __device__ inline uint32_t shared_prefix(const uint32_t (&key)[R], uint32_t *spa
         hi = max(hi, span[w]);
         lo = min(lo, span[kSelWaves + w]);
     }
-    if (lo >= hi) {  // all equal, or no keys at all
+}
+
+// The leading bits that all keys between lo and hi share: returns the shared prefix and, in
+// bit0, the highest bit in which the two differ (-1: lo >= hi, all keys equal or none).
+__device__ inline uint32_t shared_prefix(uint32_t lo, uint32_t hi, int &bit0) {
+    if (lo >= hi) {
         bit0 = -1;
         return hi;
     }
     bit0 = 31 - __clz(hi ^ lo);
     return bit0 == 31 ? 0u : hi & ~((2u << bit0) - 1u);
 }
+
+// Scratch of the bucket selection: a histogram of the candidates over 1024 equal key ranges
+// between the smallest and the largest candidate, and the candidates of the one range in which
+// the k-th largest falls.
+constexpr int kSelBins = 1024;
+struct SelScratch {
+    uint32_t hist[kSelBins];
+    uint32_t cont_key[kSelBins];
+    uint32_t cont_idx[kSelBins];
+    uint32_t cont_count;
+    uint32_t bin, above;        // the range of the k-th key and the number of keys in higher ranges
+    uint32_t sel_key, sel_idx;  // the k-th key and, among equal keys, the largest index still selected
+};
 
 // The same search over keys in memory (any count).
 template <typename KeyAt>
@@ -765,17 +783,69 @@ struct SelectOut {
 template <int R>
 __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
                                      int k, SelectOut out, uint32_t (*red)[kSelWaves],
-                                     uint32_t *wsum, float *ref1_out) {
+                                     uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     const int tid = threadIdx.x;
     int step = 0;
     bool exact = false;
     uint32_t tkey = 0u;
+    uint32_t idx_thr = 0xffffffffu;
+    bool ties = false;
+    bool searched = false;
+    uint32_t lo_key = 0u, hi_key = 0u;
     if (k > 0) {
-        // candidates all lie between the threshold and the row maximum: their keys share the leading
-        // bits, which the search need not visit
-        int bit0;
-        const uint32_t t0 = shared_prefix<0u>(key, wsum, bit0);
-        tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact, t0, bit0);
+        // Candidates lie between the threshold and the row maximum.  Histogram them over 1024
+        // equal ranges of that span, find the range that holds the k-th largest (one wave), and
+        // rank the few candidates of that range against each other, equal keys by index: five
+        // barriers where a bit-by-bit search takes one per bit.
+        block_min_max<0u>(key, wsum, lo_key, hi_key);
+        const uint32_t range = hi_key >= lo_key ? hi_key - lo_key : 0u;
+        const int shift = range < (uint32_t)kSelBins ? 0 : (31 - __clz(range)) - 9;
+        uint32_t bucket[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            bucket[r] = key[r] != 0u ? (key[r] - lo_key) >> shift : 0xffffffffu;
+            if (key[r] != 0u) atomicAdd(&ss->hist[bucket[r]], 1u);
+        }
+        if (tid == 0) ss->bin = 0xffffffffu;
+        __syncthreads();
+        if (tid < kWave) find_from_top(ss->hist, kSelBins, (uint32_t)k, &ss->bin, &ss->above);
+        __syncthreads();
+        const uint32_t bin = ss->bin;
+        const uint32_t crowd = bin < (uint32_t)kSelBins ? ss->hist[bin] : 0u;
+        if (bin >= (uint32_t)kSelBins) {  // fewer than k candidates: all of them are selected
+            tkey = lo_key <= hi_key ? lo_key : 0u;
+            searched = true;
+        } else if (crowd <= (uint32_t)kSelBins) {
+            const uint32_t need = (uint32_t)k - ss->above;  // 1-based rank of the k-th key inside its range
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (bucket[r] != bin) continue;
+                const uint32_t slot = atomicAdd(&ss->cont_count, 1u);
+                ss->cont_key[slot] = key[r];
+                ss->cont_idx[slot] = where[r];
+            }
+            __syncthreads();
+            if ((uint32_t)tid < crowd) {
+                const uint32_t mk = ss->cont_key[tid], mi = ss->cont_idx[tid];
+                uint32_t ahead = 0;  // candidates of the range that come before this one: larger key, or equal key and lower index
+                for (uint32_t j = 0; j < crowd; ++j) {
+                    const uint32_t kj = ss->cont_key[j], ij = ss->cont_idx[j];
+                    ahead += (kj > mk || (kj == mk && ij < mi)) ? 1u : 0u;
+                }
+                if (ahead == need - 1u) {
+                    ss->sel_key = mk;
+                    ss->sel_idx = mi;
+                }
+            }
+            __syncthreads();
+            tkey = ss->sel_key;
+            idx_thr = ss->sel_idx;
+            ties = true;  // equal keys with a higher index lose: fold the rule into the keys
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (key[r] == tkey && where[r] > idx_thr) key[r] = tkey - 1u, where[r] |= 0x80000000u;
+            searched = true;
+        }
     } else {  // nothing is selected: the reference of the losers' weights is the largest key
         uint32_t kmax = 0u;
 #pragma unroll
@@ -786,40 +856,45 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         __syncthreads();
         for (int w = 0; w < kSelWaves; ++w) tkey = max(tkey, wsum[w]);
     }
-    // ties at the boundary (only when the search ran to the last bit): keep the lowest indices
-    uint32_t idx_thr = 0xffffffffu;
-    bool ties = false;
-    if (k > 0 && !exact) {
-        uint32_t c_gt = 0, c_eq = 0;
+    if (k > 0 && !searched) {
+        // more than 1024 candidates in the k-th key's range (many equal keys): bit-by-bit search
+        // below the leading bits that all candidates share
+        int bit0;
+        const uint32_t t0 = shared_prefix(lo_key, hi_key, bit0);
+        tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact, t0, bit0);
+        if (!exact) {  // ties at the boundary: keep the lowest indices
+            uint32_t c_gt = 0, c_eq = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            c_gt += wave_count_if(key[r] > tkey);
-            c_eq += wave_count_if(key[r] == tkey);
-        }
-        c_gt = block_total_of_waves(c_gt, red, step++);
-        c_eq = block_total_of_waves(c_eq, red, step++);
-        const uint32_t want_ties = (uint32_t)k - c_gt;
-        if (c_eq > want_ties) {
-            // largest I with count(key == T && index < I) < want_ties: the want_ties-th lowest tie index
-            ties = true;
-            uint32_t tidx[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                tidx[r] = key[r] == tkey ? where[r] : 0xffffffffu;
-            int bit1;
-            uint32_t lo = shared_prefix<0xffffffffu>(tidx, wsum, bit1);  // the tied indices' common leading bits
-            for (int bit = bit1; bit >= 0; --bit) {
-                const uint32_t trial = lo | (1u << bit);
-                uint32_t c = 0;
-#pragma unroll
-                for (int r = 0; r < R; ++r) c += wave_count_if(tidx[r] < trial);
-                c = block_total_of_waves(c, red, step++);
-                if (c < want_ties) lo = trial;
+            for (int r = 0; r < R; ++r) {
+                c_gt += wave_count_if(key[r] > tkey);
+                c_eq += wave_count_if(key[r] == tkey);
             }
-            idx_thr = lo;
+            c_gt = block_total_of_waves(c_gt, red, step++);
+            c_eq = block_total_of_waves(c_eq, red, step++);
+            const uint32_t want_ties = (uint32_t)k - c_gt;
+            if (c_eq > want_ties) {
+                // largest I with count(key == T && index < I) < want_ties: the want_ties-th lowest tie index
+                ties = true;
+                uint32_t tidx[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r)  // fold the tie rule into the keys: losers of the tie drop below T
-                if (key[r] == tkey && tidx[r] > idx_thr) key[r] = tkey - 1u, where[r] |= 0x80000000u;
+                for (int r = 0; r < R; ++r) tidx[r] = key[r] == tkey ? where[r] : 0xffffffffu;
+                uint32_t tlo, thi;
+                block_min_max<0xffffffffu>(tidx, wsum, tlo, thi);
+                int bit1;
+                uint32_t lo = shared_prefix(tlo, thi, bit1);  // the tied indices' common leading bits
+                for (int bit = bit1; bit >= 0; --bit) {
+                    const uint32_t trial = lo | (1u << bit);
+                    uint32_t c = 0;
+#pragma unroll
+                    for (int r = 0; r < R; ++r) c += wave_count_if(tidx[r] < trial);
+                    c = block_total_of_waves(c, red, step++);
+                    if (c < want_ties) lo = trial;
+                }
+                idx_thr = lo;
+#pragma unroll
+                for (int r = 0; r < R; ++r)  // fold the tie rule into the keys: losers of the tie drop below T
+                    if (key[r] == tkey && tidx[r] > idx_thr) key[r] = tkey - 1u, where[r] |= 0x80000000u;
+            }
         }
     }
     out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
@@ -858,7 +933,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
 template <int R>
 __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
                                    SelectOut out, uint32_t (*red)[kSelWaves],
-                                   uint32_t *wsum, float *ref1_out) {
+                                   uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     uint32_t key[R], where[R], list[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
@@ -868,7 +943,7 @@ __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, cons
         where[r] = pr.y;
         list[r] = (aux && p < cnt) ? aux[p] : 0u;
     }
-    select_loaded<R>(key, where, list, cnt, k, out, red, wsum, ref1_out);
+    select_loaded<R>(key, where, list, cnt, k, out, red, wsum, ss, ref1_out);
 }
 
 // Candidates in memory (any count): the same selection, streaming the pairs on every pass.
@@ -952,6 +1027,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
     __shared__ uint32_t wsum[2 * kSelWaves];
+    __shared__ SelScratch ss;
     float *mx = reinterpret_cast<float *>(smem);  // [L] (the re-scan parks its [128 + L] tables here first)
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
@@ -1007,6 +1083,8 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
 
     if (mass_out)
         for (int l = tid; l < a.L; l += kSelThreads) mx[l] = 0.0f;
+    for (int i = tid; i < kSelBins; i += kSelThreads) ss.hist[i] = 0u;
+    if (tid == 0) ss.cont_count = 0u;
     __syncthreads();
     SelectOut out;
     out.out_idx = a.topk_idx + orow * a.k_cap;
@@ -1022,15 +1100,15 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             for (int r = 0; r < RS; ++r) {
                 if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, swhere[r] = 0u, slist[r] = 0u;
             }
-            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ref1);
+            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1);
             done = true;
         }
     }
     if (!done) {
         if constexpr (RS == 0) {  // no estimate: pick the register variant from the count
-            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, out, red, wsum, &ref1);
-            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, out, red, wsum, &ref1);
-            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, out, red, wsum, &ref1);
+            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
             else select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
         } else {  // the estimate was exceeded, or the row was re-scanned (rare): stream from memory
             select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
