@@ -89,16 +89,6 @@ __device__ inline void lds_vec(const float *p, float (&v)[GP]) {
     }
 }
 
-__device__ inline uint32_t wave_incl_scan_u32(uint32_t v) {
-    const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const uint32_t o = (uint32_t)__shfl_up((int)v, off, kWave);
-        if (lane >= off) v += o;
-    }
-    return v;
-}
-
 // logit of one stored key for one query row, in the fixed summation order of the CPU oracle
 __device__ inline float score_one(const float *lut_col, const float *ls_col, uint32_t code, uint32_t lid, float qn,
                                   float kn, float scale) {
@@ -437,7 +427,7 @@ __device__ inline void find_from_top(const uint32_t *hist, int nbins, uint32_t w
     const int top = nbins - 1 - lane * per;  // lane 0 owns the highest bins
     uint32_t mine = 0;
     for (int t = 0; t < per; ++t) mine += hist[top - t];
-    const uint32_t incl = wave_incl_scan_u32(mine);
+    const uint32_t incl = wave_prefix_u32(mine);
     const uint32_t excl = incl - mine;
     if (want > 0 && excl < want && want <= incl) {
         uint32_t c = excl;
@@ -825,14 +815,20 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
                 ss->cont_idx[slot] = where[r];
             }
             __syncthreads();
-            if ((uint32_t)tid < crowd) {
-                const uint32_t mk = ss->cont_key[tid], mi = ss->cont_idx[tid];
-                uint32_t ahead = 0;  // candidates of the range that come before this one: larger key, or equal key and lower index
-                for (uint32_t j = 0; j < crowd; ++j) {
-                    const uint32_t kj = ss->cont_key[j], ij = ss->cont_idx[j];
-                    ahead += (kj > mk || (kj == mk && ij < mi)) ? 1u : 0u;
+            // wave w ranks candidates w, w + 16, ... of the range: its lanes each hold one candidate
+            // of the range and vote on whether it comes before (larger key, or equal key and lower
+            // index); the candidate with need - 1 others before it is the k-th key
+            const int lane = tid & (kWave - 1);
+            for (uint32_t i = (uint32_t)tid / kWave; i < crowd; i += kSelWaves) {
+                const uint32_t mk = ss->cont_key[i], mi = ss->cont_idx[i];
+                uint32_t ahead = 0;
+                for (uint32_t j0 = 0; j0 < crowd; j0 += kWave) {
+                    const uint32_t j = j0 + lane;
+                    const uint32_t kj = j < crowd ? ss->cont_key[j] : 0u;
+                    const uint32_t ij = j < crowd ? ss->cont_idx[j] : 0u;
+                    ahead += wave_count_if(j < crowd && (kj > mk || (kj == mk && ij < mi)));
                 }
-                if (ahead == need - 1u) {
+                if (lane == 0 && ahead == need - 1u) {
                     ss->sel_key = mk;
                     ss->sel_idx = mi;
                 }
