@@ -628,6 +628,9 @@ template <int R>
 __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
+    __shared__ uint32_t wsum[2 * kSelWaves];
+    __shared__ uint32_t hist[kSelBins];
+    __shared__ uint32_t found[2];
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
     const int bh = blockIdx.y;
@@ -682,6 +685,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         return;
     }
     const uint32_t want = (uint32_t)want_d;
+    for (int i = tid; i < kSelBins; i += kSelThreads) hist[i] = 0u;
     __syncthreads();
     uint32_t key[R];
 #pragma unroll
@@ -694,10 +698,32 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
             key[r0 + r] = p < ns ? max(order_key(score_one(lut_s, ls_s, code[r], lid[r], qn, kn[r], a.scale)), 1u) : 0u;
         }
     }
-    int step = 0;
-    bool exact;
-    // any threshold that keeps between want and 9/8 want sampled keys serves: fewer search steps
-    const uint32_t t = bisect_regs<R>(key, want, want / 8u, red, step, exact);
+    // Any threshold that keeps between want and 9/8 want sampled keys serves.  The want-th largest
+    // sampled logit is normally within a factor 16 of the largest: histogram the keys of that
+    // window (four exponent steps below the largest key) over 1024 equal ranges and take the
+    // lower edge of the range that holds the want-th largest (one wave finds it).  If the window
+    // holds fewer than want keys, or that range is crowded, the bit-by-bit search takes over.
+    uint32_t lo_key, hi_key;
+    block_min_max<0u>(key, wsum, lo_key, hi_key);
+    constexpr uint32_t kWindow = 1u << 25;
+    const uint32_t wbase = hi_key > kWindow ? max(hi_key - kWindow, lo_key) : lo_key;
+    const uint32_t range = hi_key >= wbase ? hi_key - wbase : 0u;
+    const int shift = range < (uint32_t)kSelBins ? 0 : (31 - __clz(range)) - 9;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        if (key[r] != 0u && key[r] >= wbase) atomicAdd(&hist[(key[r] - wbase) >> shift], 1u);
+    if (tid == 0) found[0] = 0xffffffffu;
+    __syncthreads();
+    if (tid < kWave) find_from_top(hist, kSelBins, want, &found[0], &found[1]);
+    __syncthreads();
+    uint32_t t;
+    if (found[0] < (uint32_t)kSelBins && hist[found[0]] <= max(want / 8u, 16u)) {
+        t = wbase + (found[0] << shift);
+    } else {
+        int step = 0;
+        bool exact;
+        t = bisect_regs<R>(key, want, want / 8u, red, step, exact);
+    }
     if (tid == 0) {
         a.thr_key[row] = t;
         a.k_row[row] = k;
