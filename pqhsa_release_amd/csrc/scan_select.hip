@@ -468,6 +468,38 @@ __global__ __launch_bounds__(kWave) void thresh_kernel(const uint32_t *__restric
     }
 }
 
+// The same search for a 1024-bin histogram in LDS (16-byte aligned): every lane takes 16
+// neighbouring bins with four 128-bit reads and keeps them in registers; lane 63 owns the top.
+__device__ inline void find_from_top_1024(const uint32_t *hist, uint32_t want, uint32_t *out_bin,
+                                          uint32_t *out_above) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t h[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint4 v = reinterpret_cast<const uint4 *>(hist)[lane * 4 + q];
+        h[4 * q] = v.x; h[4 * q + 1] = v.y; h[4 * q + 2] = v.z; h[4 * q + 3] = v.w;
+    }
+    uint32_t mine = 0;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) mine += h[t];
+    const uint32_t incl = wave_prefix_u32(mine);
+    const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    const uint32_t above_me = total - incl;  // keys in the bins of higher lanes
+    if (want > 0 && above_me < want && want <= above_me + mine) {
+        uint32_t c = above_me;
+#pragma unroll
+        for (int t = 15; t >= 0; --t) {
+            const uint32_t c2 = c + h[t];
+            if (c2 >= want) {
+                *out_bin = (uint32_t)(lane * 16 + t);
+                *out_above = c;
+                break;
+            }
+            c = c2;
+        }
+    }
+}
+
 // ---- block-wide helpers of the selection kernels (1024 threads, all active) -----------------
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / kWave;
@@ -559,8 +591,8 @@ __device__ inline uint32_t shared_prefix(uint32_t lo, uint32_t hi, int &bit0) {
 // Scratch of the bucket selection: a histogram of the candidates over 1024 equal key ranges
 // between the smallest and the largest candidate, and the candidates of the one range in which
 // the k-th largest falls.
-constexpr int kSelBins = 1024;
-struct SelScratch {
+constexpr int kSelBins = 1024;  // find_from_top_1024 is written for this count
+struct __align__(16) SelScratch {
     uint32_t hist[kSelBins];
     uint32_t cont_key[kSelBins];
     uint32_t cont_idx[kSelBins];
@@ -629,7 +661,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
     __shared__ uint32_t wsum[2 * kSelWaves];
-    __shared__ uint32_t hist[kSelBins];
+    __shared__ __align__(16) uint32_t hist[kSelBins];
     __shared__ uint32_t found[2];
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
@@ -714,7 +746,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         if (key[r] != 0u && key[r] >= wbase) atomicAdd(&hist[(key[r] - wbase) >> shift], 1u);
     if (tid == 0) found[0] = 0xffffffffu;
     __syncthreads();
-    if (tid < kWave) find_from_top(hist, kSelBins, want, &found[0], &found[1]);
+    if (tid < kWave) find_from_top_1024(hist, want, &found[0], &found[1]);
     __syncthreads();
     uint32_t t;
     if (found[0] < (uint32_t)kSelBins && hist[found[0]] <= max(want / 8u, 16u)) {
@@ -824,7 +856,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         }
         if (tid == 0) ss->bin = 0xffffffffu;
         __syncthreads();
-        if (tid < kWave) find_from_top(ss->hist, kSelBins, (uint32_t)k, &ss->bin, &ss->above);
+        if (tid < kWave) find_from_top_1024(ss->hist, (uint32_t)k, &ss->bin, &ss->above);
         __syncthreads();
         const uint32_t bin = ss->bin;
         const uint32_t crowd = bin < (uint32_t)kSelBins ? ss->hist[bin] : 0u;
