@@ -385,11 +385,22 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             for (int g = 0; g < GP; ++g) wcnt_s[wave * GP + g] = wcnt[g];
         }
         __syncthreads();
+        // the reservation's round trip to memory overlaps the flush of the per-list sums
+        uint32_t at = 0;
         if (tid < GP) {
             uint32_t total = 0;
 #pragma unroll
             for (int w = 0; w < kScanWaves; ++w) total += wcnt_s[w * GP + tid];
-            uint32_t at = total ? atomicAdd(&a.emit_count[(size_t)bh * GP + tid], total) : 0u;
+            at = total ? atomicAdd(&a.emit_count[(size_t)bh * GP + tid], total) : 0u;
+        }
+        if (want_mass) {
+            float *dst = a.mass + (size_t)bh * L * GP;
+            for (int i = tid; i < L * GP; i += kScanThreads) {
+                const float v = mass_s[i];
+                if (v != 0.0f) unsafeAtomicAdd(&dst[i], v);
+            }
+        }
+        if (tid < GP) {
 #pragma unroll
             for (int w = 0; w < kScanWaves; ++w) {
                 base_s[w * GP + tid] = at;
@@ -405,13 +416,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             for (uint32_t i = lane; i < c; i += kWave) {
                 a.emit_pairs[o + i] = stage_s[srow + i];
                 if (a.emit_aux) a.emit_aux[o + i] = stage_aux[srow + i];
-            }
-        }
-        if (want_mass) {
-            float *dst = a.mass + (size_t)bh * L * GP;
-            for (int i = tid; i < L * GP; i += kScanThreads) {
-                const float v = mass_s[i];
-                if (v != 0.0f) unsafeAtomicAdd(&dst[i], v);
             }
         }
     }
