@@ -112,9 +112,13 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int L = a.L;
 
     // ---- LDS carve-up ----------------------------------------------------------------
-    float *lut_s = reinterpret_cast<float *>(smem);
-    float *ls_s = lut_s + (SRC == kIndex ? kM * kCodes * GP : 0);
-    const size_t table_bytes = SRC == kIndex ? (((size_t)(kM * kCodes + L) * GP * sizeof(float) + 15) & ~(size_t)15) : 0;
+    // The PQ table has a fixed size and sits in static LDS: its address is a constant, so the 32
+    // look-ups per lane and iteration fold the table offset into the instruction.  The list scores
+    // (L varies) lead the dynamic part.
+    __shared__ __align__(16) float lut_static[SRC == kIndex ? kM * kCodes * GP : 4];
+    float *lut_s = lut_static;
+    float *ls_s = reinterpret_cast<float *>(smem);
+    const size_t table_bytes = SRC == kIndex ? (((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15) : 0;
     unsigned char *after = smem + table_bytes;
     uint32_t *hist_s = reinterpret_cast<uint32_t *>(after);                // kHist: [GP][2048]
     float *mass_s = reinterpret_cast<float *>(after);                      // kEmit: [L][GP]
@@ -196,11 +200,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             constexpr int KB = GP <= 2 ? 4 : (GP == 4 ? 2 : 1);
 #pragma unroll
             for (int j0 = 0; j0 < 4; j0 += KB) {
-#pragma unroll
-                for (int j = j0; j < j0 + KB; ++j) {
-#pragma unroll
-                    for (int g = 0; g < GP; ++g) s[j][g] = 0.0f;
-                }
+                // the sum starts from the first entry: table entries are fma chains from +0 and never
+                // -0, so 0 + entry (the oracle's first step) is the entry itself
 #pragma unroll
                 for (int m = 0; m < kM; ++m) {
 #pragma unroll
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
                         float v[GP];
                         lds_vec<GP>(lut_s + (size_t)(m * kCodes + ((c[j] >> (4 * m)) & 15u)) * GP, v);
 #pragma unroll
-                        for (int g = 0; g < GP; ++g) s[j][g] = s[j][g] + v[g];
+                        for (int g = 0; g < GP; ++g) s[j][g] = m == 0 ? v[g] : s[j][g] + v[g];
                     }
                 }
 #pragma unroll
@@ -1197,7 +1198,7 @@ int launch_fill_zero(void *p, size_t bytes, hipStream_t stream) {
 // ---- host side --------------------------------------------------------------------------
 static size_t scan_lds_bytes(int GP, int L, int mode, int src, bool mass, bool aux, int stage_cap) {
     size_t b = 0;
-    if (src == kIndex) b += ((size_t)(kM * kCodes + L) * GP * sizeof(float) + 15) & ~(size_t)15;
+    if (src == kIndex) b += ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;  // the PQ table is static
     if (mode == kHist) b += (size_t)GP * kHistBins * sizeof(uint32_t);
     if (mode == kEmit) {
         if (mass) b += ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;
