@@ -543,3 +543,36 @@ def test_decode_step_wide_groups_and_many_lists(groups, lists, lens):
         for g in range(p.G):
             assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (b, h, g)
         assert np.abs(o[b, h] - want_out).max() <= 2e-3, (b, h)
+
+
+def test_topk_radix_on_tie_heavy_matrices():
+    """Logit matrices made to stress the selection's tie handling: quantised values (long runs of
+    equal logits on both sides of the k boundary), a handful of distinct values with both zeros,
+    constants, denormal-range values; k from 0 to n.  The index set must be the oracle's."""
+    dev = _cuda()
+    rng = np.random.default_rng(23)
+    for case, kind in enumerate(["quant1", "quant2", "few", "const", "mixed", "tiny", "quant1", "few"]):
+        rows, stride = int(rng.integers(2, 7)), int(rng.choice([300, 5000, 30000]))
+        x = rng.standard_normal((rows, stride)).astype(np.float32)
+        if kind == "quant1":
+            x = np.round(x, 1)
+        elif kind == "quant2":
+            x = np.round(x * 3) / 3
+        elif kind == "few":
+            x = rng.choice(np.array([-1.5, 0.0, -0.0, 2.25, 7.0], dtype=np.float32), size=(rows, stride))
+        elif kind == "const":
+            x[:] = 0.125
+        elif kind == "mixed":
+            x[:, ::3], x[:, 1::7] = np.float32(1.0), np.float32(-0.0)
+        elif kind == "tiny":
+            x *= np.float32(1e-30)
+        n = [int(rng.integers(1, stride + 1)) for _ in range(rows)]
+        k = [int(min(n[r], rng.choice([0, 1, 17, n[r] // 50 + 1, n[r] // 3 + 1, n[r]]))) for r in range(rows)]
+        idx, val = ops.topk_radix(torch.from_numpy(x).to(dev), n, k)
+        torch.cuda.synchronize()
+        idx, val = idx.cpu().numpy(), val.cpu().numpy()
+        for r in range(rows):
+            want_idx, _ = fixed.topk(x[r, : n[r]], k[r])
+            got = idx[r, : k[r]]
+            assert np.array_equal(np.sort(got), np.sort(want_idx)), (case, kind, r, n[r], k[r])
+            assert np.array_equal(val[r, : k[r]], x[r, got]), (case, kind, r)
