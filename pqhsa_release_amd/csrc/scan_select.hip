@@ -14,13 +14,15 @@
 //           straight to memory.  Stored keys are ordered by list, so the per-list sums are
 //           wave-level segment sums with one LDS update per (wave, list) instead of one per key.
 // sample_thresh_kernel scores a fixed random subset of the stored keys and takes, as the
-// threshold, the sampled key whose rank keeps, with a wide safety margin, more than k keys of the
-// full row; select_final_kernel finds the exact k-th largest key among the candidates by
-// bisection on the 32-bit key, below the leading bits that all candidates share (ties at the
-// boundary go to the lowest index), compacts the winners, and returns the losers' weights to
-// their lists.  A row whose estimate kept fewer than
-// k candidates is re-scanned in full by its select workgroup, so the result is always the exact
-// top-k.
+// threshold, a sampled key whose rank keeps, with a wide safety margin, more than k keys of the
+// full row.  select_final_kernel finds the exact k-th largest key among the candidates: an LDS
+// histogram over 1024 equal key ranges between the smallest and the largest candidate names the
+// range of the k-th key, and the few candidates of that range are ranked against each other
+// (equal keys by lower index, the reference's tie rule); it then compacts the winners and returns
+// the losers' weights to their lists.  Both kernels keep a bit-by-bit search on the 32-bit key
+// (one barrier per bit) for inputs the histogram does not resolve: a crowded range, or a wanted
+// rank outside the sampled window.  A row whose estimate kept fewer than k candidates is
+// re-scanned in full by its select workgroup, so the result is always the exact top-k.
 #include <cstdlib>
 
 #include "common.h"
@@ -606,7 +608,7 @@ struct __align__(16) SelScratch {
     uint32_t sel_key, sel_idx;  // the k-th key and, among equal keys, the largest index still selected
 };
 
-// The same search over keys in memory (any count).
+// The bit-by-bit search over keys in memory (any count).
 template <typename KeyAt>
 __device__ inline uint32_t bisect_mem(KeyAt key_at, uint32_t cnt, uint32_t want, uint32_t (*red)[kSelWaves],
                                       int &step, bool &exact) {
