@@ -618,7 +618,6 @@ __device__ inline uint32_t bisect_mem(KeyAt key_at, uint32_t cnt, uint32_t want,
     for (int bit = 31; bit >= 0; --bit) {
         const uint32_t trial = t | (1u << bit);
         uint32_t c = 0;
-#pragma unroll 8
         for (uint32_t r = 0; r < rounds; ++r) {
             const uint32_t p = r * kSelThreads + threadIdx.x;
             c += wave_count_if(p < cnt && key_at(p) >= trial);
@@ -1031,7 +1030,6 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
     uint32_t idx_thr = 0xffffffffu;
     if (k > 0 && !exact) {
         uint32_t c_gt = 0, c_eq = 0;
-#pragma unroll 4
         for (uint32_t r = 0; r < rounds; ++r) {
             const uint32_t p = r * kSelThreads + tid;
             const uint32_t kk = p < cnt ? key_at(p) : 0u;
@@ -1069,10 +1067,8 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
     out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
     *ref1_out = out.ref1;
     uint32_t mine = 0;
-#pragma unroll 4
     for (uint32_t p = tid; p < cnt; p += kSelThreads) mine += selected(pairs[p]) ? 1u : 0u;
     uint32_t at = block_exclusive_u32(mine, wsum);
-#pragma unroll 4
     for (uint32_t p = tid; p < cnt; p += kSelThreads) {
         const uint2 pr = pairs[p];
         if (selected(pr)) out.winner(at++, pr.x, pr.y);
