@@ -35,6 +35,7 @@ struct AttendArgs {
     const int32_t *topk_idx;  // [BH*G, k_cap]
     const int32_t *topk_cnt;  // [BH*G]
     int64_t k_cap;
+    int full_guess;           // sink + local rows the host expects per query row (for speculative index loads)
     float scale;
     int splits;
     float *partials;          // [BH*G, splits, kPartWidth]
@@ -110,6 +111,21 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int split = blockIdx.x, g = blockIdx.y, bh = blockIdx.z;
     const int b = bh / a.H, h = bh % a.H;
     const size_t orow = (size_t)bh * a.G + g;
+    // The selected indices of this chunk are requested before the row's counts are known, from
+    // where the chunk lies when the row is as long as the host sized the step for (the usual
+    // case); the counts then confirm the guess or the indices are read again.
+    constexpr int kSpec = 2;  // index loads per thread ahead of the counts: chunks of up to 512 rows
+    const int F_g = a.full_guess, total_g = F_g + (int)a.k_cap;
+    const int chunk_g = (total_g + a.splits - 1) / a.splits;
+    const int start_g = min(split * chunk_g, total_g);
+    const int32_t *tk = a.topk_idx + orow * a.k_cap;
+    int32_t spec[kSpec];
+#pragma unroll
+    for (int u = 0; u < kSpec; ++u) {
+        const int i = tid + u * kAttThreads;
+        const int r = start_g + i;
+        spec[u] = (i < chunk_g && r >= F_g && r < total_g) ? tk[r - F_g] : 0;
+    }
     const int len = a.seq_lens[b];
     const int n = a.n_idx[b];
     const int sink_end = min(a.sink, len);
@@ -157,15 +173,19 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     // ---- row addresses of this chunk (block-table lookups happen here, once) ---------------
     int64_t *off_s = reinterpret_cast<int64_t *>(smem);  // [chunk] element offsets of the rows
     {
-        const int32_t *tk = a.topk_idx + orow * a.k_cap;
-        for (int i = tid; i < cnt; i += kAttThreads) {
+        const bool guessed = F == F_g && total == total_g;  // then the chunk is where the guess put it
+        auto resolve = [&](int i, int32_t ahead, bool have) {
             const int r = start + i;
             int64_t pos;
             if (r < sink_end) pos = r;
             else if (r < F) pos = local_start + (r - sink_end);
-            else pos = sink_end + tk[r - F];
+            else pos = sink_end + (have ? ahead : tk[r - F]);
             off_s[i] = row_offset(a.kv, b, h, pos);
-        }
+        };
+#pragma unroll
+        for (int u = 0; u < kSpec; ++u)
+            if (tid + u * kAttThreads < cnt) resolve(tid + u * kAttThreads, spec[u], guessed);
+        for (int i = tid + kSpec * kAttThreads; i < cnt; i += kAttThreads) resolve(i, 0, false);
     }
     __syncthreads();
 
@@ -427,6 +447,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     PQHSA_REQUIRE(a.G >= 1 && a.G <= 16, "attend: G=%d outside [1, 16]", a.G);
     PQHSA_REQUIRE(a.L <= 4096, "attend: num_lists=%d too large", a.L);
     a.splits = pick_splits(BH * a.G, rows_max);
+    a.full_guess = rows_max > (int)a.k_cap ? rows_max - (int)a.k_cap : 0;
     const int chunk = (rows_max + a.splits - 1) / a.splits;
     PQHSA_REQUIRE(chunk <= 4 * kMaxChunk, "attend: %d rows per query exceed what %d splits can take", rows_max,
                   kMaxSplits);
