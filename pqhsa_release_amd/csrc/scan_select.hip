@@ -195,9 +195,10 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             const uint32_t c[4] = {cw.x, cw.y, cw.z, cw.w};
             const float kn[4] = {nw.x, nw.y, nw.z, nw.w};
             lid[0] = lw.x & 0xffffu; lid[1] = lw.x >> 16; lid[2] = lw.y & 0xffffu; lid[3] = lw.y >> 16;
+            // a stored list id is always below L; the clamp only keeps LDS accesses in range should
+            // the arrays hold anything else (keys past the tile score -inf further down, whatever their id)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (i0 + j >= tile_end || lid[j] >= (uint32_t)L) lid[j] = 0u;
+            for (int j = 0; j < 4; ++j) lid[j] = min(lid[j], (uint32_t)L - 1u);
             // keys are scored in sub-batches so that wide GQA groups stay within the register file
             constexpr int KB = GP <= 2 ? 4 : (GP == 4 ? 2 : 1);
 #pragma unroll
