@@ -188,14 +188,40 @@ class PQHSAEngine:
             self._alloc_index(n_need, self.index.num_lists)
             self.index.set_counts(counts)
 
-    def advance(self, count: int = 1) -> None:
-        """Bookkeeping after ``count`` tokens were appended to every sequence
-        (SparseKVCache.append, pq_hsa/attention/kv_cache.py:195-226)."""
+    @classmethod
+    def regroup(cls, sources) -> "PQHSAEngine":
+        """A new engine whose sequence b is sequence ``seq`` of ``engine`` for ``(engine, seq) =
+        sources[b]``: index rows and bookkeeping are copied, nothing is rebuilt.  For serving
+        batches whose membership changes (a request leaves, another joins); the caller binds the
+        K/V storage of the new batch afterwards."""
+        first = sources[0][0]
+        for eng, _ in sources:
+            eng._settle()
+            if eng.index is None:
+                raise RuntimeError("regroup: every source engine must have a built index")
+        new = cls(first.index_config, first.attention_config, batch=len(sources), kv_heads=first.H,
+                  device=first.device, growth_margin=first.growth_margin)
+        need = max(eng.index.n_host[seq] for eng, seq in sources)
+        new.index = ops.DeviceIndex.regroup([(eng.index, seq) for eng, seq in sources], need + new.growth_margin)
+        new.lens = [eng.lens[seq] for eng, seq in sources]
+        new.indexed_len = [eng.indexed_len[seq] for eng, seq in sources]
+        new.pending = [eng.pending[seq] for eng, seq in sources]
+        new.deferred_pending = any(eng.deferred_pending and eng.pending[seq] > 0 for eng, seq in sources)
+        new.seq_lens.copy_(torch.tensor(new.lens, dtype=torch.int32))
+        return new
+
+    def advance(self, count: int = 1, which=None) -> None:
+        """Bookkeeping after ``count`` tokens were appended to every sequence, or to the sequences
+        listed in ``which`` (SparseKVCache.append, pq_hsa/attention/kv_cache.py:195-226)."""
         ac = self.attention_config
-        for b in range(self.B):
+        some = range(self.B) if which is None else [int(b) for b in which]
+        for b in some:
             self.lens[b] += count
             self.pending[b] += count
-        self.seq_lens += count
+        if which is None:
+            self.seq_lens += count
+        else:
+            self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
         if self._fused_append:
             # a second append before the step that would have carried the first: settle the first now
             self._fused_append = False

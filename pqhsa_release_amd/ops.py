@@ -161,6 +161,32 @@ class DeviceIndex:
         self._struct = None
 
     @classmethod
+    def regroup(cls, sources, n_cap: int) -> "DeviceIndex":
+        """A new index whose sequence b is sequence ``seq`` of ``index`` for ``(index, seq) =
+        sources[b]``: the rows are copied on the device, nothing is re-encoded.  All sources share
+        KV heads, list count and device; ``n_cap`` is raised to the longest sequence if smaller."""
+        first = sources[0][0]
+        h, lists = first.kv_heads, first.num_lists
+        if any(ix.kv_heads != h or ix.num_lists != lists or ix.device != first.device for ix, _ in sources):
+            raise ValueError("regroup: the source indexes differ in KV heads, list count or device")
+        n_cap = max(int(n_cap), max(ix.n_host[seq] for ix, seq in sources))
+        new = cls(len(sources), h, lists, n_cap, first.device)
+        for b, (ix, seq) in enumerate(sources):
+            src, dst = slice(seq * h, (seq + 1) * h), slice(b * h, (b + 1) * h)
+            n = ix.n_host[seq]
+            for name in ("codes", "list_ids", "norms", "pos"):
+                getattr(new, name)[dst, :n].copy_(getattr(ix, name)[src, :n])
+            skeep = min(ix.s_cap, new.s_cap)
+            for name in ("s_codes", "s_list_ids", "s_norms"):
+                getattr(new, name)[dst, :skeep].copy_(getattr(ix, name)[src, :skeep])
+            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+                getattr(new, name)[dst].copy_(getattr(ix, name)[src])
+            new.s_n[b : b + 1].copy_(ix.s_n[seq : seq + 1])
+            new.n_sorted_host[b] = ix.n_sorted_host[seq]
+        new.set_counts([ix.n_host[seq] for ix, seq in sources])
+        return new
+
+    @classmethod
     def sample_size(cls, n: int) -> int:
         # a whole number of 1024-key slots (the threshold kernel holds the sample in registers, one
         # slot per thread), as close to n / SAMPLE_RATE as that allows

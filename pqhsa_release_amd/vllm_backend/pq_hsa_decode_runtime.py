@@ -54,6 +54,7 @@ STATS: dict[str, Any] = {
     "pq_batch_reqs_total": 0,
     "pq_batch_fused_steps": 0,
     "pq_batch_group_builds": 0,
+    "pq_batch_regroups": 0,
     "batch_mode": False,
 }
 
@@ -180,6 +181,21 @@ def host_seq_lens(attn_metadata) -> list[int]:
     except Exception:
         pass
     return lens
+
+
+def host_first_blocks(attn_metadata) -> list[int]:
+    """First physical block of every request of the batch, as host integers: what tells one
+    request from another while it lives (vLLM moves requests between batch rows when one
+    finishes).  Read once per step and kept on the metadata object, like the lengths."""
+    cached = getattr(attn_metadata, "_pq_host_first_blocks", None)
+    if cached is not None:
+        return cached
+    first = [int(x) for x in attn_metadata.block_table[:, 0].tolist()]
+    try:
+        attn_metadata._pq_host_first_blocks = first
+    except Exception:
+        pass
+    return first
 
 
 def should_pq_decode(attn_metadata) -> bool:
@@ -364,40 +380,64 @@ def _int32_table(attn_metadata, num_reqs: int) -> torch.Tensor:
 
 def run_pq_decode_group(impl, layer, query, key, value, kv_cache, attn_metadata, output) -> torch.Tensor:
     """All requests of the decode batch through one engine: the step's appends ride on the decode
-    launches and every sequence, KV head and query row is served by the same six kernels.  The
-    group is rebuilt whenever the batch is not the previous one advanced by one token each."""
+    launches and every sequence, KV head and query row is served by the same six kernels.
+    Requests are told apart by their first physical block.  When the batch is the previous one
+    advanced by one token each, the step is one call; when requests left, joined or changed rows,
+    the index rows of those that continue are copied into a new group (nothing is re-encoded)
+    and only the newcomers are built."""
     from ..attention.engine import PQHSAEngine
 
     st = state_for(impl, layer)
     num_reqs = int(attn_metadata.seq_lens.shape[0])
-    lens = list(host_seq_lens(attn_metadata))
+    lens = list(host_seq_lens(attn_metadata))[:num_reqs]
+    ids = list(host_first_blocks(attn_metadata))[:num_reqs]
     grp = st.get("group")
-    sequential = (grp is not None and len(grp["lens"]) == num_reqs
-                  and all(now == before + 1 for now, before in zip(lens, grp["lens"])))
     table = _int32_table(attn_metadata, num_reqs)
-    if not sequential:
-        t0 = time.perf_counter()
-        eng = PQHSAEngine(paper_index_config(), paper_attention_config(impl.scale), batch=num_reqs,
-                          kv_heads=impl.num_kv_heads, device=kv_cache.device)
-        eng.bind_paged(kv_cache, table)
-        eng.build(lens)
-        grp = st["group"] = {"engine": eng, "lens": lens, "appends": 0}
-        STATS["pq_build_s_total"] += time.perf_counter() - t0
-        STATS["pq_batch_group_builds"] += 1
-        STATS["sidecar"] = "PQHSAEngine"
-    else:
+    steady = (grp is not None and grp["ids"] == ids
+              and all(now == before + 1 for now, before in zip(lens, grp["lens"])))
+    if steady:
         eng = grp["engine"]
         eng.bind_paged(kv_cache, table)      # the block table may have grown
         eng.advance(1)
         grp["lens"], grp["appends"] = lens, grp["appends"] + 1
         STATS["pq_append_calls"] += 1
+    else:
+        t0 = time.perf_counter()
+        where = {rid: j for j, rid in enumerate(grp["ids"])} if grp is not None else {}
+        going_on = [where.get(ids[r]) if where.get(ids[r]) is not None and lens[r] == grp["lens"][where[ids[r]]] + 1
+                    else None for r in range(num_reqs)]
+        fresh = [r for r in range(num_reqs) if going_on[r] is None]
+        newcomers = None
+        if fresh:
+            newcomers = PQHSAEngine(paper_index_config(), paper_attention_config(impl.scale), batch=len(fresh),
+                                    kv_heads=impl.num_kv_heads, device=kv_cache.device)
+            newcomers.bind_paged(kv_cache, table[fresh].contiguous())
+            newcomers.build([lens[r] for r in fresh])
+            STATS["pq_build_calls"] += 1
+        if len(fresh) == num_reqs:
+            eng = newcomers
+            STATS["pq_batch_group_builds"] += 1
+        else:
+            sources = [(newcomers, fresh.index(r)) if going_on[r] is None else (grp["engine"], going_on[r])
+                       for r in range(num_reqs)]
+            eng = PQHSAEngine.regroup(sources)
+            STATS["pq_batch_regroups"] += 1
+        eng.bind_paged(kv_cache, table)
+        staying = [r for r in range(num_reqs) if going_on[r] is not None]
+        if staying:
+            eng.advance(1, which=staying)     # their new token is indexed by the step below
+            STATS["pq_append_calls"] += 1
+        grp = st["group"] = {"engine": eng, "lens": lens, "ids": ids,
+                             "appends": (grp["appends"] + 1) if (grp is not None and staying) else 0}
+        STATS["pq_build_s_total"] += time.perf_counter() - t0
+        STATS["sidecar"] = "PQHSAEngine"
     q, dst = query[:num_reqs], output[:num_reqs]
     groups = impl.num_heads // impl.num_kv_heads
     if dst.shape == q.shape and dst.dtype == q.dtype == kv_cache.dtype and dst.is_contiguous():
         eng.forward(q, groups, out=dst)                      # straight into vLLM's output buffer
     else:
         copy_ctx(output, eng.forward(q, groups), num_reqs)
-    if sequential and flush_interval() > 0 and grp["appends"] % flush_interval() == 0:
+    if grp["appends"] > 0 and flush_interval() > 0 and grp["appends"] % flush_interval() == 0:
         t1 = time.perf_counter()
         eng.apply_pending_index_update()
         STATS["pq_flush_s_total"] += time.perf_counter() - t1

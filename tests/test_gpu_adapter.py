@@ -397,15 +397,38 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
 
     everyone = lambda s: [0, 1, 2]
     one_leaves = lambda s: [0, 1, 2] if s < 4 else [0, 2]
-    for reqs_at, builds in ((everyone, 1), (one_leaves, 2)):
-        fused, st_f = run("1", reqs_at)
-        single, st_s = run("0", reqs_at)
-        assert st_f["pq_batch_fused_steps"] == steps + 1 and st_f["pq_batch_group_builds"] == builds
-        assert st_s["pq_batch_fused_steps"] == 0 and st_s["pq_build_calls"] >= 3
-        for s, (a, b) in enumerate(zip(fused, single)):
-            if len(reqs_at(s)) < B:
-                # the group was rebuilt for everyone, the per-request form rebuilt only the request
-                # that moved up a row: only that row still runs on an index trained on the same keys
-                a, b = a[1:], b[1:]
-            # the same kernels on the same trained indexes: only bf16 rounding of the output differs
-            assert np.abs(a - b).max() <= 2e-3 + 2.0 ** -7 * np.abs(b).max(), (s, np.abs(a - b).max())
+    one_joins = lambda s: [0, 1] if s < 3 else [0, 1, 2]
+    rows_swap = lambda s: [0, 1, 2] if s < 3 else [2, 0, 1]
+
+    def close(a, b, what):
+        # the same kernels on the same trained indexes: only bf16 rounding of the output differs
+        assert np.abs(a - b).max() <= 2e-3 + 2.0 ** -7 * np.abs(b).max(), (what, np.abs(a - b).max())
+
+    fused, st_f = run("1", everyone)
+    single, st_s = run("0", everyone)
+    assert st_f["pq_batch_fused_steps"] == steps + 1 and st_f["pq_batch_group_builds"] == 1
+    assert st_f["pq_batch_regroups"] == 0 and st_s["pq_batch_fused_steps"] == 0 and st_s["pq_build_calls"] == 3
+    for s_, (a, b) in enumerate(zip(fused, single)):
+        close(a, b, ("everyone", s_))
+
+    # a request leaves: the group keeps the index rows of the two that stay (no rebuild); the
+    # per-request form goes by batch row, so it rebuilds the request that moved up a row
+    left, st_l = run("1", one_leaves)
+    assert st_l["pq_batch_group_builds"] == 1 and st_l["pq_batch_regroups"] == 1 and st_l["pq_build_calls"] == 1
+    for s_, a in enumerate(left):
+        want = fused[s_] if s_ < 4 else fused[s_][[0, 2]]     # what the full batch gave for the same requests
+        close(a, want, ("one leaves", s_))
+
+    # a request joins: only the newcomer is built, at the step it appears, as its own sidecar would be
+    joined, st_j = run("1", one_joins)
+    single_j, _ = run("0", one_joins)
+    assert st_j["pq_batch_group_builds"] == 1 and st_j["pq_batch_regroups"] == 1 and st_j["pq_build_calls"] == 2
+    for s_, (a, b) in enumerate(zip(joined, single_j)):
+        close(a, b, ("one joins", s_))
+
+    # requests change rows: told apart by their first block, their indexes move with them
+    swapped, st_w = run("1", rows_swap)
+    assert st_w["pq_batch_group_builds"] == 1 and st_w["pq_batch_regroups"] == 1 and st_w["pq_build_calls"] == 1
+    for s_, a in enumerate(swapped):
+        want = fused[s_] if s_ < 3 else fused[s_][[2, 0, 1]]
+        close(a, want, ("rows swap", s_))
