@@ -336,3 +336,37 @@ def test_batch_mode_per_request_sidecars(fake_stack, monkeypatch):
     assert sorted(rt.state_for(impl, layer)["batch"]) == [0, 1]
     assert rt.STATS["pq_batch_steps"] == 3 and rt.STATS["pq_batch_reqs_total"] == 8
     assert rt.STATS["pq_batch_fused_steps"] == 0
+
+
+def test_device_index_regroup_copies_rows_and_counts():
+    """Regrouping picks sequences out of existing indexes: rows, per-list tables, sampled subsets
+    and counts follow the sequence; capacity grows to what the caller asks for."""
+    from pqhsa_release_amd import ops
+
+    gen = torch.Generator().manual_seed(3)
+    def filled(batch, n_cap, counts):
+        ix = ops.DeviceIndex(batch, 2, 8, n_cap, "cpu")
+        for name in ("codes", "list_ids", "norms", "pos", "coarse", "codebooks", "vbar", "vsum", "vcount",
+                     "s_codes", "s_list_ids", "s_norms"):
+            t = getattr(ix, name)
+            t.copy_((torch.rand(t.shape, generator=gen) * 100).to(t.dtype))
+        ix.s_n.copy_(torch.tensor([c // 2 for c in counts], dtype=torch.int32))
+        ix.n_sorted_host = [c // 3 for c in counts]
+        ix.set_counts(counts)
+        return ix
+
+    a, b = filled(3, 64, [40, 10, 64]), filled(1, 200, [150])
+    new = ops.DeviceIndex.regroup([(a, 2), (b, 0), (a, 0)], n_cap=100)
+    assert new.batch == 3 and new.n_cap >= 150 and new.n_host == [64, 150, 40]
+    assert new.n_sorted_host == [21, 50, 13] and new.s_n.tolist() == [32, 75, 20]
+    assert new.n_idx.tolist() == [64, 150, 40]
+    for dst, (src, seq, n) in enumerate([(a, 2, 64), (b, 0, 150), (a, 0, 40)]):
+        rows_new, rows_old = slice(2 * dst, 2 * dst + 2), slice(2 * seq, 2 * seq + 2)
+        for name in ("codes", "list_ids", "norms", "pos"):
+            assert torch.equal(getattr(new, name)[rows_new, :n], getattr(src, name)[rows_old, :n]), name
+        for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
+            assert torch.equal(getattr(new, name)[rows_new], getattr(src, name)[rows_old]), name
+        keep = min(src.s_cap, new.s_cap)
+        assert torch.equal(new.s_codes[rows_new, :keep], src.s_codes[rows_old, :keep])
+    with pytest.raises(ValueError):
+        ops.DeviceIndex.regroup([(a, 0), (ops.DeviceIndex(1, 4, 8, 16, "cpu"), 0)], n_cap=16)
