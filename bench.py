@@ -198,6 +198,64 @@ def copy_bandwidth(device, mib=1024, reps=10):
     return 2.0 * src.numel() * 4 * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
+def standalone_kernels(layer, reps=20):
+    """The stand-alone entry points on the same layer, buffers allocated once: the LUT scan that
+    writes every logit (pqhsa_lut_scan) and the exact top-k of that logit matrix
+    (pqhsa_topk_radix, two passes over the logits).  Times by torch events on the current stream."""
+    from pqhsa_release_amd import _lib, ops
+
+    lib, idx, G = _lib.load(), layer.index, layer.G
+    bh, rows = idx.batch * idx.kv_heads, idx.batch * idx.kv_heads * layer.G
+    qnorm, lut, ls = ops.lut_build(layer.q, idx, G)
+    logits = torch.zeros(bh, G, idx.n_cap, dtype=torch.float32, device=idx.device)
+    n = [layer.n[r // (idx.kv_heads * G)] for r in range(rows)]
+    k = [math.ceil(x * FRACTION) for x in n]
+    n_t = torch.tensor(n, dtype=torch.int32, device=idx.device)
+    k_t = torch.tensor(k, dtype=torch.int32, device=idx.device)
+    n_max, k_cap = max(n), max(max(k), 1)
+    ws_bytes = lib.pqhsa_topk_workspace_bytes(rows, n_max)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=idx.device)
+    tidx = torch.empty(rows, k_cap, dtype=torch.int32, device=idx.device)
+    tval = torch.empty(rows, k_cap, dtype=torch.float32, device=idx.device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    # the layer's index is sorted by list, so logits are scattered to their retrieval-local columns;
+    # with an identity position map the same kernel writes them in stored order, as for an index
+    # that was never regrouped (same bytes, coalesced)
+    arrival = type(idx.struct()).from_buffer_copy(idx.struct())
+    ident = torch.arange(idx.n_cap, dtype=torch.int32, device=idx.device).repeat(bh, 1)
+    arrival.pos = ident.data_ptr()
+    which = {"ref": idx.ref()}
+
+    def scan():
+        _lib.check(lib.pqhsa_lut_scan(which["ref"], G, int(idx.n_max), qnorm.data_ptr(), lut.data_ptr(), ls.data_ptr(),
+                                      1.0 / math.sqrt(128), logits.data_ptr(), idx.n_cap, stream), "pqhsa_lut_scan")
+
+    def topk():
+        _lib.check(lib.pqhsa_topk_radix(logits.data_ptr(), idx.n_cap, rows, n_t.data_ptr(), k_t.data_ptr(), n_max,
+                                        tidx.data_ptr(), tval.data_ptr(), k_cap, ws.data_ptr(), ws_bytes, stream),
+                   "pqhsa_topk_radix")
+
+    out = {}
+    keys = sum(layer.n) * idx.kv_heads
+    for name, fn, nbytes in (("lut_scan_sorted_index", scan, keys * 14 + keys * G * 4),
+                             ("lut_scan_arrival_order", scan, keys * 14 + keys * G * 4),
+                             ("topk_radix", topk, 2 * keys * G * 4)):
+        which["ref"] = ctypes.byref(arrival) if name == "lut_scan_arrival_order" else idx.ref()
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1000.0 / reps
+        out[name] = {"us": round(us, 2), "MB": round(nbytes / 1e6, 2), "GBps": round(nbytes / 1e3 / us, 1),
+                     "frac_of_peak": round(nbytes / 1e3 / us / HBM_PEAK_GBPS, 4)}
+    return out
+
+
 def cpu_baseline(layer, seconds=12.0):
     """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
     the same inputs and trained index, and scale to the whole layer."""
@@ -264,6 +322,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--append", action="store_true",
                     help="every step appends one key per sequence before it attends (always on for config 4)")
+    ap.add_argument("--standalone", action="store_true",
+                    help="also time the stand-alone entry points (pqhsa_lut_scan writing all logits, "
+                         "pqhsa_topk_radix on that matrix) and report their HBM rates")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one device copy of this many MiB after the warm-up (a kernel of known HBM "
                          "traffic, the yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
@@ -407,6 +468,8 @@ def main():
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},
     }
+    if args.standalone:
+        result["standalone"] = standalone_kernels(layer)
     copy_gbps = copy_bandwidth(device)
     result["hbm_copy_GBps"] = round(copy_gbps, 1)
     result["roofline"]["frac_of_copy"] = round(result["roofline"]["achieved"] / copy_gbps, 4)

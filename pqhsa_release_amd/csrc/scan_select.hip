@@ -226,24 +226,40 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         } else {
             const float *row = a.logits_in + (size_t)bh * a.logits_in_stride;
+            // one 16-byte load where the row's start and stride keep fours aligned
+            if (i0 + 4 <= tile_end && ((reinterpret_cast<uintptr_t>(row) & 15) == 0)) {
+                const float4 v = *reinterpret_cast<const float4 *>(row + i0);
+                s[0][0] = v.x; s[1][0] = v.y; s[2][0] = v.z; s[3][0] = v.w;
+            } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                s[j][0] = (i0 + j < tile_end) ? row[i0 + j] : 0.0f;
-                lid[j] = 0u;
+                for (int j = 0; j < 4; ++j) s[j][0] = (i0 + j < tile_end) ? row[i0 + j] : 0.0f;
             }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) lid[j] = 0u;
         }
 
         if constexpr (MODE == kWrite) {
-            int32_t col[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) col[j] = (a.pos && i0 + j < tile_end) ? a.pos[base + i0 + j] : i0 + j;
+            int32_t col[4] = {i0, i0 + 1, i0 + 2, i0 + 3};
+            if (a.pos && in_range) {  // stored positions come in fours, the row's capacity is a multiple of 4
+                const int4 pw = *reinterpret_cast<const int4 *>(a.pos + base + i0);
+                col[0] = pw.x; col[1] = pw.y; col[2] = pw.z; col[3] = pw.w;
+            }
+            // four keys that land side by side (an index still in arrival order) go out as one
+            // 16-byte store when the destination row allows it
+            const bool quad = i0 + 4 <= tile_end && (col[0] & 3) == 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 &&
+                              col[3] == col[0] + 3 && (a.logits_out_stride & 3) == 0 &&
+                              (reinterpret_cast<uintptr_t>(a.logits_out) & 15) == 0;
 #pragma unroll
             for (int g = 0; g < GP; ++g) {
                 if (g >= a.G) continue;
                 float *dst = a.logits_out + ((size_t)bh * a.G + g) * a.logits_out_stride;
+                if (quad) {
+                    *reinterpret_cast<float4 *>(dst + col[0]) = make_float4(s[0][g], s[1][g], s[2][g], s[3][g]);
+                } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (i0 + j < tile_end) dst[col[j]] = s[j][g];
+                    for (int j = 0; j < 4; ++j)
+                        if (i0 + j < tile_end) dst[col[j]] = s[j][g];
+                }
             }
         } else if constexpr (MODE == kHist) {
 #pragma unroll

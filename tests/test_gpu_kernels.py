@@ -99,10 +99,41 @@ def test_lut_build_and_scan_match_oracle_bitwise(groups, dtype):
         assert np.array_equal(got, want), (b, h, np.abs(got - want).max())
 
 
-def test_topk_radix_on_logit_matrix_with_ties():
+@pytest.mark.parametrize("stride_pad,offset", [(0, 0), (3, 0), (0, 1), (5, 3)])
+def test_lut_scan_row_stride_and_alignment(stride_pad, offset):
+    # The scan writes four neighbouring logits as one 16-byte store when the destination allows it;
+    # an odd row stride or an unaligned base takes the element-wise path.  Both must give the
+    # oracle's bits, and neither may touch a column at or past n.
+    from pqhsa_release_amd import _lib
+
+    dev = _cuda()
+    groups = 4
+    p = Problem(lens=[1501, 1110], heads=2, groups=groups, lists=40, dtype=torch.bfloat16, seed=17)
+    idx = p.device_index(dev)
+    qnorm, lut, ls = ops.lut_build(p.q_tensor(), idx, groups)
+    bh, stride = idx.batch * idx.kv_heads, idx.n_cap + stride_pad
+    buf = torch.full((bh * groups * stride + 8,), -7.0, dtype=torch.float32, device=dev)
+    out = buf[offset : offset + bh * groups * stride]
+    lib = _lib.load()
+    _lib.check(lib.pqhsa_lut_scan(idx.ref(), groups, int(idx.n_max), qnorm.data_ptr(), lut.data_ptr(), ls.data_ptr(),
+                                  float(SCALE), out.data_ptr(), stride, torch.cuda.current_stream().cuda_stream),
+               "pqhsa_lut_scan")
+    torch.cuda.synchronize()
+    got_all = out.view(bh, groups, stride).cpu().numpy()
+    for (b, h), ix in p.index.items():
+        r, n = b * p.H + h, p.n(b)
+        oq, olut, ols = fixed.lut_build(p.queries[b, h].numpy(), ix["coarse"], ix["codebooks"])
+        want = fixed.scan(ix["codes"], ix["list_ids"], ix["norms"], olut, ols, oq, SCALE)
+        assert np.array_equal(got_all[r, :, :n], want)
+        assert (got_all[r, :, n:] == -7.0).all()
+    assert (buf[:offset] == -7.0).all() and (buf[offset + bh * groups * stride :] == -7.0).all()
+
+
+@pytest.mark.parametrize("stride", [5000, 5001, 5003])  # rows 16-byte aligned, and not
+def test_topk_radix_on_logit_matrix_with_ties(stride):
     dev = _cuda()
     rng = np.random.default_rng(11)
-    rows, stride = 9, 5000
+    rows = 9
     logits = rng.standard_normal((rows, stride)).astype(np.float32)
     logits[1, :] = 0.5                                    # all equal: pure lowest-index rule
     logits[2, 100:400] = logits[2].max() + 1              # wide tie at the top
