@@ -241,6 +241,25 @@ class PQHSAEngine:
             else:
                 self._refresh_index_now()
 
+    def extend(self, new_lens) -> int:
+        """The K/V store now holds ``new_lens[b]`` tokens of sequence b (at least as many as before;
+        only rows outside the indexed region may have changed).  The added rows are taken into the
+        index the way a run of appended tokens is at an index update, whatever the update interval
+        (extend_prefix, benchmarks/e2e_pq_param_sweep.py:3600-3733, steps 3 and 4).  Returns the
+        number of sequences whose index grew."""
+        self._settle()
+        new_lens = [int(x) for x in new_lens]
+        if len(new_lens) != self.B or any(n1 < n0 for n0, n1 in zip(self.lens, new_lens)):
+            raise ValueError("extend: one length per sequence, none shorter than before")
+        before = [self.n(b) for b in range(self.B)]
+        for b in range(self.B):
+            self.pending[b] += new_lens[b] - self.lens[b]
+        self.lens = new_lens
+        self.seq_lens.copy_(torch.tensor(self.lens, dtype=torch.int32))
+        self._refresh_index_now()
+        self.deferred_pending = False
+        return sum(1 for b in range(self.B) if self.n(b) > before[b])
+
     def _settle(self) -> None:
         """Bring the index up to date if an append is still waiting for the next forward()."""
         if self._fused_append:

@@ -3,13 +3,15 @@
 Same surface as the reference's ``GQASidecar`` / ``GQASidecarFast``
 (benchmarks/vllm_backend/gqa_sidecar.py:11-76, gqa_sidecar_fast.py:48-187): ``build_cache``,
 ``append``, ``lean_append``, ``append_many``, ``forward``, ``set_paged_kv_context``,
-``checkpoint_prefix`` / ``restore_prefix`` / ``prefix_checkpoint_length`` and the
+``checkpoint_prefix`` / ``restore_prefix`` / ``extend_prefix`` / ``prefix_checkpoint_length`` and the
 ``batched_heads_active`` / ``cuda_graph_active`` flags.  One batched engine serves all KV
 heads; once a paged context is set the exact rows are read from vLLM's pages in place and the
 sidecar drops its own K/V copy.
 """
 
 from __future__ import annotations
+
+import time
 
 import torch
 
@@ -115,6 +117,50 @@ class GQASidecar:
         if kv_cache is not None and attn_metadata is not None:
             self.set_paged_kv_context(kv_cache, attn_metadata, seq_idx)
         return True
+
+    def extend_prefix(self, keys: torch.Tensor | None = None, values: torch.Tensor | None = None, *, kv_cache,
+                      attn_metadata, seq_idx: int = 0, new_length: int) -> dict | None:
+        """Restore the checkpointed prefix and grow it in place to ``new_length`` tokens: the next
+        request's prompt is the checkpointed prompt followed by more tokens, which vLLM's prefill
+        has already written to the paged cache (GQAIVFPQDecodeAttentionAdapter.extend_prefix,
+        benchmarks/e2e_pq_param_sweep.py:3600-3733).  The added rows are encoded with the
+        checkpointed tables after the configured update step (one EMA move under the deferred
+        strategy), not by retraining.  The checkpoint's last row, the old request's first decode
+        token, is overwritten by the new prompt; it must still lie in the exact window.  Returns
+        counters and timings, or ``None`` when the caller has to rebuild."""
+        if self._checkpoint is None:
+            return None
+        base, new_length = int(self._checkpoint["length"]), int(new_length)
+        if new_length <= base or kv_cache is None or attn_metadata is None:
+            return None
+        info: dict = {"base_length": base, "new_length": new_length, "delta_tokens": new_length - base, "ring": False}
+        t0 = time.perf_counter()
+        if not self.restore_prefix(None, None):
+            return None
+        info["restore_s"] = time.perf_counter() - t0
+        eng = self.adapter.engine
+        delta_start = base - 1
+        if eng._retrieval_end(0) > delta_start:
+            return None                       # the row that changes is an indexed one
+        t1 = time.perf_counter()
+        if eng.keys_buf is not None:          # the sidecar keeps its own K/V copy: the new rows must land there
+            from .paged_kv_fa import gather_flashattn_kv_range
+
+            dk, dv = gather_flashattn_kv_range(kv_cache, attn_metadata, seq_idx, delta_start, new_length)
+            eng._grow_dense(new_length)
+            eng.keys_buf[0, :, delta_start:new_length].copy_(dk)
+            eng.values_buf[0, :, delta_start:new_length].copy_(dv)
+        else:
+            self.set_paged_kv_context(kv_cache, attn_metadata, seq_idx)
+        info["gather_s"] = time.perf_counter() - t1
+        t2 = time.perf_counter()
+        info["flush_applied_streams"] = eng.extend([new_length]) * self.num_kv_heads
+        info["flush_s"] = time.perf_counter() - t2
+        self.length = new_length
+        info["total_s"] = time.perf_counter() - t0
+        info["indexed_length"] = int(eng.indexed_len[0])
+        info["retrieval_len"] = int(eng.n(0))
+        return info
 
 
 # the runtime's PQ_HSA_SIDECAR switch selects between two classes in the reference; both names

@@ -5,7 +5,8 @@ same function names, environment switches, STATS keys and error conventions: ``p
 (:790-822) gates on ``pq_enabled`` / ``should_pq_decode`` (:302-341, 356-361), and
 ``run_pq_decode`` (:492-716) builds a sidecar from the paged cache on the first or a
 non-sequential step, appends + attends on sequential steps, restores a checkpointed prefix when
-the same prompt returns, and flushes the deferred index update every ``PQ_HSA_FLUSH_INTERVAL``
+the same prompt returns (or, with ``PQ_HSA_PREFIX_EXTEND=1``, extends it when the prompt continues
+it), and flushes the deferred index update every ``PQ_HSA_FLUSH_INTERVAL``
 appends.  The sidecar is the MI355X batched engine (``GQASidecar``).
 """
 
@@ -49,6 +50,11 @@ STATS: dict[str, Any] = {
     "prefix_persist_hits": 0,
     "prefix_persist_misses": 0,
     "prefix_miss_reasons": {},
+    "prefix_extend_hits": 0,
+    "prefix_extend_rejects": {},
+    "pq_extend_s_total": 0.0,
+    "pq_extend_delta_tokens_total": 0,
+    "pq_extend_last": None,
     "reject": {},
     "pq_batch_steps": 0,
     "pq_batch_reqs_total": 0,
@@ -278,6 +284,66 @@ def prefix_cache_key(attn_metadata, seq_len: int):
     return key
 
 
+def _prefix_extend_enabled() -> bool:
+    """``PQ_HSA_PREFIX_EXTEND=1``: when a request's prompt continues the checkpointed one, restore the
+    index and take in only the added tokens instead of rebuilding (runtime.py:425-428).  Off by default."""
+    return os.environ.get("PQ_HSA_PREFIX_EXTEND", "0") == "1"
+
+
+def _prefix_extend_max_frac() -> float:
+    try:
+        return float(os.environ.get("PQ_HSA_PREFIX_EXTEND_MAX_FRAC", "0.5"))
+    except ValueError:
+        return 0.5
+
+
+def prefix_extend_match(attn_metadata, old_key, checkpoint_len, seq_len: int):
+    """Does the current request's prompt strictly extend the checkpointed prompt?  ``old_key`` is the
+    ``(context_len, digest)`` stored with the checkpoint, ``checkpoint_len`` the sidecar's length at
+    that time (prompt + the first decode token).  Returns ``(ok, reason, new_key, delta_tokens)``
+    with the reference's reasons (runtime.py:438-488).  The digest of the new prompt's first
+    ``context_len`` ids is kept on the metadata object, so the layers of one step hash it once."""
+    if old_key is None or checkpoint_len is None:
+        return False, "no_checkpoint", None, 0
+    old_ctx, old_digest = int(old_key[0]), old_key[1]
+    checkpoint_len = int(checkpoint_len)
+    if checkpoint_len != old_ctx + 1:
+        return False, "checkpoint_inconsistent", None, 0
+    context_len = int(seq_len) - int(attn_metadata.max_query_len)
+    delta = int(seq_len) - checkpoint_len
+    if context_len <= old_ctx or delta <= 0:
+        return False, "not_longer", None, 0
+    if float(delta) / float(seq_len) > _prefix_extend_max_frac():
+        return False, "delta_too_large", None, delta
+    digests = getattr(attn_metadata, "_pq_prefix_ext_digests", None)
+    if digests is None:
+        digests = {}
+        try:
+            attn_metadata._pq_prefix_ext_digests = digests
+        except Exception:
+            pass
+    d = digests.get(old_ctx)
+    if d is None:
+        runner = getattr(attn_metadata, "_pq_runner", None)
+        if runner is None:
+            return False, "no_runner", None, delta
+        req_ids = runner.input_batch.req_ids
+        if not req_ids:
+            return False, "no_request", None, delta
+        request = runner.requests.get(req_ids[0])
+        prompt_ids = None if request is None else request.prompt_token_ids
+        if prompt_ids is None or len(prompt_ids) != context_len:
+            return False, "prompt_len_mismatch", None, delta
+        d = hashlib.blake2b(array("I", prompt_ids[:old_ctx]).tobytes(), digest_size=16).digest()
+        digests[old_ctx] = d
+    if d != old_digest:
+        return False, "prefix_digest_mismatch", None, delta
+    new_key = prefix_cache_key(attn_metadata, seq_len)
+    if new_key is None:
+        return False, "no_prefix_key", None, delta
+    return True, "ok", new_key, delta
+
+
 def _build_sidecar(impl, kv_cache, attn_metadata, seq_idx: int):
     t_g = time.perf_counter()
     keys, values, gathered = gather_flashattn_kv(kv_cache, attn_metadata, seq_idx)
@@ -320,6 +386,31 @@ def run_pq_decode(impl, layer, query, key, value, kv_cache, attn_metadata) -> to
             STATS["pq_forward_only_s_total"] += time.perf_counter() - t_forward
             STATS["pq_decode_calls"] += 1
             return ctx
+        if _prefix_extend_enabled() and adapter is not None and hasattr(adapter, "extend_prefix"):
+            ok, why, new_key, delta = prefix_extend_match(attn_metadata, st["prefix_key"], checkpoint_len, seq_len)
+            if ok:
+                t_ext = time.perf_counter()
+                info = adapter.extend_prefix(as_decode_qkv(key), as_decode_qkv(value), kv_cache=kv_cache,
+                                             attn_metadata=attn_metadata, seq_idx=0, new_length=seq_len)
+                ext_s = time.perf_counter() - t_ext
+                if info is None:
+                    why = "adapter_declined"
+                else:
+                    STATS["pq_extend_s_total"] += ext_s
+                    STATS["prefix_extend_hits"] += 1
+                    STATS["pq_extend_delta_tokens_total"] = int(STATS["pq_extend_delta_tokens_total"]) + int(delta)
+                    STATS["pq_extend_last"] = dict(info, wall_s=ext_s)
+                    st.update(prefix_key=new_key, seq_len=seq_len, appends=0)
+                    t_forward = time.perf_counter()
+                    ctx = adapter.forward(q)
+                    forward_s = time.perf_counter() - t_forward
+                    STATS["pq_forward_only_s_total"] += forward_s
+                    STATS["pq_forward_s_total"] += ext_s + forward_s
+                    adapter.checkpoint_prefix()          # the next turn may extend this one
+                    STATS["pq_decode_calls"] += 1
+                    return ctx
+            rej = STATS["prefix_extend_rejects"]
+            rej[why] = rej.get(why, 0) + 1
         STATS["prefix_persist_misses"] += 1
         if adapter is None:
             reason = "no_adapter"

@@ -237,6 +237,70 @@ def test_prefix_checkpoint_restore_on_same_prompt(fake_stack, monkeypatch):
     assert FakeSidecar.built == 1 and rt.STATS["prefix_persist_hits"] == 1
 
 
+def test_prefix_extend_when_the_prompt_continues_the_checkpointed_one(fake_stack, monkeypatch):
+    # reasons and counters as in the reference's runtime (pq_hsa_decode_runtime.py:431-488, 574-618)
+    impl, layer, kv_cache = fake_stack
+    monkeypatch.setenv("PQ_HSA_ENABLE", "1")
+    requests = {"r0": types.SimpleNamespace(prompt_token_ids=list(range(499)))}
+    runner = types.SimpleNamespace(input_batch=types.SimpleNamespace(req_ids=["r0"]), requests=requests)
+    calls = []
+
+    def extend_prefix(self, k, v, *, kv_cache, attn_metadata, seq_idx=0, new_length):
+        calls.append((self._ckpt, new_length))
+        if self.fail:
+            return None
+        self.length = new_length
+        return {"base_length": self._ckpt, "new_length": new_length}
+
+    monkeypatch.setattr(FakeSidecar, "extend_prefix", extend_prefix, raising=False)
+
+    def go(seq_len):
+        md = meta(seq_len)
+        md._pq_runner = runner
+        out = torch.zeros(1, 8, 128)
+        return rt.pq_or_dense_forward(impl, layer, torch.zeros(1, 8, 128), torch.zeros(1, 2, 128),
+                                      torch.zeros(1, 2, 128), kv_cache, md, out, lambda: out)
+
+    go(500)                                             # prompt of 499 tokens + the first decode token
+    go(501)
+    # next turn: the old prompt, what was generated, and 100 more tokens; switch still off -> rebuild
+    requests["r0"] = types.SimpleNamespace(prompt_token_ids=list(range(499)) + [7] * 101)
+    go(601)
+    assert FakeSidecar.built == 2 and calls == [] and rt.STATS["prefix_extend_hits"] == 0
+    monkeypatch.setenv("PQ_HSA_PREFIX_EXTEND", "1")
+    requests["r0"] = types.SimpleNamespace(prompt_token_ids=list(range(499)) + [7] * 101 + [9] * 50)
+    assert float(go(651)[0, 0, 0]) == 651.0
+    assert FakeSidecar.built == 2 and calls == [(601, 651)]
+    assert rt.STATS["prefix_extend_hits"] == 1 and rt.STATS["pq_extend_delta_tokens_total"] == 50
+    assert rt.STATS["pq_extend_last"]["new_length"] == 651
+    sc = rt.state_for(impl, layer)["sidecar"]
+    assert sc.prefix_checkpoint_length == 651           # re-armed for the turn after
+    go(652)
+    # a prompt that does not start with the checkpointed one
+    requests["r0"] = types.SimpleNamespace(prompt_token_ids=[1] * 700)
+    go(701)
+    assert FakeSidecar.built == 3 and rt.STATS["prefix_extend_rejects"] == {"prefix_digest_mismatch": 1}
+    # more than PQ_HSA_PREFIX_EXTEND_MAX_FRAC of the new length would be new
+    requests["r0"] = types.SimpleNamespace(prompt_token_ids=[1] * 700 + [2] * 900)
+    go(1601)
+    assert FakeSidecar.built == 4 and rt.STATS["prefix_extend_rejects"]["delta_too_large"] == 1
+    # the sidecar may decline (returns None): rebuild, and say why
+    requests["r0"] = types.SimpleNamespace(prompt_token_ids=[1] * 700 + [2] * 900 + [3] * 10)
+    rt.state_for(impl, layer)["sidecar"].fail = True
+    monkeypatch.setattr(FakeSidecar, "forward", lambda self, q: torch.full((1, self.hq, 128), float(self.length)))
+    go(1611)
+    assert FakeSidecar.built == 5 and rt.STATS["prefix_extend_rejects"]["adapter_declined"] == 1
+    # the pure matcher: remaining reasons
+    md = meta(800)
+    assert rt.prefix_extend_match(md, None, 500, 800)[:2] == (False, "no_checkpoint")
+    assert rt.prefix_extend_match(md, (499, b"x"), 502, 800)[:2] == (False, "checkpoint_inconsistent")
+    assert rt.prefix_extend_match(md, (799, b"x"), 800, 800)[:2] == (False, "not_longer")
+    assert rt.prefix_extend_match(md, (499, b"x"), 500, 800)[:2] == (False, "no_runner")
+    md._pq_runner = types.SimpleNamespace(input_batch=types.SimpleNamespace(req_ids=["r0"]),
+                                          requests={"r0": types.SimpleNamespace(prompt_token_ids=[0] * 5)})
+    assert rt.prefix_extend_match(md, (499, b"x"), 500, 800)[:2] == (False, "prompt_len_mismatch")
+
+
 def test_copy_ctx_and_as_decode_qkv():
     out = torch.zeros(2, 8, 128, dtype=torch.bfloat16)
     rt.copy_ctx(out, torch.ones(1, 8 * 128), 1)
