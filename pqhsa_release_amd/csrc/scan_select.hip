@@ -62,6 +62,7 @@ struct ScanArgs {
     // kWrite
     float *logits_out;
     int64_t logits_out_stride;
+    int by_xcd;  // streams are dealt to the 8 XCDs (stream count a multiple of 8): see scan_kernel
     // kHist
     uint32_t *hist;  // [rows, 2048]
     // kEmit
@@ -106,9 +107,20 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int bh = blockIdx.y;
+    int bh = blockIdx.y, tile = blockIdx.x;
+    if constexpr (MODE == kWrite) {
+        // Workgroups go to the 8 XCDs in turn, in launch order.  With an index sorted by list the
+        // logits of a stream are scattered over its whole output rows; when all workgroups of a
+        // stream run on one XCD, its L2 collects the scattered 4-byte writes into whole lines
+        // before they go to memory (2 MB of rows per stream at 131 072 keys and 4 query rows).
+        if (a.by_xcd) {
+            const uint32_t id = blockIdx.x + gridDim.x * blockIdx.y, tiles = gridDim.x;
+            bh = (int)((id & 7u) + 8u * (id / (8u * tiles)));
+            tile = (int)((id >> 3) % tiles);
+        }
+    }
     const int n = a.n_arr[bh / a.n_div];
-    const int tile0 = blockIdx.x * a.tile_keys;
+    const int tile0 = tile * a.tile_keys;
     if (tile0 >= n) return;
     const int tile_end = min(n, tile0 + a.tile_keys);
     const int L = a.L;
@@ -1418,6 +1430,7 @@ extern "C" int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max
     a.n_arr = index->n_idx; a.n_div = index->kv_heads; a.G = G;
     a.tile_keys = pick_tile_keys(n_max, streams);
     a.logits_out = logits; a.logits_out_stride = logit_stride;
+    a.by_xcd = streams % 8 == 0;
     return launch_scan(a, kWrite, kIndex, padded_groups(G), streams, n_max, static_cast<hipStream_t>(stream));
 }
 
