@@ -92,6 +92,23 @@ __device__ inline void lds_vec(const float *p, float (&v)[GP]) {
     }
 }
 
+// PQ table entry (m * 16 + code) of every query row.  In LDS the table is kept as one sub-table per
+// pair of query rows, [pair][128 entries][2]: the 16 codewords of a subspace then fill exactly one
+// 128-byte row of the 32 LDS banks, so the 64 lanes of a look-up (16 distinct addresses at most)
+// never meet in a bank, whereas 16-byte entries spread a subspace over two rows that share banks.
+template <int GP>
+__device__ inline void lut_entry(const float *lut_s, uint32_t entry, float (&v)[GP]) {
+    if constexpr (GP >= 2) {
+#pragma unroll
+        for (int p = 0; p < GP / 2; ++p) {
+            const float2 t = reinterpret_cast<const float2 *>(lut_s)[p * (kM * kCodes) + entry];
+            v[2 * p] = t.x; v[2 * p + 1] = t.y;
+        }
+    } else {
+        v[0] = lut_s[entry];
+    }
+}
+
 // logit of one stored key for one query row, in the fixed summation order of the CPU oracle
 __device__ inline float score_one(const float *lut_col, const float *ls_col, uint32_t code, uint32_t lid, float qn,
                                   float kn, float scale) {
@@ -144,16 +161,76 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int cap_w = MODE == kEmit ? a.stage_cap : 0;
     uint16_t *stage_aux = reinterpret_cast<uint16_t *>(stage_s + (size_t)kScanWaves * GP * cap_w);
 
+    // The index words of a block of keys.  A thread asks for its next block before it works on the
+    // one it holds, and for its first block before the tables are staged, so that the memory
+    // round trips overlap the table fill and the arithmetic.
+    struct KeyWords {
+        uint4 cw;
+        uint2 lw;
+        float4 nw;
+        int4 pw;
+    };
+    const size_t base = (size_t)bh * a.n_cap;
+    auto fetch = [&](int i) {
+        KeyWords w;
+        w.cw = make_uint4(0, 0, 0, 0); w.lw = make_uint2(0, 0); w.nw = make_float4(0, 0, 0, 0);
+        w.pw = make_int4(i, i + 1, i + 2, i + 3);
+        if constexpr (SRC == kIndex) {
+            if (i < tile_end) {
+                w.cw = *reinterpret_cast<const uint4 *>(a.codes + base + i);
+                w.lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + i);
+                w.nw = *reinterpret_cast<const float4 *>(a.norms + base + i);
+                // candidates are recorded, and logits written, under the retrieval-local index
+                if (a.pos) w.pw = *reinterpret_cast<const int4 *>(a.pos + base + i);
+            }
+        }
+        return w;
+    };
+    KeyWords cur = fetch(tile0 + tid * kKeysPerThread);
+
     float qn[GP];
     if constexpr (SRC == kIndex) {
+        // all table loads are requested before the first is stored
+        constexpr int kLutVec = kM * kCodes * GP / 4;                       // float4 words of the PQ table
+        constexpr int kLutPer = (kLutVec + kScanThreads - 1) / kScanThreads;
         const float4 *src = reinterpret_cast<const float4 *>(a.lut + (size_t)bh * kM * kCodes * GP);
-        for (int i = tid; i < kM * kCodes * GP / 4; i += kScanThreads) reinterpret_cast<float4 *>(lut_s)[i] = src[i];
+        float4 lut_r[kLutPer];
+#pragma unroll
+        for (int u = 0; u < kLutPer; ++u) {
+            const int i = tid + u * kScanThreads;
+            lut_r[u] = i < kLutVec ? src[i] : make_float4(0, 0, 0, 0);
+        }
         if constexpr (GP >= 4) {
             const float4 *ls = reinterpret_cast<const float4 *>(a.list_scores + (size_t)bh * L * GP);
-            for (int i = tid; i < L * GP / 4; i += kScanThreads) reinterpret_cast<float4 *>(ls_s)[i] = ls[i];
+            const int nvec = L * GP / 4;
+            float4 ls_r[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = tid + u * kScanThreads;
+                ls_r[u] = i < nvec ? ls[i] : make_float4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = tid + u * kScanThreads;
+                if (i < nvec) reinterpret_cast<float4 *>(ls_s)[i] = ls_r[u];
+            }
+            for (int i = tid + 2 * kScanThreads; i < nvec; i += kScanThreads) reinterpret_cast<float4 *>(ls_s)[i] = ls[i];
         } else {
             const float *ls = a.list_scores + (size_t)bh * L * GP;
             for (int i = tid; i < L * GP; i += kScanThreads) ls_s[i] = ls[i];
+        }
+#pragma unroll
+        for (int u = 0; u < kLutPer; ++u) {
+            const int i = tid + u * kScanThreads;
+            if (i >= kLutVec) continue;
+            if constexpr (GP >= 4) {  // word i holds rows 4q .. 4q+3 of entry e: two pair sub-tables
+                const int e = i / (GP / 4), q = i % (GP / 4);
+                float2 *pair = reinterpret_cast<float2 *>(lut_s);
+                pair[(2 * q) * (kM * kCodes) + e] = make_float2(lut_r[u].x, lut_r[u].y);
+                pair[(2 * q + 1) * (kM * kCodes) + e] = make_float2(lut_r[u].z, lut_r[u].w);
+            } else {
+                reinterpret_cast<float4 *>(lut_s)[i] = lut_r[u];
+            }
         }
 #pragma unroll
         for (int g = 0; g < GP; ++g) qn[g] = a.qnorm[(size_t)bh * GP + g];
@@ -182,28 +259,17 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     }
     __syncthreads();
 
-    const size_t base = (size_t)bh * a.n_cap;
     // every lane of a wave runs the same number of iterations (the wave's first key decides)
     for (int i0 = tile0 + tid * kKeysPerThread; i0 - lane * kKeysPerThread < tile_end; i0 += kKeysPerIter) {
         float s[kKeysPerThread][GP];
         uint32_t lid[kKeysPerThread];
-        uint32_t ridx[kKeysPerThread] = {(uint32_t)i0, (uint32_t)i0 + 1u, (uint32_t)i0 + 2u, (uint32_t)i0 + 3u};
-        const bool in_range = i0 < tile_end;
+        const uint4 cw = cur.cw;
+        const uint2 lw = cur.lw;
+        const float4 nw = cur.nw;
+        const int4 pw = cur.pw;
+        const uint32_t ridx[kKeysPerThread] = {(uint32_t)pw.x, (uint32_t)pw.y, (uint32_t)pw.z, (uint32_t)pw.w};
+        cur = fetch(i0 + kKeysPerIter);
         if constexpr (SRC == kIndex) {
-            uint4 cw = make_uint4(0, 0, 0, 0);
-            uint2 lw = make_uint2(0, 0);
-            float4 nw = make_float4(0, 0, 0, 0);
-            if (in_range) {
-                cw = *reinterpret_cast<const uint4 *>(a.codes + base + i0);
-                lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + i0);
-                nw = *reinterpret_cast<const float4 *>(a.norms + base + i0);
-                if constexpr (MODE == kEmit) {  // candidates are recorded under their retrieval-local index
-                    if (a.pos) {
-                        const int4 pw = *reinterpret_cast<const int4 *>(a.pos + base + i0);
-                        ridx[0] = (uint32_t)pw.x; ridx[1] = (uint32_t)pw.y; ridx[2] = (uint32_t)pw.z; ridx[3] = (uint32_t)pw.w;
-                    }
-                }
-            }
             const uint32_t c[4] = {cw.x, cw.y, cw.z, cw.w};
             const float kn[4] = {nw.x, nw.y, nw.z, nw.w};
             lid[0] = lw.x & 0xffffu; lid[1] = lw.x >> 16; lid[2] = lw.y & 0xffffu; lid[3] = lw.y >> 16;
@@ -222,7 +288,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
 #pragma unroll
                     for (int j = j0; j < j0 + KB; ++j) {
                         float v[GP];
-                        lds_vec<GP>(lut_s + (size_t)(m * kCodes + ((c[j] >> (4 * m)) & 15u)) * GP, v);
+                        lut_entry<GP>(lut_s, m * kCodes + ((c[j] >> (4 * m)) & 15u), v);
 #pragma unroll
                         for (int g = 0; g < GP; ++g) s[j][g] = m == 0 ? v[g] : s[j][g] + v[g];
                     }
@@ -251,11 +317,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         }
 
         if constexpr (MODE == kWrite) {
-            int32_t col[4] = {i0, i0 + 1, i0 + 2, i0 + 3};
-            if (a.pos && in_range) {  // stored positions come in fours, the row's capacity is a multiple of 4
-                const int4 pw = *reinterpret_cast<const int4 *>(a.pos + base + i0);
-                col[0] = pw.x; col[1] = pw.y; col[2] = pw.z; col[3] = pw.w;
-            }
+            const int32_t col[4] = {pw.x, pw.y, pw.z, pw.w};
             // four keys that land side by side (an index still in arrival order) go out as one
             // 16-byte store when the destination row allows it
             const bool quad = i0 + 4 <= tile_end && (col[0] & 3) == 0 && col[1] == col[0] + 1 && col[2] == col[0] + 2 &&

@@ -353,7 +353,7 @@ def lut_scan(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scale: fl
 
 def topk_radix(logits: torch.Tensor, n, k):
     """Exact top-k of each row of ``logits [rows, stride]``; ``n``/``k`` per row.  Returns
-    (indices int32 [rows, k_cap], values f32 [rows, k_cap]) in ascending index order."""
+    (indices int32 [rows, k_cap], values f32 [rows, k_cap]), the selected keys in no particular order."""
     _need_cuda(logits)
     lib = _lib.load()
     if logits.ndim != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
