@@ -252,7 +252,11 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         for (int g = 0; g < GP; ++g) {
             const uint32_t tk = a.thr_key[(size_t)bh * GP + g];
             const float rv = a.ref_val[(size_t)bh * GP + g];
-            thr_f[g] = tk == 0u ? -3.402823466e38f : key_to_float(tk);
+            // Keys up to that of -inf (0x007fffff) are not keys of ordered floats: such a
+            // threshold keeps every key.  Index logits are finite and slots past the tile carry
+            // -inf, so the bound is the lowest finite float; a logit matrix may hold -inf itself
+            // (masked entries), so there the bound is -inf and the slots past the tile carry NaN.
+            thr_f[g] = tk <= 0x007fffffu ? (SRC == kLogits ? -INFINITY : -3.402823466e38f) : key_to_float(tk);
             nref2[g] = g < a.G ? (__builtin_isfinite(rv) ? -rv * kLog2e : 0.0f) : -INFINITY;
             wcnt[g] = 0u;
         }
@@ -347,14 +351,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         } else {
             // ---- candidates and background weights ------------------------------------------
-            // Keys past the end of the tile score -inf: never candidates, weight 0.
+            // Keys past the end of the tile score -inf (NaN for a logit matrix): never candidates, weight 0.
             const int wave_first = i0 - lane * kKeysPerThread;
             if (wave_first + kWaveKeys > tile_end) {  // wave-uniform: only the last window of a row
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     if (i0 + j < tile_end) continue;
 #pragma unroll
-                    for (int g = 0; g < GP; ++g) s[j][g] = -INFINITY;
+                    for (int g = 0; g < GP; ++g) s[j][g] = SRC == kLogits ? __builtin_nanf("") : -INFINITY;
                 }
             }
             uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
@@ -698,30 +702,6 @@ struct __align__(16) SelScratch {
     uint32_t bin, above;        // the range of the k-th key and the number of keys in higher ranges
     uint32_t sel_key, sel_idx;  // the k-th key and, among equal keys, the largest index still selected
 };
-
-// The bit-by-bit search over keys in memory (any count).
-template <typename KeyAt>
-__device__ inline uint32_t bisect_mem(KeyAt key_at, uint32_t cnt, uint32_t want, uint32_t (*red)[kSelWaves],
-                                      int &step, bool &exact) {
-    uint32_t t = 0u;
-    exact = false;
-    const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
-    for (int bit = 31; bit >= 0; --bit) {
-        const uint32_t trial = t | (1u << bit);
-        uint32_t c = 0;
-        for (uint32_t r = 0; r < rounds; ++r) {
-            const uint32_t p = r * kSelThreads + threadIdx.x;
-            c += wave_count_if(p < cnt && key_at(p) >= trial);
-        }
-        c = block_total_of_waves(c, red, step++);
-        if (c >= want) t = trial;
-        if (c == want) {
-            exact = true;
-            break;
-        }
-    }
-    return t;
-}
 
 // ---- threshold estimate from the sampled keys ---------------------------------------------------
 // One workgroup per (query row, stream).  With ns sampled keys out of n, keeping every key down
@@ -1097,18 +1077,91 @@ __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, cons
     select_loaded<R>(key, where, list, cnt, k, out, red, wsum, ss, ref1_out);
 }
 
+// The want-th largest of the values val_at(p) (p < cnt; val_at returns false for entries that do
+// not take part), any count, values read from memory on every pass.  The range [lo, hi] that holds
+// the answer starts as [smallest, largest] and shrinks by a factor of 1024 per pass: a histogram
+// of the values over 1024 equal sub-ranges tells which sub-range the want-th largest falls in.
+// At most four passes after the one that finds the range, whatever the values (equal values
+// included).  `above` returns how many values are larger than the result.  With fewer than want
+// values the result is the smallest one.  All 1024 threads call this; `span` is 2 * kSelWaves words.
+template <typename ValAt>
+__device__ inline uint32_t kth_largest_mem(ValAt val_at, uint32_t cnt, uint32_t want, SelScratch *ss, uint32_t *span,
+                                           uint32_t &above) {
+    const int tid = threadIdx.x;
+    uint32_t hi = 0u, lo = 0xffffffffu;
+    for (uint32_t p = tid; p < cnt; p += kSelThreads) {
+        uint32_t v;
+        if (val_at(p, v)) {
+            hi = max(hi, v);
+            lo = min(lo, v);
+        }
+    }
+    hi = wave_max_u32(hi);
+    lo = ~wave_max_u32(~lo);
+    __syncthreads();
+    if ((tid & (kWave - 1)) == 0) {
+        span[tid / kWave] = hi;
+        span[kSelWaves + tid / kWave] = lo;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) {
+        hi = max(hi, span[w]);
+        lo = min(lo, span[kSelWaves + w]);
+    }
+    above = 0u;
+    while (lo < hi) {  // the same for every thread
+        const int shift = max(0, (32 - __clz(hi - lo)) - 10);  // (hi - lo) >> shift < 1024
+        for (int i = tid; i < kSelBins; i += kSelThreads) ss->hist[i] = 0u;
+        if (tid == 0) {
+            ss->bin = 0u;
+            ss->above = 0u;
+        }
+        __syncthreads();
+        for (uint32_t p = tid; p < cnt; p += kSelThreads) {
+            uint32_t v;
+            if (val_at(p, v) && v >= lo && v <= hi) atomicAdd(&ss->hist[(v - lo) >> shift], 1u);
+        }
+        __syncthreads();
+        if (tid < kWave) find_from_top_1024(ss->hist, want - above, &ss->bin, &ss->above);
+        __syncthreads();
+        const uint32_t nlo = lo + (ss->bin << shift);
+        const uint32_t width = (1u << shift) - 1u;
+        above += ss->above;
+        hi = hi - nlo > width ? nlo + width : hi;
+        lo = nlo;
+        __syncthreads();  // everyone has read the result before the histogram is cleared again
+    }
+    return lo;
+}
+
 // Candidates in memory (any count): the same selection, streaming the pairs on every pass.
 __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
                                   SelectOut out, uint32_t (*red)[kSelWaves],
-                                  uint32_t *wsum, float *ref1_out) {
+                                  uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     const int tid = threadIdx.x;
     const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
     auto key_at = [=](uint32_t p) { return pairs[p].x; };
     int step = 0;
-    bool exact = false;
     uint32_t tkey = 0u;
+    uint32_t idx_thr = 0xffffffffu;
     if (k > 0) {
-        tkey = bisect_mem(key_at, cnt, (uint32_t)k, red, step, exact);
+        uint32_t c_gt = 0u;
+        tkey = kth_largest_mem([=](uint32_t p, uint32_t &v) { v = pairs[p].x; return true; }, cnt, (uint32_t)k, ss, wsum, c_gt);
+        uint32_t c_eq = 0;
+        for (uint32_t r = 0; r < rounds; ++r) {
+            const uint32_t p = r * kSelThreads + tid;
+            c_eq += wave_count_if(p < cnt && key_at(p) == tkey);
+        }
+        c_eq = block_total_of_waves(c_eq, red, step++);
+        const uint32_t want_ties = (uint32_t)k > c_gt ? (uint32_t)k - c_gt : 0u;
+        if (c_eq > want_ties) {
+            // among equal keys the lowest indices win: the want_ties-th largest of ~index
+            uint32_t unused;
+            const uint32_t t = tkey;
+            idx_thr = ~kth_largest_mem([=](uint32_t p, uint32_t &v) { const uint2 pr = pairs[p]; v = ~pr.y; return pr.x == t; },
+                                       cnt, want_ties, ss, wsum, unused);
+        }
     } else {
         uint32_t kmax = 0u;
         for (uint32_t p = tid; p < cnt; p += kSelThreads) kmax = max(kmax, key_at(p));
@@ -1117,38 +1170,6 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
         if ((tid & (kWave - 1)) == 0) wsum[tid / kWave] = kmax;
         __syncthreads();
         for (int w = 0; w < kSelWaves; ++w) tkey = max(tkey, wsum[w]);
-    }
-    uint32_t idx_thr = 0xffffffffu;
-    if (k > 0 && !exact) {
-        uint32_t c_gt = 0, c_eq = 0;
-        for (uint32_t r = 0; r < rounds; ++r) {
-            const uint32_t p = r * kSelThreads + tid;
-            const uint32_t kk = p < cnt ? key_at(p) : 0u;
-            c_gt += wave_count_if(p < cnt && kk > tkey);
-            c_eq += wave_count_if(p < cnt && kk == tkey);
-        }
-        c_gt = block_total_of_waves(c_gt, red, step++);
-        c_eq = block_total_of_waves(c_eq, red, step++);
-        const uint32_t want_ties = (uint32_t)k - c_gt;
-        if (c_eq > want_ties) {
-            uint32_t lo = 0u;
-            for (int bit = 31; bit >= 0; --bit) {
-                const uint32_t trial = lo | (1u << bit);
-                uint32_t c = 0;
-                for (uint32_t r = 0; r < rounds; ++r) {
-                    const uint32_t p = r * kSelThreads + tid;
-                    bool hit = false;
-                    if (p < cnt) {
-                        const uint2 pr = pairs[p];
-                        hit = pr.x == tkey && pr.y < trial;
-                    }
-                    c += wave_count_if(hit);
-                }
-                c = block_total_of_waves(c, red, step++);
-                if (c < want_ties) lo = trial;
-            }
-            idx_thr = lo;
-        }
     }
     auto selected = [=](uint2 pr) {
         if (k <= 0) return false;
@@ -1257,9 +1278,9 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
             else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
             else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
+            else select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
         } else {  // the estimate was exceeded, or the row was re-scanned (rare): stream from memory
-            select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ref1);
+            select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
         }
     }
     __syncthreads();

@@ -607,3 +607,37 @@ def test_topk_radix_on_tie_heavy_matrices():
             got = idx[r, : k[r]]
             assert np.array_equal(np.sort(got), np.sort(want_idx)), (case, kind, r, n[r], k[r])
             assert np.array_equal(val[r, : k[r]], x[r, got]), (case, kind, r)
+
+
+def test_topk_radix_many_candidates_selected_from_memory():
+    """More than 16 384 candidates per row (large k, or a k-th value shared by most of the row) are
+    selected by passes over the candidates in memory: a 1024-way range split per pass, on the keys
+    and then on the indices of the keys that tie.  Rows cover the whole float range (several
+    splits), infinities, two-valued and constant rows (every candidate ties)."""
+    dev = _cuda()
+    rng = np.random.default_rng(29)
+    stride = 70000
+    wide = rng.integers(0, 2 ** 32, size=stride, dtype=np.uint64).astype(np.uint32).view(np.float32).copy()
+    wide[np.isnan(wide)] = 0.0
+    rows = [
+        (np.full(stride, 0.125, np.float32), stride, 2000),                      # all equal: indices 0..k-1
+        (np.full(stride, -np.inf, np.float32), 65537, 40000),
+        (rng.choice(np.array([1.0, 2.0], np.float32), size=stride), stride, 50000),   # boundary inside the 1.0 ties
+        (rng.standard_normal(stride).astype(np.float32), stride, stride // 3),
+        (rng.standard_normal(stride).astype(np.float32), 60001, 60001),          # k = n
+        (wide, stride, 30000),                                                    # bit patterns over the whole range
+        (np.round(rng.standard_normal(stride), 1).astype(np.float32), stride, 35000),
+        (np.where(rng.random(stride) < 0.9, np.float32(3.0), rng.standard_normal(stride).astype(np.float32)).astype(np.float32),
+         stride, 100),                                                            # small k, k-th value shared by 90 % of the row
+    ]
+    x = np.stack([r[0] for r in rows])
+    n, k = [r[1] for r in rows], [r[2] for r in rows]
+    idx, val = ops.topk_radix(torch.from_numpy(x).to(dev), n, k)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    for r in range(len(rows)):
+        want_idx, _ = fixed.topk(x[r, : n[r]], k[r])
+        got = idx[r, : k[r]]
+        assert np.array_equal(np.sort(got), np.sort(want_idx)), (r, n[r], k[r])
+        assert np.array_equal(val[r, : k[r]], x[r, got]), r
+
