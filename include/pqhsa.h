@@ -178,7 +178,9 @@ int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max, const flo
  * Exact top-k of each row of a logit matrix [rows, stride] by radix selection on the fp32
  * bit pattern (no sort); ties at the k boundary go to the lowest index; the k winners are
  * written (in no particular order) with their logits.  n[r] and k[r] are per-row device
- * arrays.  Replaces torch.topk in the reference path
+ * arrays.  Entries are ordered by bit pattern: -0 equals +0, -inf is the lowest value, +inf
+ * the highest number, and a NaN with the sign bit clear ranks above +inf (torch.topk's rule).
+ * Replaces torch.topk in the reference path
  * (pq_hsa/attention/sparse_attention.py:661-666) and the binding pq_topk_radix
  * (pq_hsa/kernels/cuda/pq_fused_h20.cu:3624-3688).
  */

@@ -238,10 +238,11 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     if constexpr (MODE == kHist) {
         for (int i = tid; i < GP * kHistBins; i += kScanThreads) hist_s[i] = 0u;
     }
-    // A key is a candidate when its logit, as a float, reaches the threshold: the same order as
-    // on the 32-bit keys (-0 and +0 compare equal, as their keys do).  Threshold key 0 keeps every
-    // key, key 0xffffffff (a NaN as a float) keeps none.
+    // A key of the index is a candidate when its logit, as a float, reaches the threshold: the same
+    // order as on the 32-bit keys (-0 and +0 compare equal, as their keys do).  Threshold key 0
+    // keeps every key, key 0xffffffff (a NaN as a float) keeps none.
     float thr_f[GP];
+    uint32_t thr_k[GP];  // a logit matrix may hold infinities and NaNs: its entries are compared by key
     float nref2[GP];    // -reference * log2(e); -inf for padded rows so that their weights are 0
     uint32_t wcnt[GP];  // candidates this wave has staged per row (wave-uniform)
     constexpr float kLog2e = 1.4426950408889634f;
@@ -252,11 +253,10 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         for (int g = 0; g < GP; ++g) {
             const uint32_t tk = a.thr_key[(size_t)bh * GP + g];
             const float rv = a.ref_val[(size_t)bh * GP + g];
-            // Keys up to that of -inf (0x007fffff) are not keys of ordered floats: such a
-            // threshold keeps every key.  Index logits are finite and slots past the tile carry
-            // -inf, so the bound is the lowest finite float; a logit matrix may hold -inf itself
-            // (masked entries), so there the bound is -inf and the slots past the tile carry NaN.
-            thr_f[g] = tk <= 0x007fffffu ? (SRC == kLogits ? -INFINITY : -3.402823466e38f) : key_to_float(tk);
+            // keys below that of the lowest finite float are not keys of ordered floats: such a
+            // threshold keeps every key of the index (its logits are finite)
+            thr_f[g] = tk < 0x00800000u ? -3.402823466e38f : key_to_float(tk);
+            thr_k[g] = tk;
             nref2[g] = g < a.G ? (__builtin_isfinite(rv) ? -rv * kLog2e : 0.0f) : -INFINITY;
             wcnt[g] = 0u;
         }
@@ -351,14 +351,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         } else {
             // ---- candidates and background weights ------------------------------------------
-            // Keys past the end of the tile score -inf (NaN for a logit matrix): never candidates, weight 0.
+            // Keys past the end of the tile score -inf: never candidates, weight 0.
             const int wave_first = i0 - lane * kKeysPerThread;
             if (wave_first + kWaveKeys > tile_end) {  // wave-uniform: only the last window of a row
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     if (i0 + j < tile_end) continue;
 #pragma unroll
-                    for (int g = 0; g < GP; ++g) s[j][g] = SRC == kLogits ? __builtin_nanf("") : -INFINITY;
+                    for (int g = 0; g < GP; ++g) s[j][g] = -INFINITY;
                 }
             }
             uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
@@ -369,7 +369,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
                 emit_mask[g] = 0u;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const bool cand = s[j][g] >= thr_f[g];
+                    const bool cand = SRC == kLogits ? (i0 + j < tile_end && order_key(s[j][g]) >= thr_k[g])
+                                                     : s[j][g] >= thr_f[g];
                     if (cand) emit_mask[g] |= 1u << j;
                     if (want_mass) e[j][g] = cand ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
                 }

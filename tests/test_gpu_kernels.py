@@ -630,6 +630,11 @@ def test_topk_radix_many_candidates_selected_from_memory():
         (np.where(rng.random(stride) < 0.9, np.float32(3.0), rng.standard_normal(stride).astype(np.float32)).astype(np.float32),
          stride, 100),                                                            # small k, k-th value shared by 90 % of the row
     ]
+    # special values order by their bit patterns, as in the oracle: NaN above +inf, -inf lowest
+    special = rng.standard_normal(stride).astype(np.float32)
+    u = rng.random(stride)
+    special[u < 0.05], special[(u >= 0.05) & (u < 0.10)], special[u > 0.80] = np.nan, np.inf, -np.inf
+    rows += [(special, stride, 2000), (special, stride, 9000), (special, 69999, 60000)]
     x = np.stack([r[0] for r in rows])
     n, k = [r[1] for r in rows], [r[2] for r in rows]
     idx, val = ops.topk_radix(torch.from_numpy(x).to(dev), n, k)
@@ -639,5 +644,5 @@ def test_topk_radix_many_candidates_selected_from_memory():
         want_idx, _ = fixed.topk(x[r, : n[r]], k[r])
         got = idx[r, : k[r]]
         assert np.array_equal(np.sort(got), np.sort(want_idx)), (r, n[r], k[r])
-        assert np.array_equal(val[r, : k[r]], x[r, got]), r
+        assert np.array_equal(val[r, : k[r]], x[r, got], equal_nan=True), r
 
