@@ -318,6 +318,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--layers", type=int, default=3, help="distinct resident layers rotated through (defeats cache reuse)")
+    ap.add_argument("--event-every", type=int, default=8,
+                    help="in the timed region the dominant kernel is bracketed by HIP events on one step in this many")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--append", action="store_true",
@@ -366,10 +368,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    def logged_run(count, only):
-        """count steps with the HIP-event log on the stream; returns (ms per step, per-kernel ms)."""
+    def logged_run(count, only, every=1):
+        """count steps with the HIP-event log on the stream, one step in `every` carrying the
+        records; returns (ms per step, per-kernel ms averaged over the logged steps)."""
         _lib.check(lib.pqhsa_profile_enable(count), "pqhsa_profile_enable")
         _lib.check(lib.pqhsa_profile_only(only), "pqhsa_profile_only")
+        _lib.check(lib.pqhsa_profile_every(every), "pqhsa_profile_every")
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         run_steps(count)
@@ -378,17 +382,17 @@ def main():
         kms = (ctypes.c_float * len(KERNELS))()
         seen = ctypes.c_int32(0)
         _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
-        assert seen.value == count, (seen.value, count)
+        assert seen.value == (count + every - 1) // every, (seen.value, count, every)
         return (t1 - t0) * 1000.0 / count, [float(v) for v in kms]
 
     # untimed survey with every kernel bracketed by events: finds the dominant kernel
     _, survey = logged_run(max(args.warmup, 20), -1)
     dominant_i = max(range(len(KERNELS)), key=lambda i: survey[i])
     dominant = KERNELS[dominant_i]
-    # timed region: exactly --steps steps; only the dominant kernel carries events (two records
-    # per step), which is what its roofline figure is measured from
-    ms_per_step, dom_ms = logged_run(args.steps, dominant_i)
-    # the same steps with no event at all, to show what the two records cost
+    # timed region: exactly --steps steps; the dominant kernel carries two event records on one
+    # step in --event-every, spread over the whole region: what its roofline figure is measured from
+    ms_per_step, dom_ms = logged_run(args.steps, dominant_i, max(1, args.event_every))
+    # the same steps with no event at all, to show what the records cost
     run_steps(args.warmup)
     torch.cuda.synchronize()
     t2 = time.perf_counter()
@@ -433,6 +437,7 @@ def main():
         "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get(dominant),
         "algorithmic_bytes": dom_bytes,
         "launch_us": round(dom_us, 3),
+        "launches_timed": (args.steps + max(1, args.event_every) - 1) // max(1, args.event_every),
     }
     scan_us = kus["scan_emit"]
     result = {

@@ -294,11 +294,15 @@ int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq,
  * attend_partial, attend_reduce) and the number of steps seen, and turns profiling off.
  * pqhsa_profile_only(kernel), called after enable, restricts the log to the two events around
  * one kernel (-1: all), so that a timed run carries two event records per step instead of
- * seven; the other entries of kernel_ms are then 0.  Not thread-safe; meant for benchmarks.
+ * seven; the other entries of kernel_ms are then 0.  pqhsa_profile_every(stride), also after
+ * enable, logs one decode step in `stride` (the first, then every stride-th): a timed run then
+ * carries the event records on a sample of its steps only, and `steps` counts the logged ones.
+ * Not thread-safe; meant for benchmarks.
  */
 #define PQHSA_PROFILE_KERNELS 6
 int pqhsa_profile_enable(int32_t max_steps);
 int pqhsa_profile_only(int32_t kernel);
+int pqhsa_profile_every(int32_t stride);
 int pqhsa_profile_collect(float *kernel_ms, int32_t *steps);
 
 #ifdef __cplusplus

@@ -106,6 +106,7 @@ SIGNATURES = {
                                                 c_void_p]),
     "pqhsa_profile_enable": (ctypes.c_int, [c_int32]),
     "pqhsa_profile_only": (ctypes.c_int, [c_int32]),
+    "pqhsa_profile_every": (ctypes.c_int, [c_int32]),
     "pqhsa_profile_collect": (ctypes.c_int, [c_void_p, c_void_p]),
     "pqhsa_paged_gather_at": (ctypes.c_int, [_P(KvView), c_int32, c_int32, c_void_p, c_int64, c_void_p, c_void_p,
                                              c_void_p]),

@@ -53,12 +53,18 @@ static std::vector<hipEvent_t> g_events;
 static int g_prof_steps = 0, g_prof_step = 0;
 static bool g_prof_on = false;
 static int g_prof_only = -1;  // >= 0: only this kernel is bracketed by events
+static int g_prof_every = 1;  // one decode step in this many is logged
+static int g_prof_seen = 0;   // decode steps since the log was enabled
 
 void profile_mark(int slot, hipStream_t stream) {
     if (!g_prof_on || g_prof_step >= g_prof_steps) return;
-    if (g_prof_only < 0 || slot == g_prof_only || slot == g_prof_only + 1)
+    const bool logged = g_prof_seen % g_prof_every == 0;
+    if (logged && (g_prof_only < 0 || slot == g_prof_only || slot == g_prof_only + 1))
         (void)hipEventRecord(g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot], stream);
-    if (slot == kProfKernels) ++g_prof_step;
+    if (slot == kProfKernels) {
+        if (logged) ++g_prof_step;
+        ++g_prof_seen;
+    }
 }
 
 }  // namespace pqhsa
@@ -78,6 +84,15 @@ extern "C" int pqhsa_profile_enable(int32_t max_steps) {
     g_prof_step = 0;
     g_prof_on = true;
     g_prof_only = -1;
+    g_prof_every = 1;
+    g_prof_seen = 0;
+    return PQHSA_OK;
+}
+
+extern "C" int pqhsa_profile_every(int32_t stride) {
+    using namespace pqhsa;
+    PQHSA_REQUIRE(stride >= 1, "profile_every: stride=%d", stride);
+    g_prof_every = stride;
     return PQHSA_OK;
 }
 
