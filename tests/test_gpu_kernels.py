@@ -646,3 +646,43 @@ def test_topk_radix_many_candidates_selected_from_memory():
         assert np.array_equal(np.sort(got), np.sort(want_idx)), (r, n[r], k[r])
         assert np.array_equal(val[r, : k[r]], x[r, got], equal_nan=True), r
 
+
+def test_event_log_counts_steps_and_samples_them():
+    """The per-kernel event log of the decode step: every step logged, one kernel only, and one
+    step in three; the number of logged steps and which kernels carry a time."""
+    import ctypes
+    from pqhsa_release_amd import _lib
+
+    dev = _cuda()
+    lib = _lib.load()
+    p = Problem(lens=[3000], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=61)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.02, 0))
+    q = p.q_tensor()
+    out = torch.empty_like(q)
+
+    def steps(count):
+        for _ in range(count):
+            ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
+                            fraction=0.02, topk=0, scale=SCALE, workspace=ws)
+
+    def collect():
+        kms = (ctypes.c_float * 6)()
+        seen = ctypes.c_int32(-1)
+        _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
+        return seen.value, [float(v) for v in kms]
+
+    _lib.check(lib.pqhsa_profile_enable(16), "enable")
+    steps(5)
+    seen, kms = collect()
+    assert seen == 5 and all(0.0 < v < 50.0 for v in kms), (seen, kms)
+    _lib.check(lib.pqhsa_profile_enable(16), "enable")
+    _lib.check(lib.pqhsa_profile_only(4), "only")
+    _lib.check(lib.pqhsa_profile_every(3), "every")
+    steps(7)                                       # steps 0, 3 and 6 are logged
+    seen, kms = collect()
+    assert seen == 3 and kms[4] > 0.0 and all(v == 0.0 for i, v in enumerate(kms) if i != 4), (seen, kms)
+    steps(2)                                       # the log is off again: nothing recorded, nothing to collect
+    assert lib.pqhsa_profile_every(0) != 0 and b"stride" in lib.pqhsa_last_error()
+
