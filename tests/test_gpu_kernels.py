@@ -361,50 +361,55 @@ def test_hybrid_attend_paged_alone_matches_oracle():
         assert np.abs(o[b, h] - w).max() <= 2e-3, (b, h, np.abs(o[b, h] - w).max())
 
 
-def test_full_size_step_properties_at_the_cfg1_shape():
-    """At a full configuration size (context 32 768, 8 KV heads, GQA 4, bf16 paged) the oracle is
-    too slow, so the step is checked through properties: the selected set is exactly the k best of
-    the logits pqhsa_lut_scan writes for the same tables, nothing was re-scanned, and the output
-    equals a dense torch attention in which unselected stored keys are replaced by their list's
-    mean value under the approximate logits."""
+@pytest.mark.parametrize("cfg", [1, 2])
+def test_full_size_step_properties_at_the_benchmark_shapes(cfg):
+    """At the full configuration sizes (cfg 1: context 32 768, one sequence; cfg 2, the headline:
+    context 131 072, batch 4; both 8 KV heads, GQA 4, bf16 paged) the oracle is too slow, so the
+    step is checked through properties: the selected set is exactly the k best of the logits
+    pqhsa_lut_scan writes for the same tables, nothing was re-scanned, and the output equals a
+    dense torch attention in which unselected stored keys are replaced by their list's mean value
+    under the approximate logits."""
     import bench
 
     dev = _cuda()
-    layer = bench.Layer(1, 4242, torch.device(dev))
+    layer = bench.Layer(cfg, 4242, torch.device(dev))
     layer.call.run(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    idx, G, H = layer.index, layer.G, layer.H
+    idx, G, H, B = layer.index, layer.G, layer.H, layer.B
     n = layer.n[0]
+    assert all(x == n for x in layer.n)
     k = ops.resolve_topk(n, bench.FRACTION, 0)
     qnorm, lut, ls = ops.lut_build(layer.q, idx, G)
     logits = ops.lut_scan(idx, G, qnorm, lut, ls, 1.0 / np.sqrt(128.0))       # [BH, G, n_cap] by key index
-    tidx = layer.ws.topk_idx.view(H, G, -1)[:, :, :k].to(torch.int64)
-    tval = layer.ws.topk_val.view(H, G, -1)[:, :, :k]
-    lg = logits.view(H, G, -1)[:, :, :n]
+    tidx = layer.ws.topk_idx.view(B * H, G, -1)[:, :, :k].to(torch.int64)
+    tval = layer.ws.topk_val.view(B * H, G, -1)[:, :, :k]
+    lg = logits.view(B * H, G, -1)[:, :, :n]
     assert torch.equal(torch.gather(lg, 2, tidx), tval)                        # the selected logits, bit for bit
     kth = torch.topk(lg, k, dim=2).values[:, :, -1:]
     assert bool((tval >= kth).all()) and bool((tidx.sort(dim=2).values.diff(dim=2) > 0).all())   # k distinct keys, none below the k-th
     assert layer.ws.rescans() == 0
-    # reference combination in fp64 on the device for one KV head
-    h = 3
-    kk, vv = ops.paged_gather_range(layer.kv, 0, 0, layer.lens[0])
+    # reference combination in fp64 on the device for one KV head of the last sequence
+    b, h = B - 1, 3
+    bh = b * H + h
+    kk, vv = ops.paged_gather_range(layer.kv, b, 0, layer.lens[b])
     K, V = kk[h].double(), vv[h].double()
-    q = layer.q[0, h * G : (h + 1) * G].double()
+    del kk, vv
+    q = layer.q[b, h * G : (h + 1) * G].double()
     sink = bench.SINK
     sel = torch.zeros(G, n, dtype=torch.bool, device=dev)
-    sel.scatter_(1, tidx[h], True)
+    sel.scatter_(1, tidx[bh], True)
     exact = (q @ K.T) / np.sqrt(128.0)
-    _, lists, _ = idx.by_key(h, n)
+    _, lists, _ = idx.by_key(bh, n)
     lists = lists.to(torch.int64) & 0xFFFF
-    m = torch.maximum(exact.max(dim=1).values, lg[h].double().max(dim=1).values)[:, None]
+    m = torch.maximum(exact.max(dim=1).values, lg[bh].double().max(dim=1).values)[:, None]
     w_exact = torch.exp(exact - m)
     w_exact[:, sink : sink + n] *= sel                                            # unselected stored keys leave the exact part
-    w_bg = torch.exp(lg[h].double() - m) * (~sel)
+    w_bg = torch.exp(lg[bh].double() - m) * (~sel)
     mass = torch.zeros(G, idx.num_lists, dtype=torch.float64, device=dev).index_add_(1, lists, w_bg)
-    num = w_exact @ V + mass @ idx.vbar[h].double()
+    num = w_exact @ V + mass @ idx.vbar[bh].double()
     den = w_exact.sum(dim=1, keepdim=True) + mass.sum(dim=1, keepdim=True)
     want = (num / den).float()
-    got = layer.out[0, h * G : (h + 1) * G].float()
+    got = layer.out[b, h * G : (h + 1) * G].float()
     err = (got - want).abs()
     assert bool((err <= 2e-3 + 2.0 ** -8 * want.abs()).all()), float(err.max())
 
