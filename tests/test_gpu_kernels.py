@@ -361,10 +361,12 @@ def test_hybrid_attend_paged_alone_matches_oracle():
         assert np.abs(o[b, h] - w).max() <= 2e-3, (b, h, np.abs(o[b, h] - w).max())
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4])
 def test_full_size_step_properties_at_the_benchmark_shapes(cfg):
     """At the full configuration sizes (cfg 1: context 32 768, one sequence; cfg 2, the headline:
-    context 131 072, batch 4; both 8 KV heads, GQA 4, bf16 paged) the oracle is too slow, so the
+    context 131 072, batch 4; cfg 3: 16 sequences of 16 384 to 65 536 tokens in shuffled blocks;
+    these with 8 KV heads, GQA 4; cfg 4: context 262 144, 4 KV heads, GQA 7; all bf16 paged) the
+    oracle is too slow, so the
     step is checked through properties: the selected set is exactly the k best of the logits
     pqhsa_lut_scan writes for the same tables, nothing was re-scanned, and the output equals a
     dense torch attention in which unselected stored keys are replaced by their list's mean value
@@ -376,35 +378,38 @@ def test_full_size_step_properties_at_the_benchmark_shapes(cfg):
     layer.call.run(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     idx, G, H, B = layer.index, layer.G, layer.H, layer.B
-    n = layer.n[0]
-    assert all(x == n for x in layer.n)
-    k = ops.resolve_topk(n, bench.FRACTION, 0)
     qnorm, lut, ls = ops.lut_build(layer.q, idx, G)
     logits = ops.lut_scan(idx, G, qnorm, lut, ls, 1.0 / np.sqrt(128.0))       # [BH, G, n_cap] by key index
-    tidx = layer.ws.topk_idx.view(B * H, G, -1)[:, :, :k].to(torch.int64)
-    tval = layer.ws.topk_val.view(B * H, G, -1)[:, :, :k]
-    lg = logits.view(B * H, G, -1)[:, :, :n]
-    assert torch.equal(torch.gather(lg, 2, tidx), tval)                        # the selected logits, bit for bit
-    kth = torch.topk(lg, k, dim=2).values[:, :, -1:]
-    assert bool((tval >= kth).all()) and bool((tidx.sort(dim=2).values.diff(dim=2) > 0).all())   # k distinct keys, none below the k-th
+    for b in range(B):                                                          # sequences differ in length at cfg 3
+        n = layer.n[b]
+        k = ops.resolve_topk(n, bench.FRACTION, 0)
+        rows = slice(b * H, (b + 1) * H)
+        tidx = layer.ws.topk_idx.view(B * H, G, -1)[rows, :, :k].to(torch.int64)
+        tval = layer.ws.topk_val.view(B * H, G, -1)[rows, :, :k]
+        lg = logits.view(B * H, G, -1)[rows, :, :n]
+        assert torch.equal(torch.gather(lg, 2, tidx), tval), b                  # the selected logits, bit for bit
+        kth = torch.topk(lg, k, dim=2).values[:, :, -1:]
+        assert bool((tval >= kth).all()), b                                     # none below the k-th best
+        assert bool((tidx.sort(dim=2).values.diff(dim=2) > 0).all()), b        # k distinct keys
     assert layer.ws.rescans() == 0
     # reference combination in fp64 on the device for one KV head of the last sequence
     b, h = B - 1, 3
     bh = b * H + h
+    sel_idx, lg_h = tidx[h], lg[h]                      # of sequence B - 1, the loop's last
     kk, vv = ops.paged_gather_range(layer.kv, b, 0, layer.lens[b])
     K, V = kk[h].double(), vv[h].double()
     del kk, vv
     q = layer.q[b, h * G : (h + 1) * G].double()
     sink = bench.SINK
     sel = torch.zeros(G, n, dtype=torch.bool, device=dev)
-    sel.scatter_(1, tidx[bh], True)
+    sel.scatter_(1, sel_idx, True)
     exact = (q @ K.T) / np.sqrt(128.0)
     _, lists, _ = idx.by_key(bh, n)
     lists = lists.to(torch.int64) & 0xFFFF
-    m = torch.maximum(exact.max(dim=1).values, lg[bh].double().max(dim=1).values)[:, None]
+    m = torch.maximum(exact.max(dim=1).values, lg_h.double().max(dim=1).values)[:, None]
     w_exact = torch.exp(exact - m)
     w_exact[:, sink : sink + n] *= sel                                            # unselected stored keys leave the exact part
-    w_bg = torch.exp(lg[bh].double() - m) * (~sel)
+    w_bg = torch.exp(lg_h.double() - m) * (~sel)
     mass = torch.zeros(G, idx.num_lists, dtype=torch.float64, device=dev).index_add_(1, lists, w_bg)
     num = w_exact @ V + mass @ idx.vbar[bh].double()
     den = w_exact.sum(dim=1, keepdim=True) + mass.sum(dim=1, keepdim=True)
