@@ -155,6 +155,7 @@ def test_topk_radix_on_logit_matrix_with_ties(stride):
 
 @pytest.mark.parametrize("case", [
     dict(lens=[2048], heads=1, groups=1, lists=64, dtype=torch.float32, fraction=0.02, kv="dense"),
+    dict(lens=[8192], heads=1, groups=1, lists=512, dtype=torch.float32, fraction=0.02, kv="dense"),   # cfg 0 in full
     dict(lens=[3000, 1800], heads=2, groups=4, lists=64, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
     dict(lens=[2500, 1900, 700], heads=2, groups=4, lists=32, dtype=torch.bfloat16, fraction=0.05, kv="4d"),
     dict(lens=[2200], heads=2, groups=7, lists=48, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
