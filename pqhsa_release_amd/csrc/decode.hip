@@ -65,7 +65,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
     c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
-    c.thr_key = reinterpret_cast<uint32_t *>(take(rows * 4));
+    c.thr_key = reinterpret_cast<uint32_t *>(take(rows * 8));  // thresholds, then the largest sampled keys
     c.k_row = reinterpret_cast<int32_t *>(take(rows * 4));
     c.ref_val = reinterpret_cast<float *>(take(rows * 4));
     c.ref_extra = reinterpret_cast<float *>(take(rows * 4));

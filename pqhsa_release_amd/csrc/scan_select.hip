@@ -724,6 +724,7 @@ struct SampleArgs {
     int topk;
     int k_cap;                 // room of the caller's top-k arrays: k never exceeds it
     uint32_t *thr_key;         // [BH * GP]
+    uint32_t *hi_key;          // [BH * GP] largest sampled key of the row (0: no estimate); may be NULL
     int32_t *k_row;
     float *ref_val;
     AppendFinish append;       // count != NULL: one more workgroup per stream completes the step's append
@@ -752,6 +753,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     if (g >= a.G) {
         if (tid == 0) {
             a.thr_key[row] = 0xffffffffu;
+            if (a.hi_key) a.hi_key[row] = 0u;
             a.k_row[row] = 0;
             a.ref_val[row] = -INFINITY;
         }
@@ -789,6 +791,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         // sample too small to say anything: every key is a candidate and no background sum is formed
         if (tid == 0) {
             a.thr_key[row] = 0u;
+            if (a.hi_key) a.hi_key[row] = 0u;
             a.k_row[row] = k;
             a.ref_val[row] = -INFINITY;
         }
@@ -836,6 +839,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     }
     if (tid == 0) {
         a.thr_key[row] = t;
+        if (a.hi_key) a.hi_key[row] = hi_key;
         a.k_row[row] = k;
         a.ref_val[row] = t == 0u ? -INFINITY : key_to_float(t);
     }
@@ -848,6 +852,10 @@ struct SelectArgs {
     int64_t emit_cap;
     uint32_t *emit_count;  // [rows]
     const int32_t *k_row;  // [rows]
+    // where the candidates' keys lie, as far as the threshold estimate knows: the threshold and the
+    // largest sampled key (NULL or 0: unknown); hints only, the selection is exact without them
+    const uint32_t *thr_key;
+    const uint32_t *hi_key;
     const int32_t *n_arr;
     int rows_per_n;
     int GP, G;
@@ -909,7 +917,8 @@ struct SelectOut {
 template <int R>
 __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
                                      int k, SelectOut out, uint32_t (*red)[kSelWaves],
-                                     uint32_t *wsum, SelScratch *ss, float *ref1_out) {
+                                     uint32_t *wsum, SelScratch *ss, float *ref1_out, uint32_t lo_hint = 0u,
+                                     uint32_t hi_hint = 0u) {
     const int tid = threadIdx.x;
     int step = 0;
     bool exact = false;
@@ -918,18 +927,30 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
     bool ties = false;
     bool searched = false;
     uint32_t lo_key = 0u, hi_key = 0u;
+    const bool hinted = lo_hint != 0u && hi_hint > lo_hint;
     if (k > 0) {
         // Candidates lie between the threshold and the row maximum.  Histogram them over 1024
         // equal ranges of that span, find the range that holds the k-th largest (one wave), and
         // rank the few candidates of that range against each other, equal keys by index: five
         // barriers where a bit-by-bit search takes one per bit.
-        block_min_max<0u>(key, wsum, lo_key, hi_key);
+        // With a hint of where the keys lie (the threshold they passed, the largest sampled key and
+        // an eighth of the span on top) the smallest and largest key need not be found first.
+        // Keys outside the hinted span fall into the first or last range, which keeps the ranges
+        // in key order, so the selection stays exact whatever the hint.
+        if (hinted) {
+            const uint32_t span = hi_hint - lo_hint;
+            lo_key = lo_hint;
+            hi_key = hi_hint + min(span >> 3, 0xffffffffu - hi_hint);
+        } else {
+            block_min_max<0u>(key, wsum, lo_key, hi_key);
+        }
         const uint32_t range = hi_key >= lo_key ? hi_key - lo_key : 0u;
         const int shift = range < (uint32_t)kSelBins ? 0 : (31 - __clz(range)) - 9;
         uint32_t bucket[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            bucket[r] = key[r] != 0u ? (key[r] - lo_key) >> shift : 0xffffffffu;
+            bucket[r] = key[r] == 0u ? 0xffffffffu
+                        : key[r] <= lo_key ? 0u : min((key[r] - lo_key) >> shift, (uint32_t)kSelBins - 1u);
             if (key[r] != 0u) atomicAdd(&ss->hist[bucket[r]], 1u);
         }
         if (tid == 0) ss->bin = 0xffffffffu;
@@ -939,6 +960,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         const uint32_t bin = ss->bin;
         const uint32_t crowd = bin < (uint32_t)kSelBins ? ss->hist[bin] : 0u;
         if (bin >= (uint32_t)kSelBins) {  // fewer than k candidates: all of them are selected
+            if (hinted) block_min_max<0u>(key, wsum, lo_key, hi_key);
             tkey = lo_key <= hi_key ? lo_key : 0u;
             searched = true;
         } else if (crowd <= (uint32_t)kSelBins) {
@@ -992,6 +1014,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         // more than 1024 candidates in the k-th key's range (many equal keys): bit-by-bit search
         // below the leading bits that all candidates share
         int bit0;
+        if (hinted) block_min_max<0u>(key, wsum, lo_key, hi_key);  // the search needs the true span
         const uint32_t t0 = shared_prefix(lo_key, hi_key, bit0);
         tkey = bisect_regs<R>(key, (uint32_t)k, 0u, red, step, exact, t0, bit0);
         if (!exact) {  // ties at the boundary: keep the lowest indices
@@ -1222,6 +1245,8 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
         }
     }
     uint32_t cnt = a.emit_count[row];
+    const uint32_t lo_hint = a.thr_key ? a.thr_key[row] : 0u;
+    const uint32_t hi_hint = a.hi_key ? a.hi_key[row] : 0u;
     float *mass_out = a.mass_extra ? a.mass_extra + (size_t)bh * a.L * a.GP + g : nullptr;
     const bool rescan = cnt < (uint32_t)k && a.codes;
 
@@ -1270,7 +1295,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             for (int r = 0; r < RS; ++r) {
                 if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, swhere[r] = 0u, slist[r] = 0u;
             }
-            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1);
+            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1, lo_hint, hi_hint);
             done = true;
         }
     }
@@ -1456,7 +1481,8 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
     sa.k_cap = select->k_cap;
     if (append) sa.append = *append;
-    sa.thr_key = thr_key; sa.k_row = k_row; sa.ref_val = ref_val;
+    uint32_t *hi_key = thr_key + (size_t)streams * GP;  // the threshold array is two rows long
+    sa.thr_key = thr_key; sa.hi_key = hi_key; sa.k_row = k_row; sa.ref_val = ref_val;
     int rc = launch_sample_thresh(sa, streams, stream);
     if (rc) return rc;
     profile_mark(kProfEmit, stream);
@@ -1476,7 +1502,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     // 3. exact selection among the candidates
     SelectArgs s = {};
     s.pairs = static_cast<uint2 *>(pairs); s.aux = aux; s.emit_cap = index->n_cap; s.emit_count = emit_count;
-    s.k_row = k_row; s.n_arr = index->n_idx; s.rows_per_n = index->kv_heads * GP; s.GP = GP; s.G = G;
+    s.k_row = k_row; s.thr_key = thr_key; s.hi_key = hi_key; s.n_arr = index->n_idx; s.rows_per_n = index->kv_heads * GP; s.GP = GP; s.G = G;
     s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = topk_cnt; s.k_cap = select->k_cap;
     s.mass = mass; s.mass_extra = mass_extra; s.ref_extra = ref_extra; s.L = index->num_lists;
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
