@@ -52,6 +52,7 @@ extern "C" {
 #define PQHSA_HEAD_DIM 128
 #define PQHSA_SUBSPACES 8
 #define PQHSA_HIST_BINS 2048
+#define PQHSA_STATIC_SCRATCH_MIB 32 /* scratch built into the library for pqhsa_decode_step_static */
 
 /*
  * Where the full-precision K/V rows live.  Row (b, h, pos) starts at element
@@ -239,6 +240,24 @@ int pqhsa_append_decode_step(const void *q, int32_t q_dtype, void *out, const pq
                              int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                              void *workspace, size_t workspace_bytes,
                              const int32_t *append_count, void *stream);
+
+/*
+ * pqhsa_decode_step for callers that cannot allocate or hand over a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The step's scratch (tables, candidate records, per-list sums, split partials)
+ * lives in a PQHSA_STATIC_SCRATCH_MIB MiB device array built into the library, one per GPU the
+ * library runs on, held until the process ends; the call allocates and frees nothing.  A shape
+ * whose pqhsa_decode_workspace_bytes exceeds pqhsa_static_scratch_bytes() is rejected with
+ * PQHSA_ENOSPC.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (different streams, different threads) race; each call clears what it needs to start at zero.
+ * topk_idx / topk_val / topk_cnt may be NULL.  Results are those of pqhsa_decode_step.
+ */
+size_t pqhsa_static_scratch_bytes(void);
+int pqhsa_decode_step_static(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                             const pqhsa_index *index, int32_t G, const int32_t *seq_lens,
+                             int32_t sink, int32_t n_max, int32_t full_max,
+                             const pqhsa_select *select, float scale, float eps, int32_t *topk_idx,
+                             float *topk_val, int32_t *topk_cnt, void *stream);
 
 /*
  * Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full since

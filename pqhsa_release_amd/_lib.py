@@ -92,6 +92,10 @@ SIGNATURES = {
     "pqhsa_decode_step": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32, c_void_p,
                                          c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_size_t, c_void_p]),
+    "pqhsa_static_scratch_bytes": (c_size_t, []),
+    "pqhsa_decode_step_static": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32, c_void_p,
+                                                c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p,
+                                                c_void_p, c_void_p, c_void_p]),
     "pqhsa_append_decode_step": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32, c_void_p,
                                                 c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p,
                                                 c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),

@@ -1,9 +1,20 @@
 // One decode-attention step of a layer: orchestration of the kernels on one stream, plus the
 // carve-up of the caller's workspace.
+#include <mutex>
+
 #include "common.h"
 #include "encode_row.h"
 
 namespace pqhsa {
+
+// Scratch of pqhsa_decode_step_static: one array per GPU the library runs on, held until the
+// process ends.  In host code the array's name is only a stand-in; the device address comes from
+// hipGetSymbolAddress, once per device, and is what kernels and host calls are given.
+constexpr size_t kStaticScratchBytes = (size_t)PQHSA_STATIC_SCRATCH_MIB << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void *scratch_ptr[kMaxDevices];
+static std::mutex scratch_mutex;
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps, float *qnorm,
                      float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words,
@@ -176,6 +187,46 @@ extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, cons
                                  size_t workspace_bytes, void *stream) {
     return decode_step_impl(q, q_dtype, out, kv, index, G, seq_lens, sink, n_max, full_max, select, scale, eps,
                             topk_idx, topk_val, topk_cnt, workspace, workspace_bytes, nullptr, stream);
+}
+
+// The static-scratch variant: no allocation of any kind on this path.
+extern "C" size_t pqhsa_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int pqhsa_decode_step_static(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
+                                        const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
+                                        int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale,
+                                        float eps, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
+                                        void *stream) {
+    PQHSA_REQUIRE(index && select, "decode_step_static: NULL argument");
+    const size_t need = pqhsa_decode_workspace_bytes(index->batch, index->kv_heads, G, index->n_cap, index->num_lists,
+                                                     select->k_cap);
+    if (need > kStaticScratchBytes) {
+        set_error("decode_step_static: this shape needs %zu bytes of scratch, the built-in array holds %zu "
+                  "(use pqhsa_decode_step with a caller workspace)", need, kStaticScratchBytes);
+        return PQHSA_ENOSPC;
+    }
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("decode_step_static: no current device (%s)", hipGetErrorString(e));
+        return PQHSA_ELAUNCH;
+    }
+    void *ptr;
+    {
+        std::lock_guard<std::mutex> lock(scratch_mutex);
+        if (!scratch_ptr[dev]) {
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p) {
+                set_error("decode_step_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+                return PQHSA_ELAUNCH;
+            }
+            scratch_ptr[dev] = p;
+        }
+        ptr = scratch_ptr[dev];
+    }
+    return decode_step_impl(q, q_dtype, out, kv, index, G, seq_lens, sink, n_max, full_max, select, scale, eps,
+                            topk_idx, topk_val, topk_cnt, ptr, kStaticScratchBytes, nullptr, stream);
 }
 
 extern "C" int pqhsa_append_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
