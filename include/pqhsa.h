@@ -263,15 +263,13 @@ int pqhsa_decode_step_static(const void *q, int32_t q_dtype, void *out, const pq
  * Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full since
  * the workspace was first used (a device-memory counter inside the workspace, for monitoring).
  */
-const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t B, int32_t H, int32_t G,
-                                            int64_t n_cap, int32_t num_lists, int32_t k_cap);
+const uint32_t *pqhsa_decode_rescan_counter(void *workspace);
 
 /*
  * Candidates the last step's scan kept per query row: u32 [B*H, padded_groups(G)] inside the
  * workspace (device memory, for monitoring the threshold estimate; rows of a padded group hold 0).
  */
-const uint32_t *pqhsa_decode_candidate_counts(void *workspace, int32_t B, int32_t H, int32_t G,
-                                              int64_t n_cap, int32_t num_lists, int32_t k_cap);
+const uint32_t *pqhsa_decode_candidate_counts(void *workspace);
 
 /*
  * Hybrid exact attention alone, given the selection and the per-list masses:

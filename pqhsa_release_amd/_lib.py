@@ -99,8 +99,8 @@ SIGNATURES = {
     "pqhsa_append_decode_step": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32, c_void_p,
                                                 c_int32, c_int32, c_int32, _P(Select), c_float, c_float, c_void_p,
                                                 c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
-    "pqhsa_decode_rescan_counter": (c_void_p, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
-    "pqhsa_decode_candidate_counts": (c_void_p, [c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
+    "pqhsa_decode_rescan_counter": (c_void_p, [c_void_p]),
+    "pqhsa_decode_candidate_counts": (c_void_p, [c_void_p]),
     "pqhsa_attend_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "pqhsa_hybrid_attend_paged": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32,
                                                  c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,

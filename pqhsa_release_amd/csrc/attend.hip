@@ -36,6 +36,7 @@ struct AttendArgs {
     const int32_t *topk_cnt;  // [BH*G]
     int64_t k_cap;
     int full_guess;           // sink + local rows the host expects per query row (for speculative index loads)
+    int chunk_cap;            // rows a workgroup's address list in LDS holds: full_max + k_cap are hard bounds
     float scale;
     int splits;
     float *partials;          // [BH*G, splits, kPartWidth]
@@ -132,7 +133,8 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int local_start = sink_end + n;
     const int F = sink_end + max(len - local_start, 0);
     const int k = min(a.topk_cnt[orow], (int)a.k_cap);  // never read past the row of the index array
-    const int total = F + k;
+    // (device-side lengths that ran ahead of the host's full_max are cut to what the launch was sized for)
+    const int total = min(F + k, a.chunk_cap * a.splits);
     const int chunk = (total + a.splits - 1) / a.splits;
     const int start = min(split * chunk, total);
     const int end = min(start + chunk, total);
@@ -451,6 +453,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     const int chunk = (rows_max + a.splits - 1) / a.splits;
     PQHSA_REQUIRE(chunk <= 4 * kMaxChunk, "attend: %d rows per query exceed what %d splits can take", rows_max,
                   kMaxSplits);
+    a.chunk_cap = chunk;
     const size_t lds = (size_t)chunk * sizeof(int64_t) + 16;
     dim3 grid(a.splits, a.G, BH);
 #define PQHSA_ATT(KD, QD)                                                                              \
@@ -486,17 +489,16 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
 
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
-                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
-                  const float *ref_val, const float *ref_extra, float scale, float *partials,
-                  const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream) {
+                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
+                  float *partials, const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
     a.topk_idx = topk_idx; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
     a.partials = partials;
     const int64_t L = index->num_lists;
-    a.mass0 = mass; a.mass1 = mass_extra; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
-    a.ref0 = ref_val; a.ref1 = ref_extra; a.ref_stride = GP;
+    a.mass0 = mass; a.mass1 = nullptr; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
+    a.ref0 = ref_val; a.ref1 = nullptr; a.ref_stride = GP;
     a.vbar = index->vbar; a.L = index->num_lists;
     a.n_commit_src = n_commit_src; a.n_commit_dst = n_commit_dst;
     return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream);

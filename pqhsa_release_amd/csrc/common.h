@@ -40,6 +40,28 @@ inline int padded_groups(int G) {
     return p;
 }
 
+// ---- per-workgroup phase clocks of a tuning build (-DPQHSA_TRACE); nothing in a normal build ----
+// PQHSA_TRACE_DECL(name) declares a buffer of [workgroup][8] wall-clock ticks (100 MHz) in the
+// translation unit and a C getter pqhsa_trace_read_<name>(host buffer); PQHSA_TRACE_MARK stores
+// the clock of thread 0 into slot `slot` of workgroup `wg`.
+#ifdef PQHSA_TRACE
+#define PQHSA_TRACE_SLOTS 8
+#define PQHSA_TRACE_WGS 8192
+#define PQHSA_TRACE_DECL(name)                                                                      \
+    static __device__ unsigned long long name[PQHSA_TRACE_WGS * PQHSA_TRACE_SLOTS];                 \
+    extern "C" int pqhsa_trace_read_##name(unsigned long long *host) {                             \
+        return hipMemcpyFromSymbol(host, HIP_SYMBOL(name), sizeof(name)) == hipSuccess ? 0 : -2;    \
+    }
+#define PQHSA_TRACE_MARK(name, wg, slot)                                                            \
+    do {                                                                                            \
+        if (threadIdx.x == 0 && (size_t)(wg) < PQHSA_TRACE_WGS)                                     \
+            name[(size_t)(wg) * PQHSA_TRACE_SLOTS + (slot)] = wall_clock64();                       \
+    } while (0)
+#else
+#define PQHSA_TRACE_DECL(name)
+#define PQHSA_TRACE_MARK(name, wg, slot) do {} while (0)
+#endif
+
 // ---- order-preserving float <-> uint32 keys --------------------------------------------
 // Larger float = larger key; -0 is folded onto +0 so that equal values have equal keys.
 __host__ __device__ inline uint32_t order_key(float f) {
@@ -89,6 +111,22 @@ __device__ inline int64_t row_offset(const KvView &v, int b, int h, int64_t pos)
         return phys * v.stride_block + row * v.stride_tok + (int64_t)h * v.stride_head;
     }
     return (int64_t)b * v.stride_seq + (int64_t)h * v.stride_head + pos * v.stride_tok;
+}
+
+// ---- the rows every query attends to in full: the sink prefix and the local window ----------------
+// A sequence of `len` cached tokens with n indexed keys: tokens [0, sink_end) and
+// [sink_end + n, len).  `full_max` is the caller's hard upper bound on their number (it sized the
+// row lists); rows beyond it are left out.
+struct FullRows {
+    int sink_end, local_start, count;
+    __device__ inline int64_t position(int i) const { return i < sink_end ? i : local_start + (i - sink_end); }
+};
+__device__ inline FullRows full_rows(int len, int n, int sink, int full_max) {
+    FullRows f;
+    f.sink_end = min(sink, len);
+    f.local_start = f.sink_end + n;
+    f.count = min(f.sink_end + max(len - f.local_start, 0), full_max);
+    return f;
 }
 
 // ---- typed 8-element row slices ---------------------------------------------------------

@@ -22,15 +22,14 @@ int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G
 int lut_list_blocks(int num_lists);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select,
-                       uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra,
-                       void *pairs, uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans,
+                       uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val,
+                       void *pairs, uint16_t *aux, float *mass, uint32_t *rescans,
                        int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                        const AppendFinish *append, hipStream_t stream);
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
-                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *mass_extra,
-                  const float *ref_val, const float *ref_extra, float scale, float *partials,
-                  const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream);
+                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
+                  float *partials, const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream);
 int emit_tile_keys_for(int64_t n_cap, int streams);
 size_t attend_partials_bytes(int rows);
 
@@ -43,7 +42,7 @@ struct Carve {
     size_t zero_words;
     uint32_t *thr_key;
     int32_t *k_row;
-    float *ref_val, *ref_extra, *mass_extra;
+    float *ref_val;
     void *pairs;
     uint16_t *aux;
     int32_t *topk_idx;
@@ -68,19 +67,17 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
         off += al(bytes);
         return p;
     };
-    c.qnorm = reinterpret_cast<float *>(take(rows * 4));
-    c.lut = reinterpret_cast<float *>(take(rows * kM * kCodes * 4));
-    c.ls = reinterpret_cast<float *>(take(rows * L * 4));
+    c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
     const size_t z0 = off;  // everything from here to zero_words is cleared at the start of a step
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
-    c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
+    c.qnorm = reinterpret_cast<float *>(take(rows * 4));
+    c.lut = reinterpret_cast<float *>(take(rows * kM * kCodes * 4));
+    c.ls = reinterpret_cast<float *>(take(rows * L * 4));
     c.thr_key = reinterpret_cast<uint32_t *>(take(rows * 8));  // thresholds, then the largest sampled keys
     c.k_row = reinterpret_cast<int32_t *>(take(rows * 4));
     c.ref_val = reinterpret_cast<float *>(take(rows * 4));
-    c.ref_extra = reinterpret_cast<float *>(take(rows * 4));
-    c.mass_extra = reinterpret_cast<float *>(take(rows * L * 4));
     c.pairs = take(rows * (size_t)n_cap * 8);
     c.aux = reinterpret_cast<uint16_t *>(take(rows * (size_t)n_cap * 2));
     c.topk_idx = reinterpret_cast<int32_t *>(take(BH * G * (size_t)k_cap * 4));
@@ -104,16 +101,14 @@ extern "C" size_t pqhsa_decode_workspace_bytes(int32_t B, int32_t H, int32_t G, 
 
 // Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full, since
 // the workspace was created (device counter; reading it synchronises nothing by itself).
-extern "C" const uint32_t *pqhsa_decode_rescan_counter(void *workspace, int32_t B, int32_t H, int32_t G,
-                                                       int64_t n_cap, int32_t num_lists, int32_t k_cap) {
+extern "C" const uint32_t *pqhsa_decode_rescan_counter(void *workspace) {
     char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
-    return carve(base, B, H, G, n_cap, num_lists, k_cap).rescans;
+    return reinterpret_cast<const uint32_t *>(base);  // the first block of the carve-up
 }
 
-extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace, int32_t B, int32_t H, int32_t G,
-                                                         int64_t n_cap, int32_t num_lists, int32_t k_cap) {
+extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace) {
     char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
-    return carve(base, B, H, G, n_cap, num_lists, k_cap).emit_count;
+    return reinterpret_cast<const uint32_t *>(base + 256);  // the second block of the carve-up
 }
 
 static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
@@ -171,11 +166,11 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     if (rc) return rc;
     profile_mark(kProfSample, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
-                            c.k_row, c.ref_val, c.ref_extra, c.pairs, c.aux, c.mass, c.mass_extra, c.rescans,
+                            c.k_row, c.ref_val, c.pairs, c.aux, c.mass, c.rescans,
                             c.tile_keys, topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
-                         topk_cnt, select->k_cap, c.mass, c.mass_extra, c.ref_val, c.ref_extra, scale, c.partials,
+                         topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials,
                          append_count ? c.n_after : nullptr,
                          append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
 }

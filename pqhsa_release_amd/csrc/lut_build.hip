@@ -17,6 +17,7 @@ namespace pqhsa {
 constexpr int kLutThreads = 256;  // at least; one wave per padded query row when the group is wider than 4
 constexpr int kListsPerBlock = 64;
 constexpr int kMaxG = 16;
+PQHSA_TRACE_DECL(trace_lut)
 
 int lut_list_blocks(int num_lists);
 
@@ -36,6 +37,8 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
     const int nthr = blockDim.x;
     const int bh = blockIdx.y;
     const int b = bh / H, h = bh % H;
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
+    PQHSA_TRACE_MARK(trace_lut, trace_wg, 0);
 
     // list blocks: their 64 x 128 centroid tile (2048 float4, 8 per thread) is requested before
     // anything else, so the loads are all in flight while the query rows are normalised
@@ -75,6 +78,7 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         qh[g][d] = load1<DT>(qrow0 + (size_t)g * kD * esz, d);
     }
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_lut, trace_wg, 1);
     if (tid < G) {
         float ss = 0.0f;
         for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(qh[tid][d], qh[tid][d], ss);
@@ -94,6 +98,7 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
     }
     if (appending && tid < kD) kx[tid] = kx[tid] / kn_s;
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_lut, trace_wg, 2);
 
     if (blockIdx.x == 0) {
         if (tid < Gp) qnorm[(size_t)bh * Gp + tid] = tid < G ? qn[tid] : 0.0f;
@@ -111,6 +116,8 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
             }
             out[e] = acc;
         }
+        PQHSA_TRACE_MARK(trace_lut, trace_wg, 3);
+        PQHSA_TRACE_MARK(trace_lut, trace_wg, 4);
         return;
     }
 
@@ -122,6 +129,7 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
     }
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_lut, trace_wg, 3);
     const int lane = tid % kListsPerBlock;
     const int wave = tid / kListsPerBlock;
     float *out = list_scores + ((size_t)bh * L + l0) * Gp;
@@ -150,6 +158,7 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         key = wave_min_u64(key, kWave);
         if (lane == 0) nearest[(size_t)bh * (gridDim.x - 1) + (blockIdx.x - 1)] = key;
     }
+    PQHSA_TRACE_MARK(trace_lut, trace_wg, 4);
 }
 
 int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G, float eps,

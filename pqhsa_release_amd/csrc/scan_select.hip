@@ -37,6 +37,9 @@ constexpr int kKeysPerIter = kScanThreads * kKeysPerThread;
 constexpr int kWaveKeys = kWave * kKeysPerThread;
 
 enum { kWrite = 0, kHist = 1, kEmit = 2 };
+PQHSA_TRACE_DECL(trace_scan)
+PQHSA_TRACE_DECL(trace_sample)
+PQHSA_TRACE_DECL(trace_select)
 enum { kIndex = 0, kLogits = 1 };
 
 struct ScanArgs {
@@ -139,6 +142,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int n = a.n_arr[bh / a.n_div];
     const int tile0 = tile * a.tile_keys;
     if (tile0 >= n) return;
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
+    PQHSA_TRACE_MARK(trace_scan, trace_wg, 0);
     const int tile_end = min(n, tile0 + a.tile_keys);
     const int L = a.L;
 
@@ -262,6 +267,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         }
     }
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_scan, trace_wg, 1);
 
     // every lane of a wave runs the same number of iterations (the wave's first key decides)
     for (int i0 = tile0 + tid * kKeysPerThread; i0 - lane * kKeysPerThread < tile_end; i0 += kKeysPerIter) {
@@ -470,6 +476,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         }
     }
 
+    PQHSA_TRACE_MARK(trace_scan, trace_wg, 2);
     if constexpr (MODE == kHist) {
         __syncthreads();
         uint32_t *dst = a.hist + (size_t)bh * GP * kHistBins;
@@ -518,6 +525,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         }
     }
+    PQHSA_TRACE_MARK(trace_scan, trace_wg, 3);
 }
 
 // ---- wave-level search of a histogram from its top bin ----------------------------------
@@ -750,6 +758,8 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         return;
     }
     const size_t row = (size_t)bh * a.GP + g;
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 0);
     if (g >= a.G) {
         if (tid == 0) {
             a.thr_key[row] = 0xffffffffu;
@@ -800,6 +810,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     const uint32_t want = (uint32_t)want_d;
     for (int i = tid; i < kSelBins; i += kSelThreads) hist[i] = 0u;
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 1);
     uint32_t key[R];
 #pragma unroll
     for (int r0 = 0; r0 < R; r0 += kBatch) {
@@ -817,7 +828,9 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     // lower edge of the range that holds the want-th largest (one wave finds it).  If the window
     // holds fewer than want keys, or that range is crowded, the bit-by-bit search takes over.
     uint32_t lo_key, hi_key;
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 2);
     block_min_max<0u>(key, wsum, lo_key, hi_key);
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 3);
     constexpr uint32_t kWindow = 1u << 25;
     const uint32_t wbase = hi_key > kWindow ? max(hi_key - kWindow, lo_key) : lo_key;
     const uint32_t range = hi_key >= wbase ? hi_key - wbase : 0u;
@@ -837,6 +850,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         bool exact;
         t = bisect_regs<R>(key, want, want / 8u, red, step, exact);
     }
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 4);
     if (tid == 0) {
         a.thr_key[row] = t;
         if (a.hi_key) a.hi_key[row] = hi_key;
@@ -865,8 +879,7 @@ struct SelectArgs {
     int64_t k_cap;
     // background mass of the candidates that lose the selection (optional)
     float *mass;           // [BH, L, GP]: zeroed for a row that is re-scanned in full
-    float *mass_extra;     // [BH, L, GP]
-    float *ref_extra;      // [rows] reference logit of mass_extra
+    float *ref_val;        // [rows] reference logit of mass: read, and replaced when the row's sums start over
     int L;
     // the index: retrieval-local index of every stored position, and what a full re-scan needs
     const int32_t *pos;    // [BH, n_cap] (NULL: a candidate's position is its index)
@@ -900,7 +913,7 @@ struct SelectOut {
     float *out_val;
     uint32_t k_cap;
     float *mx;               // LDS [L] (NULL: no background)
-    float ref1;
+    float ref1;              // reference of the losers' weights: the k-th logit
     __device__ inline void winner(uint32_t at, uint32_t key, uint32_t where) const {
         if (at < k_cap) {
             out_idx[at] = (int32_t)where;
@@ -955,6 +968,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         }
         if (tid == 0) ss->bin = 0xffffffffu;
         __syncthreads();
+        PQHSA_TRACE_MARK(trace_select, blockIdx.x + (size_t)gridDim.x * blockIdx.y, 2);
         if (tid < kWave) find_from_top_1024(ss->hist, (uint32_t)k, &ss->bin, &ss->above);
         __syncthreads();
         const uint32_t bin = ss->bin;
@@ -1054,10 +1068,12 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
     }
     out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
     *ref1_out = out.ref1;
+    PQHSA_TRACE_MARK(trace_select, blockIdx.x + (size_t)gridDim.x * blockIdx.y, 3);
     uint32_t mine = 0;
 #pragma unroll
     for (int r = 0; r < R; ++r) mine += (k > 0 && key[r] >= tkey) ? 1u : 0u;
     uint32_t at = block_exclusive_u32(mine, wsum);
+    PQHSA_TRACE_MARK(trace_select, blockIdx.x + (size_t)gridDim.x * blockIdx.y, 4);
     const int lane = tid & (kWave - 1);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -1227,6 +1243,8 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     const int bh = blockIdx.y;
     const size_t row = (size_t)bh * a.GP + g;
     const size_t orow = (size_t)bh * a.G + g;
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
+    PQHSA_TRACE_MARK(trace_select, trace_wg, 0);
     const int n = a.n_arr[row / a.rows_per_n];
     const int k = a.k_row[row];
     uint2 *pairs = a.pairs + row * a.emit_cap;
@@ -1247,19 +1265,19 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     uint32_t cnt = a.emit_count[row];
     const uint32_t lo_hint = a.thr_key ? a.thr_key[row] : 0u;
     const uint32_t hi_hint = a.hi_key ? a.hi_key[row] : 0u;
-    float *mass_out = a.mass_extra ? a.mass_extra + (size_t)bh * a.L * a.GP + g : nullptr;
+    // losers' weights join the scan's per-list sums of the row (same reference), unless those have to start over
+    float *mass_out = a.mass ? a.mass + (size_t)bh * a.L * a.GP + g : nullptr;
+    const float ref0 = mass_out ? a.ref_val[row] : -INFINITY;
     const bool rescan = cnt < (uint32_t)k && a.codes;
 
     if (rescan) {
         // The estimate kept too few keys: score the whole row again and treat every key as a
-        // candidate.  The row's background sums start over (all of them land in mass_extra).
+        // candidate.  The row's background sums start over, relative to the k-th logit.
         if (tid == 0 && a.rescans) atomicAdd(a.rescans, 1u);
         float *lut_s = reinterpret_cast<float *>(smem);
         float *ls_s = lut_s + kM * kCodes;
         for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
         for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
-        if (a.mass)
-            for (int l = tid; l < a.L; l += kSelThreads) a.mass[((size_t)bh * a.L + l) * a.GP + g] = 0.0f;
         const float qn = a.qnorm[row];
         __syncthreads();
         const size_t base = (size_t)bh * a.n_cap;
@@ -1281,6 +1299,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     for (int i = tid; i < kSelBins; i += kSelThreads) ss.hist[i] = 0u;
     if (tid == 0) ss.cont_count = 0u;
     __syncthreads();
+    PQHSA_TRACE_MARK(trace_select, trace_wg, 1);
     SelectOut out;
     out.out_idx = a.topk_idx + orow * a.k_cap;
     out.out_val = a.topk_val ? a.topk_val + orow * a.k_cap : nullptr;
@@ -1309,12 +1328,23 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
         }
     }
+    PQHSA_TRACE_MARK(trace_select, trace_wg, 5);
     __syncthreads();
     if (mass_out) {
-        for (int l = tid; l < a.L; l += kSelThreads) mass_out[(size_t)l * a.GP] = mx[l];
-        if (tid == 0) a.ref_extra[row] = ref1;
+        // The row's sums move to the k-th logit as their reference (it is at or above the scan's, so
+        // the factor is at most 1); a row without usable sums from the scan starts from the losers alone.
+        const bool fresh = rescan || !__builtin_isfinite(ref0);
+        if (fresh || __builtin_isfinite(ref1)) {
+            const float f = fresh ? 0.0f : __expf(ref0 - ref1);
+            for (int l = tid; l < a.L; l += kSelThreads) {
+                float *m = mass_out + (size_t)l * a.GP;
+                *m = fresh ? mx[l] : __builtin_fmaf(*m, f, mx[l]);
+            }
+            if (tid == 0) a.ref_val[row] = ref1;
+        }
     }
     if (tid == 0) a.topk_cnt[orow] = max(k, 0);
+    PQHSA_TRACE_MARK(trace_select, trace_wg, 6);
 }
 
 __global__ void fill_zero_kernel(uint32_t *p, size_t words) {
@@ -1468,8 +1498,8 @@ int emit_tile_keys_for(int64_t n_cap, int streams) {
 // sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
-                       uint32_t *thr_key, int32_t *k_row, float *ref_val, float *ref_extra, void *pairs,
-                       uint16_t *aux, float *mass, float *mass_extra, uint32_t *rescans, int emit_tile_keys,
+                       uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
+                       uint16_t *aux, float *mass, uint32_t *rescans, int emit_tile_keys,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
                        hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
@@ -1504,7 +1534,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.pairs = static_cast<uint2 *>(pairs); s.aux = aux; s.emit_cap = index->n_cap; s.emit_count = emit_count;
     s.k_row = k_row; s.thr_key = thr_key; s.hi_key = hi_key; s.n_arr = index->n_idx; s.rows_per_n = index->kv_heads * GP; s.GP = GP; s.G = G;
     s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = topk_cnt; s.k_cap = select->k_cap;
-    s.mass = mass; s.mass_extra = mass_extra; s.ref_extra = ref_extra; s.L = index->num_lists;
+    s.mass = mass; s.ref_val = ref_val; s.L = index->num_lists;
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
     s.n_cap = index->n_cap; s.qnorm = qnorm; s.lut = lut; s.list_scores = list_scores; s.scale = scale;
     s.rescans = rescans;

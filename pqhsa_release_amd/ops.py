@@ -379,28 +379,27 @@ class DecodeWorkspace:
         lib = _lib.load()
         self.k_cap = max(int(k_cap), 1)
         self.groups = groups
-        self.bytes = lib.pqhsa_decode_workspace_bytes(index.batch, index.kv_heads, groups, index.n_cap,
-                                                      index.num_lists, self.k_cap)
-        self.buf = torch.empty(self.bytes, dtype=torch.uint8, device=index.device)
+        self._shape = (index.batch, index.kv_heads, groups, index.n_cap, index.num_lists, self.k_cap)
+        self.bytes = lib.pqhsa_decode_workspace_bytes(*self._shape)
+        self.buf = torch.zeros(self.bytes, dtype=torch.uint8, device=index.device)
         rows = index.batch * index.kv_heads * groups
         self.topk_idx = torch.full((rows, self.k_cap), -1, dtype=torch.int32, device=index.device)
         self.topk_val = torch.zeros(rows, self.k_cap, dtype=torch.float32, device=index.device)
         self.topk_cnt = torch.zeros(rows, dtype=torch.int32, device=index.device)
-        self.buf.zero_()
-        self._shape = (index.batch, index.kv_heads, groups, index.n_cap, index.num_lists, self.k_cap)
+
+    def _head_offset(self, getter) -> int:
+        return getter(self.buf.data_ptr()) - self.buf.data_ptr()
 
     def rescans(self) -> int:
         """Rows re-scanned in full because the sampled threshold kept fewer than k candidates
         (synchronises: reads a device counter)."""
-        ptr = _lib.load().pqhsa_decode_rescan_counter(self.buf.data_ptr(), *self._shape)
-        off = ptr - self.buf.data_ptr()
+        off = self._head_offset(_lib.load().pqhsa_decode_rescan_counter)
         return int(self.buf[off : off + 4].view(torch.int32).item())
 
     def candidate_counts(self) -> torch.Tensor:
         """Candidates the last step's scan kept per query row, int32 [B*H, padded groups]
         (a view of device memory inside the workspace; rows of a padded group hold 0)."""
-        ptr = _lib.load().pqhsa_decode_candidate_counts(self.buf.data_ptr(), *self._shape)
-        off = ptr - self.buf.data_ptr()
+        off = self._head_offset(_lib.load().pqhsa_decode_candidate_counts)
         b, h, g = self._shape[:3]
         gp = _lib.load().pqhsa_padded_groups(g)
         return self.buf[off : off + 4 * b * h * gp].view(torch.int32).view(b * h, gp)
@@ -470,12 +469,12 @@ class DecodeCall:
         self._keep = (q, out, kv, index, seq_lens, workspace, append_count)
         self.n_max = index.n_max if n_max is None else int(n_max)
         self.full_max = int(full_max)
+        self._workspace = workspace
         self._head = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups)
         self._seq_lens = seq_lens.data_ptr()
         self._sink = int(sink)
         self._tail = (ctypes.byref(self._sel), float(scale), eps, workspace.topk_idx.data_ptr(),
-                      workspace.topk_val.data_ptr(), workspace.topk_cnt.data_ptr(), workspace.buf.data_ptr(),
-                      workspace.bytes)
+                      workspace.topk_val.data_ptr(), workspace.topk_cnt.data_ptr())
         self.out = out
 
     def run(self, stream: int | None = None, seq_lens_ptr: int | None = None) -> None:
@@ -483,8 +482,10 @@ class DecodeCall:
         step: ``n_max`` must already count the appended key, and the caller records the append in
         the index's host-side mirror afterwards (``DeviceIndex.note_appended``).  ``seq_lens_ptr``
         overrides the sequence-length array for this step (an int32 [B] device pointer)."""
+        ws = self._workspace
         rc = self._fn(*self._head, self._seq_lens if seq_lens_ptr is None else seq_lens_ptr, self._sink, self.n_max,
-                      self.full_max, *self._tail, *self._append, _stream() if stream is None else stream)
+                      self.full_max, *self._tail, ws.buf.data_ptr(), ws.bytes, *self._append,
+                      _stream() if stream is None else stream)
         if rc:
             _lib.check(rc, "pqhsa_decode_step")
 
