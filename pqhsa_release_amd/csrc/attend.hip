@@ -11,7 +11,6 @@
 // attend_reduce_kernel: grid (G, BH).  Folds the split partials under the final row maximum,
 // rescales the two background parts from their reference logits, and normalises.
 #include <cfloat>
-#include <cstdlib>
 
 #include "common.h"
 
@@ -431,7 +430,7 @@ __global__ __launch_bounds__(kAttThreads) void subtract_selected_kernel(const fl
 }
 
 int pick_splits(int streams_rows, int rows_max) {
-    static const int target = getenv("PQHSA_ATT_WGS") ? atoi(getenv("PQHSA_ATT_WGS")) : 1024;
+    constexpr int target = 1024;  // workgroups of the launch: four per compute unit
     int s = (target + streams_rows - 1) / (streams_rows > 0 ? streams_rows : 1);
     // chunks of at most 384 rows: short enough that a ragged batch (rows of very different
     // lengths) still spreads evenly over the compute units
@@ -442,13 +441,19 @@ int pick_splits(int streams_rows, int rows_max) {
     return s;
 }
 
-size_t attend_partials_bytes(int rows) { return (size_t)rows * kMaxSplits * kPartWidth * sizeof(float); }
+// Splits the partials area of a workspace has room for: what a step with up to 4096 sink and
+// window rows on top of its k_cap selected keys takes (a step with more simply gets longer chunks).
+static int splits_room(int rows, int k_cap) { return pick_splits(rows, (k_cap > 0 ? k_cap : 0) + 4096); }
+
+size_t attend_partials_bytes(int rows, int k_cap) {
+    return (size_t)rows * splits_room(rows, k_cap) * kPartWidth * sizeof(float);
+}
 
 int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max, bool mark, hipStream_t stream) {
     if (BH == 0) return PQHSA_OK;
     PQHSA_REQUIRE(a.G >= 1 && a.G <= 16, "attend: G=%d outside [1, 16]", a.G);
     PQHSA_REQUIRE(a.L <= 4096, "attend: num_lists=%d too large", a.L);
-    a.splits = pick_splits(BH * a.G, rows_max);
+    a.splits = min(pick_splits(BH * a.G, rows_max), splits_room(BH * a.G, (int)a.k_cap));
     a.full_guess = rows_max > (int)a.k_cap ? rows_max - (int)a.k_cap : 0;
     const int chunk = (rows_max + a.splits - 1) / a.splits;
     PQHSA_REQUIRE(chunk <= 4 * kMaxChunk, "attend: %d rows per query exceed what %d splits can take", rows_max,
@@ -509,7 +514,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
 using namespace pqhsa;
 
 extern "C" size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t num_lists) {
-    return attend_partials_bytes(B * H * G) + (size_t)B * H * G * num_lists * sizeof(float) + 512;
+    return attend_partials_bytes(B * H * G, 1 << 20) + (size_t)B * H * G * num_lists * sizeof(float) + 512;
 }
 
 extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
@@ -531,7 +536,7 @@ extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *o
     if (BH == 0) return PQHSA_OK;
     char *w = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
     float *partials = reinterpret_cast<float *>(w);
-    float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G));
+    float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G, 1 << 20));
     hipLaunchKernelGGL(subtract_selected_kernel, dim3(G, BH), dim3(kAttThreads), (size_t)L * sizeof(float), stream,
                        list_mass, row_max, topk_idx, topk_val, topk_cnt, (int64_t)k_cap, key_lists, key_list_stride, G,
                        L, mass_adj);

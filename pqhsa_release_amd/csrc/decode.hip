@@ -23,15 +23,14 @@ int lut_list_blocks(int num_lists);
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select,
                        uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val,
-                       void *pairs, uint16_t *aux, float *mass, uint32_t *rescans,
-                       int emit_tile_keys, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
+                       void *pairs, uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
+                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                        const AppendFinish *append, hipStream_t stream);
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
                   float *partials, const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream);
-int emit_tile_keys_for(int64_t n_cap, int streams);
-size_t attend_partials_bytes(int rows);
+size_t attend_partials_bytes(int rows, int k_cap);
 
 static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -45,6 +44,7 @@ struct Carve {
     float *ref_val;
     void *pairs;
     uint16_t *aux;
+    int64_t emit_cap;  // candidate records per query row
     int32_t *topk_idx;
     float *topk_val;
     int32_t *topk_cnt;
@@ -52,7 +52,6 @@ struct Carve {
     int32_t *n_after;  // [B] keys per sequence after this step's append
     unsigned long long *nearest;  // [BH, list blocks] nearest centroid to the appended key, per list block
     size_t total;
-    int tile_keys;
 };
 
 static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_cap) {
@@ -60,7 +59,6 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     const size_t BH = (size_t)B * H;
     const size_t GP = padded_groups(G);
     const size_t rows = BH * GP;
-    c.tile_keys = emit_tile_keys_for(n_cap, (int)BH);
     size_t off = 0;
     auto take = [&](size_t bytes) {
         char *p = base + off;
@@ -78,12 +76,18 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.thr_key = reinterpret_cast<uint32_t *>(take(rows * 8));  // thresholds, then the largest sampled keys
     c.k_row = reinterpret_cast<int32_t *>(take(rows * 4));
     c.ref_val = reinterpret_cast<float *>(take(rows * 4));
-    c.pairs = take(rows * (size_t)n_cap * 8);
-    c.aux = reinterpret_cast<uint16_t *>(take(rows * (size_t)n_cap * 2));
+    // Candidate records: the threshold estimate aims at about 2.2 k candidates per row; room for
+    // 3 k and a margin (never more than the row has keys).  A row that outgrows it is selected
+    // from a full pass over its keys instead, like a row whose estimate kept too few.
+    c.emit_cap = 3 * (int64_t)k_cap + 2048;
+    if (c.emit_cap > n_cap) c.emit_cap = n_cap;
+    c.emit_cap = (c.emit_cap + 7) / 8 * 8;
+    c.pairs = take(rows * (size_t)c.emit_cap * 8);
+    c.aux = reinterpret_cast<uint16_t *>(take(rows * (size_t)c.emit_cap * 2));
     c.topk_idx = reinterpret_cast<int32_t *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_val = reinterpret_cast<float *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_cnt = reinterpret_cast<int32_t *>(take(BH * G * 4));
-    c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G))));
+    c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G), k_cap)));
     c.n_after = reinterpret_cast<int32_t *>(take((size_t)B * 4));
     c.nearest = reinterpret_cast<unsigned long long *>(take(BH * (size_t)lut_list_blocks(L) * 8));
     c.total = off;
@@ -166,8 +170,8 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     if (rc) return rc;
     profile_mark(kProfSample, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
-                            c.k_row, c.ref_val, c.pairs, c.aux, c.mass, c.rescans,
-                            c.tile_keys, topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
+                            c.k_row, c.ref_val, c.pairs, c.aux, c.emit_cap, c.mass, c.rescans,
+                            topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials,

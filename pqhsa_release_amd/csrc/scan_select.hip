@@ -23,103 +23,14 @@
 // (one barrier per bit) for inputs the histogram does not resolve: a crowded range, or a wanted
 // rank outside the sampled window.  A row whose estimate kept fewer than k candidates is
 // re-scanned in full by its select workgroup, so the result is always the exact top-k.
-#include <cstdlib>
-
 #include "common.h"
 #include "encode_row.h"
+#include "scan_common.h"
 
 namespace pqhsa {
 
-constexpr int kScanThreads = 256;
-constexpr int kScanWaves = kScanThreads / kWave;
-constexpr int kKeysPerThread = 4;
-constexpr int kKeysPerIter = kScanThreads * kKeysPerThread;
-constexpr int kWaveKeys = kWave * kKeysPerThread;
-
-enum { kWrite = 0, kHist = 1, kEmit = 2 };
-PQHSA_TRACE_DECL(trace_scan)
 PQHSA_TRACE_DECL(trace_sample)
 PQHSA_TRACE_DECL(trace_select)
-enum { kIndex = 0, kLogits = 1 };
-
-struct ScanArgs {
-    // index source
-    const uint32_t *codes;
-    const uint16_t *list_ids;
-    const float *norms;
-    const int32_t *pos;        // retrieval-local index per stored position (NULL: identity)
-    int64_t n_cap;             // row stride of the arrays above
-    const float *qnorm;        // [BH, GP]
-    const float *lut;          // [BH, 128, GP]
-    const float *list_scores;  // [BH, L, GP]
-    float scale;
-    int L;
-    // logit-matrix source
-    const float *logits_in;
-    int64_t logits_in_stride;
-    // shape
-    const int32_t *n_arr;       // n = n_arr[stream / n_div]
-    int n_div;
-    int G;
-    int tile_keys;
-    // kWrite
-    float *logits_out;
-    int64_t logits_out_stride;
-    int by_xcd;  // streams are dealt to the 8 XCDs (stream count a multiple of 8): see scan_kernel
-    // kHist
-    uint32_t *hist;  // [rows, 2048]
-    // kEmit
-    const uint32_t *thr_key;  // [rows] keys at or above it are candidates
-    const float *ref_val;     // [rows] reference logit of the background sums
-    uint32_t *emit_count;     // [rows]
-    uint2 *emit_pairs;        // [rows, emit_cap] (key, retrieval-local index)
-    uint16_t *emit_aux;       // [rows, emit_cap] list id of the candidate (NULL: none)
-    int64_t emit_cap;
-    float *mass;              // [BH, L, GP] accumulated with atomics (NULL: none)
-    int stage_cap;            // candidates one wave stages in LDS per row before it writes straight to memory
-};
-
-template <int GP>
-__device__ inline void lds_vec(const float *p, float (&v)[GP]) {
-    if constexpr (GP >= 4) {
-#pragma unroll
-        for (int i = 0; i < GP / 4; ++i) {
-            float4 t = reinterpret_cast<const float4 *>(p)[i];
-            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
-        }
-    } else if constexpr (GP == 2) {
-        float2 t = *reinterpret_cast<const float2 *>(p);
-        v[0] = t.x; v[1] = t.y;
-    } else {
-        v[0] = p[0];
-    }
-}
-
-// PQ table entry (m * 16 + code) of every query row.  In LDS the table is kept as one sub-table per
-// pair of query rows, [pair][128 entries][2]: the 16 codewords of a subspace then fill exactly one
-// 128-byte row of the 32 LDS banks, so the 64 lanes of a look-up (16 distinct addresses at most)
-// never meet in a bank, whereas 16-byte entries spread a subspace over two rows that share banks.
-template <int GP>
-__device__ inline void lut_entry(const float *lut_s, uint32_t entry, float (&v)[GP]) {
-    if constexpr (GP >= 2) {
-#pragma unroll
-        for (int p = 0; p < GP / 2; ++p) {
-            const float2 t = reinterpret_cast<const float2 *>(lut_s)[p * (kM * kCodes) + entry];
-            v[2 * p] = t.x; v[2 * p + 1] = t.y;
-        }
-    } else {
-        v[0] = lut_s[entry];
-    }
-}
-
-// logit of one stored key for one query row, in the fixed summation order of the CPU oracle
-__device__ inline float score_one(const float *lut_col, const float *ls_col, uint32_t code, uint32_t lid, float qn,
-                                  float kn, float scale) {
-    float s = 0.0f;
-#pragma unroll
-    for (int m = 0; m < kM; ++m) s = s + lut_col[m * kCodes + ((code >> (4 * m)) & 15u)];
-    return (((s + ls_col[lid]) * qn) * kn) * scale;
-}
 
 template <int GP, int MODE, int SRC>
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
@@ -142,8 +53,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
     const int n = a.n_arr[bh / a.n_div];
     const int tile0 = tile * a.tile_keys;
     if (tile0 >= n) return;
-    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
-    PQHSA_TRACE_MARK(trace_scan, trace_wg, 0);
     const int tile_end = min(n, tile0 + a.tile_keys);
     const int L = a.L;
 
@@ -267,7 +176,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
         }
     }
     __syncthreads();
-    PQHSA_TRACE_MARK(trace_scan, trace_wg, 1);
 
     // every lane of a wave runs the same number of iterations (the wave's first key decides)
     for (int i0 = tile0 + tid * kKeysPerThread; i0 - lane * kKeysPerThread < tile_end; i0 += kKeysPerIter) {
@@ -475,8 +383,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         }
     }
-
-    PQHSA_TRACE_MARK(trace_scan, trace_wg, 2);
     if constexpr (MODE == kHist) {
         __syncthreads();
         uint32_t *dst = a.hist + (size_t)bh * GP * kHistBins;
@@ -525,7 +431,6 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
             }
         }
     }
-    PQHSA_TRACE_MARK(trace_scan, trace_wg, 3);
 }
 
 // ---- wave-level search of a histogram from its top bin ----------------------------------
@@ -862,6 +767,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
 // ---- exact selection among the candidates -----------------------------------------------
 struct SelectArgs {
     uint2 *pairs;          // [rows, emit_cap] (key, retrieval-local index)
+    int raw_keys;          // the pairs hold logit bit patterns, not order-preserving keys (the decode step's scan writes those)
     uint16_t *aux;         // [rows, emit_cap] list ids (NULL: none)
     int64_t emit_cap;
     uint32_t *emit_count;  // [rows]
@@ -1101,8 +1007,11 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
     }
 }
 
+// order-preserving key of a candidate record: the record holds it, or the logit's bit pattern
+__device__ inline uint32_t record_key(uint32_t x, int raw) { return raw ? order_key(__uint_as_float(x)) : x; }
+
 template <int R>
-__device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
+__device__ inline void select_regs(int raw, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
                                    SelectOut out, uint32_t (*red)[kSelWaves],
                                    uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     uint32_t key[R], where[R], list[R];
@@ -1110,7 +1019,7 @@ __device__ inline void select_regs(uint32_t cnt, int k, const uint2 *pairs, cons
     for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
         const uint32_t p = (uint32_t)r * kSelThreads + threadIdx.x;
         const uint2 pr = p < cnt ? pairs[p] : make_uint2(0u, 0u);
-        key[r] = pr.x;
+        key[r] = p < cnt ? record_key(pr.x, raw) : 0u;
         where[r] = pr.y;
         list[r] = (aux && p < cnt) ? aux[p] : 0u;
     }
@@ -1175,23 +1084,57 @@ __device__ inline uint32_t kth_largest_mem(ValAt val_at, uint32_t cnt, uint32_t 
     return lo;
 }
 
-// Candidates in memory (any count): the same selection, streaming the pairs on every pass.
-__device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
-                                  SelectOut out, uint32_t (*red)[kSelWaves],
-                                  uint32_t *wsum, SelScratch *ss, float *ref1_out) {
+// One candidate as the streaming selection sees it.
+struct CandRec {
+    uint32_t key, where, list;
+};
+// candidates in memory: (key or logit bits, retrieval-local index) pairs and list ids
+struct MemRecords {
+    const uint2 *pairs;
+    const uint16_t *aux;
+    int raw;
+    __device__ inline uint32_t key(uint32_t p) const { return record_key(pairs[p].x, raw); }
+    __device__ inline CandRec rec(uint32_t p) const {
+        const uint2 pr = pairs[p];
+        return {record_key(pr.x, raw), pr.y, aux ? (uint32_t)aux[p] : 0u};
+    }
+};
+// every stored key of a stream as a candidate, scored again on every pass (a row whose estimate
+// failed: nothing is kept in memory, so the candidate area need not hold a whole row)
+struct IndexRecords {
+    const float *lut_s, *ls_s;  // LDS: the row's PQ table [128] and list scores [L]
+    const uint32_t *codes;
+    const uint16_t *list_ids;
+    const float *norms;
+    const int32_t *pos;
+    float qn, scale;
+    uint32_t L;
+    __device__ inline uint32_t lid(uint32_t p) const {
+        const uint32_t l = list_ids[p];
+        return l < L ? l : 0u;
+    }
+    __device__ inline uint32_t key(uint32_t p) const {
+        return order_key(score_one(lut_s, ls_s, codes[p], lid(p), qn, norms[p], scale));
+    }
+    __device__ inline CandRec rec(uint32_t p) const { return {key(p), pos ? (uint32_t)pos[p] : p, lid(p)}; }
+};
+
+// Any number of candidates, read (or scored) again on every pass.
+template <typename Records>
+__device__ inline void select_stream(const Records &src, uint32_t cnt, int k, SelectOut out, uint32_t (*red)[kSelWaves],
+                                     uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     const int tid = threadIdx.x;
     const uint32_t rounds = (cnt + kSelThreads - 1) / kSelThreads;
-    auto key_at = [=](uint32_t p) { return pairs[p].x; };
     int step = 0;
     uint32_t tkey = 0u;
     uint32_t idx_thr = 0xffffffffu;
     if (k > 0) {
         uint32_t c_gt = 0u;
-        tkey = kth_largest_mem([=](uint32_t p, uint32_t &v) { v = pairs[p].x; return true; }, cnt, (uint32_t)k, ss, wsum, c_gt);
+        tkey = kth_largest_mem([&](uint32_t p, uint32_t &v) { v = src.key(p); return true; }, cnt, (uint32_t)k, ss, wsum, c_gt);
         uint32_t c_eq = 0;
         for (uint32_t r = 0; r < rounds; ++r) {
             const uint32_t p = r * kSelThreads + tid;
-            c_eq += wave_count_if(p < cnt && key_at(p) == tkey);
+            c_eq += wave_count_if(p < cnt && src.key(p) == tkey);
         }
         c_eq = block_total_of_waves(c_eq, red, step++);
         const uint32_t want_ties = (uint32_t)k > c_gt ? (uint32_t)k - c_gt : 0u;
@@ -1199,32 +1142,32 @@ __device__ inline void select_mem(const SelectArgs &a, uint32_t cnt, int k, cons
             // among equal keys the lowest indices win: the want_ties-th largest of ~index
             uint32_t unused;
             const uint32_t t = tkey;
-            idx_thr = ~kth_largest_mem([=](uint32_t p, uint32_t &v) { const uint2 pr = pairs[p]; v = ~pr.y; return pr.x == t; },
+            idx_thr = ~kth_largest_mem([&](uint32_t p, uint32_t &v) { const CandRec c = src.rec(p); v = ~c.where; return c.key == t; },
                                        cnt, want_ties, ss, wsum, unused);
         }
     } else {
         uint32_t kmax = 0u;
-        for (uint32_t p = tid; p < cnt; p += kSelThreads) kmax = max(kmax, key_at(p));
+        for (uint32_t p = tid; p < cnt; p += kSelThreads) kmax = max(kmax, src.key(p));
         kmax = wave_max_u32(kmax);
         __syncthreads();
         if ((tid & (kWave - 1)) == 0) wsum[tid / kWave] = kmax;
         __syncthreads();
         for (int w = 0; w < kSelWaves; ++w) tkey = max(tkey, wsum[w]);
     }
-    auto selected = [=](uint2 pr) {
+    auto selected = [=](const CandRec &c) {
         if (k <= 0) return false;
-        if (pr.x != tkey || idx_thr == 0xffffffffu) return pr.x >= tkey;
-        return pr.y <= idx_thr;
+        if (c.key != tkey || idx_thr == 0xffffffffu) return c.key >= tkey;
+        return c.where <= idx_thr;
     };
     out.ref1 = (k > 0 || cnt > 0) ? key_to_float(tkey) : -INFINITY;
     *ref1_out = out.ref1;
     uint32_t mine = 0;
-    for (uint32_t p = tid; p < cnt; p += kSelThreads) mine += selected(pairs[p]) ? 1u : 0u;
+    for (uint32_t p = tid; p < cnt; p += kSelThreads) mine += selected(src.rec(p)) ? 1u : 0u;
     uint32_t at = block_exclusive_u32(mine, wsum);
     for (uint32_t p = tid; p < cnt; p += kSelThreads) {
-        const uint2 pr = pairs[p];
-        if (selected(pr)) out.winner(at++, pr.x, pr.y);
-        else out.loser(pr.x, aux ? aux[p] : 0u);
+        const CandRec c = src.rec(p);
+        if (selected(c)) out.winner(at++, c.key, c.where);
+        else out.loser(c.key, c.list);
     }
 }
 
@@ -1237,7 +1180,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
     __shared__ uint32_t wsum[2 * kSelWaves];
     __shared__ SelScratch ss;
-    float *mx = reinterpret_cast<float *>(smem);  // [L] (the re-scan parks its [128 + L] tables here first)
+    float *mx = reinterpret_cast<float *>(smem);  // [L] losers' weights per list; a re-scan keeps its [128 + L] tables behind it
     const int tid = threadIdx.x;
     const int g = blockIdx.x;
     const int bh = blockIdx.y;
@@ -1257,7 +1200,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             const int64_t p = (int64_t)r * kSelThreads + tid;
             const bool ok = p < a.emit_cap;
             const uint2 pr = ok ? pairs[p] : make_uint2(0u, 0u);
-            skey[r] = pr.x;
+            skey[r] = record_key(pr.x, a.raw_keys);
             swhere[r] = pr.y;
             slist[r] = (aux && ok) ? aux[p] : 0u;
         }
@@ -1268,31 +1211,19 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     // losers' weights join the scan's per-list sums of the row (same reference), unless those have to start over
     float *mass_out = a.mass ? a.mass + (size_t)bh * a.L * a.GP + g : nullptr;
     const float ref0 = mass_out ? a.ref_val[row] : -INFINITY;
-    const bool rescan = cnt < (uint32_t)k && a.codes;
-
+    // The estimate kept too few keys, or more than the candidate area holds: every stored key of
+    // the row becomes a candidate, scored again on each pass of the selection, and the row's
+    // background sums start over, relative to the k-th logit.
+    const bool rescan = (cnt < (uint32_t)k || (int64_t)cnt > a.emit_cap) && a.codes;
+    float *lut_s = mx + a.L;
+    float *ls_s = lut_s + kM * kCodes;
     if (rescan) {
-        // The estimate kept too few keys: score the whole row again and treat every key as a
-        // candidate.  The row's background sums start over, relative to the k-th logit.
         if (tid == 0 && a.rescans) atomicAdd(a.rescans, 1u);
-        float *lut_s = reinterpret_cast<float *>(smem);
-        float *ls_s = lut_s + kM * kCodes;
         for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
         for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
-        const float qn = a.qnorm[row];
-        __syncthreads();
-        const size_t base = (size_t)bh * a.n_cap;
-#pragma unroll 4
-        for (int p = tid; p < n; p += kSelThreads) {
-            uint32_t lid = a.list_ids[base + p];
-            if (lid >= (uint32_t)a.L) lid = 0u;
-            const float s = score_one(lut_s, ls_s, a.codes[base + p], lid, qn, a.norms[base + p], a.scale);
-            pairs[p] = make_uint2(order_key(s), a.pos ? (uint32_t)a.pos[base + p] : (uint32_t)p);
-            if (aux) aux[p] = (uint16_t)lid;
-        }
-        cnt = (uint32_t)n;
-        __threadfence_block();
-        __syncthreads();
+        cnt = (uint32_t)max(n, 0);
     }
+    cnt = (uint32_t)min((int64_t)cnt, rescan ? a.n_cap : a.emit_cap);
 
     if (mass_out)
         for (int l = tid; l < a.L; l += kSelThreads) mx[l] = 0.0f;
@@ -1318,15 +1249,21 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             done = true;
         }
     }
-    if (!done) {
+    if (!done && rescan) {
+        const size_t base = (size_t)bh * a.n_cap;
+        const IndexRecords all = {lut_s, ls_s, a.codes + base, a.list_ids + base, a.norms + base,
+                                  a.pos ? a.pos + base : nullptr, a.qnorm[row], a.scale, (uint32_t)a.L};
+        select_stream(all, cnt, k, out, red, wsum, &ss, &ref1);
+    } else if (!done) {
+        bool in_regs = false;
         if constexpr (RS == 0) {  // no estimate: pick the register variant from the count
-            if (cnt <= 4u * kSelThreads) select_regs<4>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else if (cnt <= 8u * kSelThreads) select_regs<8>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else if (cnt <= 16u * kSelThreads) select_regs<16>(cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-        } else {  // the estimate was exceeded, or the row was re-scanned (rare): stream from memory
-            select_mem(a, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            in_regs = cnt <= 16u * kSelThreads;
+            if (cnt <= 4u * kSelThreads) select_regs<4>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            else if (cnt <= 8u * kSelThreads) select_regs<8>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            else if (in_regs) select_regs<16>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
         }
+        // more candidates than the register variants hold (rare): stream them from memory
+        if (!in_regs) select_stream(MemRecords{pairs, aux, a.raw_keys}, cnt, k, out, red, wsum, &ss, &ref1);
     }
     PQHSA_TRACE_MARK(trace_select, trace_wg, 5);
     __syncthreads();
@@ -1374,11 +1311,6 @@ static size_t scan_lds_bytes(int GP, int L, int mode, int src, bool mass, bool a
     return b;
 }
 
-static int env_int(const char *name, int fallback) {
-    const char *v = getenv(name);
-    return v ? atoi(v) : fallback;
-}
-
 static int raise_lds_limit(const void *kernel, size_t lds, const char *what) {
     if (lds <= 64 * 1024) return PQHSA_OK;
     PQHSA_REQUIRE(lds <= 160 * 1024, "%s: %zu bytes of LDS needed", what, lds);
@@ -1392,7 +1324,7 @@ static int raise_lds_limit(const void *kernel, size_t lds, const char *what) {
 
 int pick_tile_keys(int64_t n_max, int streams) {
     // aim for a few workgroups per compute unit, tiles a multiple of one block iteration
-    static const int target = env_int("PQHSA_SCAN_WGS", 2048);
+    constexpr int target = 2048;
     int64_t tiles_per_stream = (target + streams - 1) / (streams > 0 ? streams : 1);
     if (tiles_per_stream < 1) tiles_per_stream = 1;
     int64_t keys = (n_max + tiles_per_stream - 1) / tiles_per_stream;
@@ -1447,7 +1379,6 @@ static int launch_scan_mode(const ScanArgs &a, int GP, int streams, int64_t n_ma
 int launch_scan(const ScanArgs &a, int mode, int src, int GP, int streams, int64_t n_max, hipStream_t stream) {
     if (src == kIndex) {
         if (mode == kWrite) return launch_scan_mode<kWrite, kIndex>(a, GP, streams, n_max, stream);
-        if (mode == kEmit) return launch_scan_mode<kEmit, kIndex>(a, GP, streams, n_max, stream);
     } else {
         if (mode == kHist) return launch_scan_mode<kHist, kLogits>(a, GP, streams, n_max, stream);
         if (mode == kEmit) return launch_scan_mode<kEmit, kLogits>(a, GP, streams, n_max, stream);
@@ -1472,7 +1403,7 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
 int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     if (streams == 0) return PQHSA_OK;
     // list weights of the losers; the re-scan path parks a (128 + L)-float table there first
-    const size_t lds = (size_t)(kM * kCodes + a.L) * sizeof(float);
+    const size_t lds = (size_t)(kM * kCodes + 2 * a.L) * sizeof(float);
     const dim3 grid(a.G, streams), block(kSelThreads);
     if (a.expected_candidates <= 0) hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
     else if (a.expected_candidates <= 4 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<4>, grid, block, lds, stream, a);
@@ -1482,24 +1413,13 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     return check_launch("select_final");
 }
 
-// Tile of the full scan of a decode step: whole 1024-key iterations, sized so that the launch has
-// about four workgroups per compute unit (256 units; PQHSA_EMIT_WGS overrides the target).
-int emit_tile_keys_for(int64_t n_cap, int streams) {
-    static const int target = env_int("PQHSA_EMIT_WGS", 1280);
-    int64_t tiles_per_stream = (target + streams - 1) / (streams > 0 ? streams : 1);
-    if (tiles_per_stream < 1) tiles_per_stream = 1;
-    int64_t keys = (n_cap + tiles_per_stream - 1) / tiles_per_stream;
-    keys = ((keys + kKeysPerIter - 1) / kKeysPerIter) * kKeysPerIter;
-    if (keys < 2 * kKeysPerIter) keys = 2 * kKeysPerIter;
-    if (keys > 16 * kKeysPerIter) keys = 16 * kKeysPerIter;
-    return (int)keys;
-}
+int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t stream);
 
 // sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
                        const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
                        uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
-                       uint16_t *aux, float *mass, uint32_t *rescans, int emit_tile_keys,
+                       uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
                        hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
@@ -1522,16 +1442,15 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.n_div = index->kv_heads; a.G = G;
     a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = index->pos;
     a.n_cap = index->n_cap; a.n_arr = index->n_idx;
-    a.tile_keys = emit_tile_keys;
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
-    a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = index->n_cap;
-    a.mass = mass; a.stage_cap = stage_cap_for(GP, emit_tile_keys);
-    rc = launch_scan(a, kEmit, kIndex, GP, streams, n_max, stream);
+    a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = emit_cap;
+    a.mass = mass;
+    rc = launch_scan_emit(a, GP, streams, n_max, stream);
     if (rc) return rc;
     profile_mark(kProfSelect, stream);
     // 3. exact selection among the candidates
     SelectArgs s = {};
-    s.pairs = static_cast<uint2 *>(pairs); s.aux = aux; s.emit_cap = index->n_cap; s.emit_count = emit_count;
+    s.pairs = static_cast<uint2 *>(pairs); s.raw_keys = 1; s.aux = aux; s.emit_cap = emit_cap; s.emit_count = emit_count;
     s.k_row = k_row; s.thr_key = thr_key; s.hi_key = hi_key; s.n_arr = index->n_idx; s.rows_per_n = index->kv_heads * GP; s.GP = GP; s.G = G;
     s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = topk_cnt; s.k_cap = select->k_cap;
     s.mass = mass; s.ref_val = ref_val; s.L = index->num_lists;

@@ -67,16 +67,16 @@ def test_static_scratch_entry_point_matches_the_workspace_one_twice_in_a_row():
 
 def test_static_scratch_entry_point_rejects_a_shape_beyond_its_array():
     lib = _lib.load()
-    idx = ops.DeviceIndex(4, 8, 512, 1 << 20, "cuda")   # far more candidates records than the array holds
-    need = lib.pqhsa_decode_workspace_bytes(4, 8, 4, idx.n_cap, 512, 4096)
+    idx = ops.DeviceIndex(16, 8, 512, 1 << 17, "cuda")   # 512 query rows x 20 000 selected keys: far more scratch
+    need = lib.pqhsa_decode_workspace_bytes(16, 8, 4, idx.n_cap, 512, 20000)
     assert need > lib.pqhsa_static_scratch_bytes()
     sel = _lib.Select()
-    sel.fraction, sel.topk, sel.k_cap = 0.0, 4096, 4096
+    sel.fraction, sel.topk, sel.k_cap = 0.0, 20000, 20000
     kvt = torch.zeros(2, 4, 16, 8, 128, dtype=torch.bfloat16, device="cuda")
-    table = torch.zeros(4, 2, dtype=torch.int32, device="cuda")
+    table = torch.zeros(16, 2, dtype=torch.int32, device="cuda")
     kv = ops.kv_paged(kvt, table)
-    q = torch.zeros(4, 32, 128, device="cuda")
-    sl = torch.zeros(4, dtype=torch.int32, device="cuda")
+    q = torch.zeros(16, 32, 128, device="cuda")
+    sl = torch.zeros(16, dtype=torch.int32, device="cuda")
     rc = lib.pqhsa_decode_step_static(q.data_ptr(), _lib.F32, q.data_ptr(), kv.ref(), idx.ref(), 4, sl.data_ptr(), 4, 0,
                                       68, ctypes.byref(sel), SCALE, ops.EPS, None, None, None,
                                       torch.cuda.current_stream().cuda_stream)
