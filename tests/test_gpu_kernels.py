@@ -433,6 +433,64 @@ def test_full_size_step_properties_at_the_benchmark_shapes(cfg):
     got = layer.out[b, h * G : (h + 1) * G].float()
     err = (got - want).abs()
     assert bool((err <= 2e-3 + 2.0 ** -8 * want.abs()).all()), float(err.max())
+    # the same step with fp32 queries and output (K/V stay bf16 in their pages): the stated bound as
+    # it is, with no allowance for a 16-bit output's own rounding
+    q32 = layer.q.float()
+    out32 = torch.empty_like(q32)
+    ops.decode_step(q32, out32, layer.kv, idx, G, layer.seq_lens, sink=sink, full_max=sink + bench.LOCAL,
+                    fraction=bench.FRACTION, topk=0, scale=1.0 / np.sqrt(128.0), workspace=layer.ws)
+    torch.cuda.synchronize()
+    err32 = (out32[b, h * G : (h + 1) * G] - want).abs()
+    assert float(err32.max()) <= 2e-3, float(err32.max())
+    print(f"cfg {cfg}: max |out - dense reference| {float(err.max()):.2e} (bf16 q/out), {float(err32.max()):.2e} (fp32 q/out)")
+
+
+def test_append_then_scan_at_the_long_context_shape():
+    """cfg 4 as the benchmark runs it: context 262 144, 4 KV heads, GQA 7, bf16 pages, and every
+    step appends one key per sequence (the one leaving the local window) before it scans.  After
+    each of a few fused append + decode steps: the new key's norm, list and codes are those of the
+    fixed-order oracle's encode of that row, the stored-key count moved, the selection is exactly
+    the k best of the logits pqhsa_lut_scan writes over the grown index, and no row was re-scanned."""
+    import bench
+    from oracle import fixed
+
+    dev = _cuda()
+    steps = 3
+    layer = bench.Layer(4, 777, torch.device(dev), room=steps + 1)
+    idx, G, H, B = layer.index, layer.G, layer.H, layer.B
+    stream = torch.cuda.current_stream().cuda_stream
+    coarse, books = idx.coarse.cpu().numpy(), idx.codebooks.cpu().numpy()
+    for t in range(1, steps + 1):
+        layer.append_step(stream)
+        torch.cuda.synchronize()
+        for b in range(B):
+            n_new = layer.n[b] + t
+            assert int(idx.n_idx[b]) == n_new and idx.n_host[b] == n_new
+            tok = bench.SINK + n_new - 1                       # the key that just left the local window
+            kk, _ = ops.paged_gather_range(layer.kv, b, tok, tok + 1)
+            for h in range(H):
+                bh = b * H + h
+                norms, lids, codes = fixed.encode(kk[h].float().cpu().numpy(), coarse[bh], books[bh])
+                at = n_new - 1                                # appended keys sit at the end, in insertion order
+                assert int(idx.pos[bh, at]) == at
+                assert u32(idx.codes[bh, at : at + 1])[0] == codes[0], (t, bh)
+                assert u16(idx.list_ids[bh, at : at + 1])[0] == lids[0], (t, bh)
+                assert float(idx.norms[bh, at]) == float(norms[0]), (t, bh)
+        qnorm, lut, ls = ops.lut_build(layer.q, idx, G)
+        logits = ops.lut_scan(idx, G, qnorm, lut, ls, 1.0 / np.sqrt(128.0))
+        for b in range(B):
+            n = layer.n[b] + t
+            k = ops.resolve_topk(n, bench.FRACTION, 0)
+            rows = slice(b * H, (b + 1) * H)
+            assert bool((layer.ws.topk_cnt.view(B * H, G)[rows] == k).all())
+            tidx = layer.ws.topk_idx.view(B * H, G, -1)[rows, :, :k].to(torch.int64)
+            tval = layer.ws.topk_val.view(B * H, G, -1)[rows, :, :k]
+            lg = logits.view(B * H, G, -1)[rows, :, :n]
+            assert torch.equal(torch.gather(lg, 2, tidx), tval), (t, b)
+            want = torch.topk(lg, k, dim=2)
+            assert torch.equal(tval.sort(dim=2, descending=True).values, want.values), (t, b)
+            assert bool((tidx.sort(dim=2).values.diff(dim=2) > 0).all()), (t, b)
+    assert layer.ws.rescans() == 0
 
 
 def test_decode_step_graph_replays_match_eager_runs():
