@@ -166,6 +166,47 @@ def index_add(index: RefIndex, keys: torch.Tensor) -> torch.Tensor:
     return list_ids
 
 
+def _ema_towards_means(table: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, lr: float, eps: float) -> torch.Tensor:
+    """Entries of ``table`` that own rows move to (1 - lr) * entry + lr * mean(rows they own); the
+    others stay (pq_hsa/index/ivfpq.py:1159-1177 for coarse centroids, pq_hsa/index/pq.py:155-170
+    for the codewords of one subspace)."""
+    sums = torch.zeros_like(table)
+    counts = torch.bincount(ids, minlength=table.shape[0]).to(rows.dtype)
+    sums.index_add_(0, ids, rows)
+    non_empty = counts > 0
+    means = sums[non_empty] / counts[non_empty].unsqueeze(1).clamp_min(eps)
+    out = table.clone()
+    out[non_empty] = (1.0 - lr) * table[non_empty] + lr * means
+    return out
+
+
+def online_refresh(index: RefIndex, keys: torch.Tensor, update_keys: torch.Tensor, lr: float = 0.05) -> RefIndex:
+    """IVFPQIndex.online_refresh (pq_hsa/index/ivfpq.py:647-707) with
+    ProductQuantizer.update_codebooks_ema (pq_hsa/index/pq.py:117-173): the update keys move the
+    coarse centroids they are assigned to, are assigned again, their residuals move the codewords
+    they are nearest to (assignments under the codebooks as they were), and then every key is
+    re-assigned and re-encoded under the moved tables."""
+    eps = index.eps
+    dirs, norms = project(keys, eps)
+    upd, _ = project(update_keys, eps)
+    coarse, books = index.coarse, index.codebooks
+    if upd.shape[0] > 0:
+        lids = torch.cdist(upd.float(), coarse.float(), p=2).argmin(dim=1)
+        coarse = _ema_towards_means(coarse, upd, lids, lr, eps)
+        lids = torch.cdist(upd.float(), coarse.float(), p=2).argmin(dim=1)
+        resid = upd - coarse[lids]
+        m, _, sd = books.shape
+        chunks = resid.reshape(resid.shape[0], m, sd)
+        moved = books.clone()
+        for s in range(m):
+            near = torch.cdist(chunks[:, s].float(), books[s].float(), p=2).argmin(dim=1)
+            moved[s] = _ema_towards_means(books[s], chunks[:, s], near, lr, eps)
+        books = moved
+    list_ids = torch.cdist(dirs.float(), coarse.float(), p=2).argmin(dim=1)
+    codes = pq_encode(dirs - coarse[list_ids], books)
+    return RefIndex(coarse, books, list_ids, pack_4bit_codes(codes), norms, eps)
+
+
 def value_sums(values: torch.Tensor, list_ids: torch.Tensor, num_lists: int):
     sums = torch.zeros(num_lists, values.shape[1], dtype=values.dtype)
     sums.index_add_(0, list_ids, values)
@@ -334,6 +375,25 @@ class RefStream:
             self._sums.index_add_(0, list_ids, self.values[old_end:new_end])
             self._counts += torch.bincount(list_ids, minlength=num_lists).to(self.values.dtype)
         self.vbar = centroids_from_sums(self._sums, self._counts)
+
+    def apply_pending_index_update(self, lr: float = 0.05) -> bool:
+        """The deferred strategy's flush (SparseKVCache.apply_pending_index_update ->
+        _refresh_index_now -> _online_refresh_index, pq_hsa/attention/kv_cache.py:266-314, 666-676):
+        the tokens appended since the last index update join the indexed length, the keys that enter
+        the retrieval region are the update batch of an online refresh over all retrieval keys, and
+        the per-list value means are rebuilt."""
+        if self.strategy != "deferred" or self.pending == 0:
+            return False
+        _, old_end = self.regions()
+        self.indexed_length = self.keys.shape[0]
+        self.pending = 0
+        s, new_end = self.regions()
+        if new_end == old_end:
+            return True
+        self.index = online_refresh(self.index, self.keys[s:new_end], self.keys[old_end:new_end], lr)
+        self.vbar = value_centroids(self.values[s:new_end], self.index.list_ids, self.index.coarse.shape[0])
+        self._sums = self._counts = None
+        return True
 
     def forward_many(self, queries, **kw):
         s, e = self.regions()

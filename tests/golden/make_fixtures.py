@@ -54,7 +54,8 @@ def index_config(num_lists: int) -> IVFPQConfig:
     )
 
 
-def attention_config(fraction: float, *, sink: int = 4, local: int = 64) -> SparseAttentionConfig:
+def attention_config(fraction: float, *, sink: int = 4, local: int = 64, strategy: str = "incremental",
+                     interval: int = 1) -> SparseAttentionConfig:
     return SparseAttentionConfig(
         sink_tokens=sink,
         local_window=local,
@@ -65,8 +66,8 @@ def attention_config(fraction: float, *, sink: int = 4, local: int = 64) -> Spar
         hybrid_value_mode="centroid",
         hybrid_topk_source="all_pq",
         hybrid_denominator_source="all_pq",
-        index_update_interval=1,
-        index_update_strategy="incremental",
+        index_update_interval=interval,
+        index_update_strategy=strategy,
         collect_attention_details=False,
     )
 
@@ -174,6 +175,54 @@ def make_case(name: str, *, ctx: int, heads: int, groups: int, num_lists: int, f
     print(name, {k: v.shape for k, v in out.items()}, os.path.getsize(path), "bytes")
 
 
+def make_deferred_case(name: str, *, ctx: int, heads: int, groups: int, num_lists: int, fraction: float,
+                       added: int, seed0: int) -> None:
+    """The deferred update strategy: ``added`` keys are appended without touching the index, then
+    ``apply_pending_index_update`` runs the reference's online refresh (EMA move of the coarse
+    centroids and PQ codewords, full re-encode, rebuilt value means).  Recorded: the trained index
+    before, everything the flush produces, and the attention output before and after it."""
+    out: dict[str, np.ndarray] = {}
+    dim = 128
+    icfg = index_config(num_lists)
+    acfg = attention_config(fraction, strategy="deferred", interval=8)
+    keys, values, queries = [], [], []
+    for h in range(heads):
+        k, v, q = make_head(ctx + added, dim=dim, groups=groups, seed=seed0 + h, num_clusters=num_lists)
+        k, v, q = k.to(torch.bfloat16).float(), v.to(torch.bfloat16).float(), q.to(torch.bfloat16).float()
+        keys.append(k)
+        values.append(v)
+        queries.append(q)
+    keys_t, values_t, queries_t = torch.stack(keys), torch.stack(values), torch.stack(queries)
+    out["keys"], out["values"], out["queries"] = np32(keys_t), np32(values_t), np32(queries_t)
+    out["meta"] = np.array([ctx, heads, groups, num_lists, added, acfg.sink_tokens, acfg.local_window],
+                           dtype=np.int64)
+    out["fraction"] = np.array([fraction], dtype=np.float64)
+    out["lr"] = np.array([icfg.online_codebook_lr], dtype=np.float64)
+    sidecar = GQASidecar(icfg, acfg, num_query_heads=heads * groups, num_kv_heads=heads)
+    sidecar.build_cache(keys_t[None, :, :ctx], values_t[None, :, :ctx])
+
+    def tables(tag: str) -> None:
+        out[f"{tag}_coarse"] = np.stack([np32(s.cache.index.coarse_centroids) for s in sidecar.streams])
+        out[f"{tag}_codebooks"] = np.stack([np32(s.cache.index.pq.codebooks) for s in sidecar.streams])
+        snaps = [snapshot(s) for s in sidecar.streams]
+        for key in snaps[0]:
+            out[f"{tag}_{key}"] = np.stack([s[key] for s in snaps])
+
+    tables("build")
+    for i in range(added):
+        sidecar.append(keys_t[None, :, ctx + i], values_t[None, :, ctx + i])
+    q_all = queries_t.reshape(1, heads * groups, dim)
+    assert all(s.cache.index.num_vectors == ctx - 4 - 64 for s in sidecar.streams)   # nothing indexed yet
+    out["pending_output"] = np32(sidecar.forward(q_all))[0]
+    flushed = [s.cache.apply_pending_index_update() for s in sidecar.streams]
+    assert all(flushed)
+    tables("flush")
+    out["flush_output"] = np32(sidecar.forward(q_all))[0]
+    path = os.path.join(HERE, f"{name}.npz")
+    np.savez_compressed(path, **out)
+    print(name, {k: v.shape for k, v in out.items()}, os.path.getsize(path), "bytes")
+
+
 def main() -> None:
     torch.manual_seed(0)
     torch.set_num_threads(4)
@@ -181,6 +230,8 @@ def main() -> None:
               bf16=False, steps=6, seed0=11)
     make_case("ref_bf16_gqa", ctx=640, heads=2, groups=4, num_lists=48, fraction=0.05,
               bf16=True, steps=4, seed0=23)
+    make_deferred_case("ref_deferred_flush", ctx=900, heads=2, groups=2, num_lists=32, fraction=0.03,
+                       added=24, seed0=41)
 
 
 if __name__ == "__main__":

@@ -525,3 +525,70 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
     for s_, a in enumerate(swapped):
         want = fused[s_] if s_ < 3 else fused[s_][[2, 0, 1]]
         close(a, want, ("rows swap", s_))
+
+
+def test_deferred_flush_reproduces_the_reference_online_refresh(golden_dir):
+    """The deferred strategy against vectors from the real reference: the reference's trained index
+    goes in, keys are appended without touching it, and apply_pending_index_update must move the
+    coarse centroids and PQ codewords to where the reference's online refresh moved them, re-encode
+    every key as the reference did, rebuild the list means, and attend as the reference does before
+    and after the flush."""
+    dev = _cuda()
+    from pqhsa_release_amd.attention import PQHSAEngine
+
+    fx = np.load(os.path.join(golden_dir, "ref_deferred_flush.npz"))
+    ctx, H, G, lists, added, sink, local = (int(x) for x in fx["meta"])
+    fraction = float(fx["fraction"][0])
+    ic, ac = _cfgs(lists, fraction, sink=sink, local=local, strategy="deferred", interval=8)
+    assert ic.online_codebook_lr == float(fx["lr"][0])
+    keys = torch.from_numpy(fx["keys"]).to(dev, torch.bfloat16)[None]
+    values = torch.from_numpy(fx["values"]).to(dev, torch.bfloat16)[None]
+    q = torch.from_numpy(fx["queries"]).reshape(1, H * G, DIM).to(dev)            # fp32 queries
+    eng = PQHSAEngine(ic, ac, batch=1, kv_heads=H, device=dev)
+    eng.adopt(keys[:, :, :ctx], values[:, :, :ctx])
+    eng.build([ctx], coarse=torch.from_numpy(fx["build_coarse"]), codebooks=torch.from_numpy(fx["build_codebooks"]))
+    n0 = eng.n(0)
+    for s in range(added):
+        eng.write_rows(keys[:, :, ctx + s], values[:, :, ctx + s])
+        eng.advance(1)
+    assert eng.n(0) == n0 and eng.deferred_pending
+    out = eng.forward(q, G)
+    assert float((out[0].cpu() - torch.from_numpy(fx["pending_output"])).abs().max()) <= 2e-3
+    assert eng.apply_pending_index_update() and not eng.apply_pending_index_update()
+    n = eng.n(0)
+    assert n == fx["flush_list_ids"].shape[1] == n0 + added
+    mismatched = 0
+    for h in range(H):
+        np.testing.assert_allclose(eng.index.coarse[h].cpu().numpy(), fx["flush_coarse"][h], rtol=0, atol=1e-6)
+        np.testing.assert_allclose(eng.index.codebooks[h].cpu().numpy(), fx["flush_codebooks"][h], rtol=0, atol=1e-6)
+        codes_t, lists_t, norms_t = eng.index.by_key(h, n)
+        got_lists, got_codes = u16(lists_t), u32(codes_t)
+        ref_lists, ref_codes = fx["flush_list_ids"][h], _words(fx["flush_packed"][h])
+        np.testing.assert_allclose(norms_t.cpu().numpy(), fx["flush_norms"][h], rtol=1e-6)
+        # the moved tables agree to 1e-6, not bit for bit (different summation order of the means):
+        # a key may change list or codeword only where its two nearest candidates are a near-tie
+        dirs = torch.from_numpy(fx["keys"][h, sink : sink + n])
+        dirs = dirs / torch.linalg.vector_norm(dirs, dim=-1, keepdim=True)
+        coarse = torch.from_numpy(fx["flush_coarse"][h])
+        d2 = torch.cdist(dirs, coarse) ** 2
+        for i in np.nonzero(got_lists != ref_lists)[0]:
+            a, b = float(d2[i, int(got_lists[i])]), float(d2[i, int(ref_lists[i])])
+            assert abs(a - b) <= 1e-5 * max(a, b), (h, i, a, b)
+            mismatched += 1
+        same_list = got_lists == ref_lists
+        books = torch.from_numpy(fx["flush_codebooks"][h])
+        resid = dirs - coarse[torch.from_numpy(ref_lists.astype(np.int64))]
+        for i in np.nonzero((got_codes != ref_codes) & same_list)[0]:
+            for m in range(8):
+                cg, cr = (int(got_codes[i]) >> (4 * m)) & 15, (int(ref_codes[i]) >> (4 * m)) & 15
+                if cg == cr:
+                    continue
+                sub = resid[i, 16 * m : 16 * m + 16]
+                a, b = float(((sub - books[m, cg]) ** 2).sum()), float(((sub - books[m, cr]) ** 2).sum())
+                assert abs(a - b) <= 1e-5 * max(a, b, 1e-6), (h, i, m, a, b)
+            mismatched += 1
+        np.testing.assert_allclose(eng.index.vbar[h].cpu().numpy(), fx["flush_vbar"][h], atol=2e-3 if mismatched else 1e-5)
+    out = eng.forward(q, G)
+    err = float((out[0].cpu() - torch.from_numpy(fx["flush_output"])).abs().max())
+    assert err <= 2e-3, err
+    print(f"deferred flush vs reference: {mismatched} near-tie keys of {H * n}, max |out - reference| {err:.2e}")

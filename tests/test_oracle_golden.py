@@ -174,3 +174,37 @@ def test_fixed_order_append_encode_and_value_summaries(golden_dir, name):
         for j in range(n1 - n0):
             fixed.value_append(fx["values"][h][s + n0 + j], int(fx["append_list_ids"][h][n0 + j]), sums, counts, vbar)
         np.testing.assert_allclose(vbar, fx["append_vbar"][h], rtol=0, atol=1e-6)
+
+
+def test_torch_restatement_reproduces_the_reference_deferred_flush(golden_dir):
+    """The deferred strategy: appended keys wait outside the index; the flush is the reference's
+    online refresh (EMA move of the coarse centroids and PQ codewords by the newly indexed keys,
+    re-encode of every retrieval key, rebuilt value means).  Vectors from the real reference."""
+    fx = np.load(os.path.join(golden_dir, "ref_deferred_flush.npz"))
+    ctx, heads, groups, lists, added, sink, local = (int(x) for x in fx["meta"])
+    fraction, lr = float(fx["fraction"][0]), float(fx["lr"][0])
+    pending, flushed = [], []
+    for h in range(heads):
+        keys, values = torch.from_numpy(fx["keys"][h]), torch.from_numpy(fx["values"][h])
+        st = tr.RefStream(sink=sink, local=local, fraction=fraction, scale=SCALE, num_lists=lists,
+                          strategy="deferred", update_interval=8).build(keys[:ctx], values[:ctx])
+        assert torch.equal(st.index.coarse, torch.from_numpy(fx["build_coarse"][h]))
+        assert torch.equal(st.index.codebooks, torch.from_numpy(fx["build_codebooks"][h]))
+        assert np.array_equal(st.index.packed.numpy(), fx["build_packed"][h])
+        for i in range(added):
+            st.append(keys[ctx + i], values[ctx + i])
+        assert st.index.list_ids.shape[0] == ctx - sink - local          # nothing indexed while deferred
+        q = torch.from_numpy(fx["queries"][h])
+        pending.append(st.forward_many(q))
+        assert st.apply_pending_index_update(lr) and not st.apply_pending_index_update(lr)
+        # the moved tables, then everything encoded under them
+        np.testing.assert_allclose(st.index.coarse.numpy(), fx["flush_coarse"][h], rtol=0, atol=1e-7)
+        np.testing.assert_allclose(st.index.codebooks.numpy(), fx["flush_codebooks"][h], rtol=0, atol=1e-7)
+        assert not np.array_equal(fx["flush_coarse"][h], fx["build_coarse"][h])
+        assert np.array_equal(st.index.list_ids.numpy(), fx["flush_list_ids"][h])
+        assert np.array_equal(st.index.packed.numpy(), fx["flush_packed"][h])
+        assert np.array_equal(st.index.norms.numpy(), fx["flush_norms"][h])
+        np.testing.assert_allclose(st.vbar.numpy(), fx["flush_vbar"][h], rtol=0, atol=1e-6)
+        flushed.append(st.forward_many(q))
+    np.testing.assert_allclose(torch.cat(pending).numpy(), fx["pending_output"], rtol=0, atol=1e-6)
+    np.testing.assert_allclose(torch.cat(flushed).numpy(), fx["flush_output"], rtol=0, atol=1e-6)
