@@ -5,6 +5,11 @@ Training happens once after prefill and is not part of the decode hot path; it p
 consume.  The procedure mirrors the reference's (pq_hsa/index/kmeans.py:134-227 seeded Lloyd
 iterations with empty-cluster reseeding; pq_hsa/index/ivfpq.py:275-348 coarse k-means on key
 directions, then PQ on the residuals with seed + 10000 + subspace; pq_hsa/index/pq.py:47-95).
+
+The seeded draws (the starting subset, replacements for empty clusters) are made with a CPU
+generator whatever device the keys are on, as the reference makes them for the CPU tensors it
+trains on: the same seed then starts the same trajectory here and there, and the arithmetic
+(torch products on the keys' device) is all that can differ.
 """
 
 from __future__ import annotations
@@ -32,16 +37,17 @@ def kmeans_l2(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed: 
         raise ValueError("cannot train k-means with zero vectors")
     if num_clusters <= 0:
         raise ValueError("num_clusters must be positive")
-    gen = torch.Generator(device=vectors.device)
+    gen = torch.Generator(device="cpu")
     gen.manual_seed(int(seed))
+    dev = vectors.device
     if initial_centroids is not None:
         if tuple(initial_centroids.shape) != (num_clusters, dim):
             raise ValueError(f"initial_centroids must have shape ({num_clusters}, {dim})")
         centroids = initial_centroids.to(device=vectors.device, dtype=vectors.dtype).clone()
     elif n >= num_clusters:
-        centroids = vectors[torch.randperm(n, generator=gen, device=vectors.device)[:num_clusters]].clone()
+        centroids = vectors[torch.randperm(n, generator=gen)[:num_clusters].to(dev)].clone()
     else:
-        extra = torch.randint(0, n, (num_clusters - n,), generator=gen, device=vectors.device)
+        extra = torch.randint(0, n, (num_clusters - n,), generator=gen).to(dev)
         centroids = torch.cat([vectors, vectors[extra]], dim=0).clone()
     assign = torch.zeros(n, dtype=torch.long, device=vectors.device)
     for _ in range(max_iter):
@@ -57,7 +63,7 @@ def kmeans_l2(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed: 
         sums[filled] /= counts[filled].unsqueeze(1).clamp_min(eps)
         empty = ~filled
         if bool(empty.any()):
-            pick = torch.randint(0, n, (int(empty.sum().item()),), generator=gen, device=vectors.device)
+            pick = torch.randint(0, n, (int(empty.sum().item()),), generator=gen).to(dev)
             sums[empty] = vectors[pick].float()
         centroids = sums.to(vectors.dtype)
     return centroids, _nearest(vectors, centroids)
@@ -98,16 +104,16 @@ class _LazyGenerators:
     """One generator per stream, all seeded alike, created only for a stream that needs a draw of
     its own (an empty cluster) and first advanced past the draws every stream shares."""
 
-    def __init__(self, streams: int, seed: int, device, n: int, shared_perm: bool) -> None:
+    def __init__(self, streams: int, seed: int, n: int, shared_perm: bool) -> None:
         self.gens = [None] * streams
-        self.seed, self.device, self.n, self.shared_perm = int(seed), device, n, shared_perm
+        self.seed, self.n, self.shared_perm = int(seed), n, shared_perm
 
     def get(self, s: int) -> torch.Generator:
         if self.gens[s] is None:
-            g = torch.Generator(device=self.device)
+            g = torch.Generator(device="cpu")
             g.manual_seed(self.seed)
             if self.shared_perm:
-                torch.randperm(self.n, generator=g, device=self.device)
+                torch.randperm(self.n, generator=g)
             self.gens[s] = g
         return self.gens[s]
 
@@ -136,16 +142,16 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
     if n == 0:
         raise ValueError("cannot train k-means with zero vectors")
     dev = vectors.device
-    gen = torch.Generator(device=dev)
+    gen = torch.Generator(device="cpu")
     gen.manual_seed(int(seed))
-    lazy = _LazyGenerators(s, seed, dev, n, shared_perm=n >= num_clusters)
+    lazy = _LazyGenerators(s, seed, n, shared_perm=n >= num_clusters)
     if n >= num_clusters:
-        centroids = vectors[:, torch.randperm(n, generator=gen, device=dev)[:num_clusters]].clone()
+        centroids = vectors[:, torch.randperm(n, generator=gen)[:num_clusters].to(dev)].clone()
     else:
-        extra = torch.randint(0, n, (num_clusters - n,), generator=gen, device=dev)
+        extra = torch.randint(0, n, (num_clusters - n,), generator=gen).to(dev)
         centroids = torch.cat([vectors, vectors[:, extra]], dim=1).clone()
         for i in range(s):  # every stream's own generator has made this draw too
-            torch.randint(0, n, (num_clusters - n,), generator=lazy.get(i), device=dev)
+            torch.randint(0, n, (num_clusters - n,), generator=lazy.get(i))
     assign = torch.zeros(s, n, dtype=torch.long, device=dev)
     live = torch.ones(s, dtype=torch.bool, device=dev)
     offsets = (torch.arange(s, device=dev) * num_clusters).unsqueeze(1)
@@ -168,7 +174,7 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
             for i in torch.nonzero(empty.any(dim=1)).flatten().tolist():
                 if not bool(live[i]):
                     continue
-                pick = torch.randint(0, n, (int(empty[i].sum().item()),), generator=lazy.get(i), device=dev)
+                pick = torch.randint(0, n, (int(empty[i].sum().item()),), generator=lazy.get(i)).to(dev)
                 sums[i][empty[i]] = vectors[i][pick].float()
         centroids = torch.where(live.view(s, 1, 1), sums.to(vectors.dtype), centroids)
     return centroids, _nearest_batched(vectors, centroids)

@@ -208,3 +208,25 @@ def test_torch_restatement_reproduces_the_reference_deferred_flush(golden_dir):
         flushed.append(st.forward_many(q))
     np.testing.assert_allclose(torch.cat(pending).numpy(), fx["pending_output"], rtol=0, atol=1e-6)
     np.testing.assert_allclose(torch.cat(flushed).numpy(), fx["flush_output"], rtol=0, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", CASES)
+def test_product_index_training_follows_the_reference_trajectory(golden_dir, name):
+    """pqhsa_release_amd.index.train (what builds an index on the device) run on CPU tensors: the
+    seeded draws and Lloyd iterations are the reference's, so the trained coarse centroids and PQ
+    codebooks are the ones the reference trained (recorded in the fixtures), per stream and for all
+    streams of a sequence at once."""
+    from pqhsa_release_amd.index.train import train_ivfpq, train_ivfpq_batched
+
+    fx, m = load(golden_dir, name)
+    retr = slice(m["sink"], m["ctx"] - m["local"])
+    keys = torch.from_numpy(fx["keys"])[:, retr]
+    for h in range(m["heads"]):
+        coarse, books = train_ivfpq(keys[h], num_lists=m["lists"], coarse_iter=1, pq_iter=2, seed=0)
+        np.testing.assert_allclose(coarse.numpy(), fx["coarse"][h], rtol=0, atol=1e-6)
+        np.testing.assert_allclose(books.numpy(), fx["codebooks"][h], rtol=0, atol=1e-6)
+        ref = tr.train_index(keys[h], num_lists=m["lists"], coarse_iter=1, pq_iter=2, seed=0)
+        assert torch.equal(ref.coarse, torch.from_numpy(fx["coarse"][h]))
+    coarse, books = train_ivfpq_batched(keys, num_lists=m["lists"], coarse_iter=1, pq_iter=2, seed=0)
+    np.testing.assert_allclose(coarse.numpy(), fx["coarse"], rtol=0, atol=1e-6)
+    np.testing.assert_allclose(books.numpy(), fx["codebooks"], rtol=0, atol=1e-6)
