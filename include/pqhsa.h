@@ -193,13 +193,22 @@ int pqhsa_topk_radix(const float *logits, int64_t stride, int32_t rows, const in
 /*
  * The whole single-token decode attention of one layer, for every sequence of the batch:
  * LUT build -> threshold estimate from the sampled keys -> one fused scan that keeps the
- * candidates above it and sums the other keys' weights per list -> exact radix selection of
- * the top-k among the candidates (a row whose estimate kept fewer than k keys is re-scanned
- * in full, so the result is always the exact top-k) -> exact attention over sink, local
- * window and the selected keys read in place from `kv`, merged with the per-list background
- * (list mass x list mean value) in one softmax.
+ * candidates above it (at most 3 k_cap + 2048 records per query row) and sums the other keys'
+ * weights per list -> exact radix selection of the top-k among the candidates (a row whose
+ * estimate kept fewer than k keys, or more than its record area holds, is selected from a full
+ * pass over its keys instead, so the result is always the exact top-k) -> exact attention over
+ * sink, local window and the selected keys read in place from `kv`, merged with the per-list
+ * background (list mass x list mean value) in one softmax.
  *   q, out     [B, H*G, 128] of q_dtype
  *   seq_lens   i32 [B] device: tokens currently in the cache of each sequence
+ *   n_max      host-side upper bound of the keys any sequence has indexed (max_b n_idx[b]);
+ *              it sizes the scan's grid.  A HARD bound: keys of a sequence beyond n_max are
+ *              not scanned (the kernels clamp to it and to index->n_cap; nothing is read out
+ *              of bounds, the result for that sequence is then not the reference's)
+ *   full_max   host-side upper bound of sink + local-window rows of any sequence
+ *              (min(sink, seq_lens[b]) + seq_lens[b] - sink - n_idx[b]); with select->k_cap it
+ *              sizes the attention launch and its LDS row list.  A HARD bound as well: a sequence
+ *              whose device-side lengths give more rows has the excess rows cut off
  *   topk_idx   i32 [BH, G, k_cap], topk_val f32 same shape, topk_cnt i32 [BH, G]: the
  *              selected keys (retrieval-local indices, unordered) — optional outputs, may be NULL
  * Replaces IVFPQSparseAttention.forward_many for mode "hybrid", value mode "centroid",
@@ -260,8 +269,9 @@ int pqhsa_decode_step_static(const void *q, int32_t q_dtype, void *out, const pq
                              float *topk_val, int32_t *topk_cnt, void *stream);
 
 /*
- * Rows whose threshold estimate kept fewer than k candidates and were re-scanned in full since
- * the workspace was first used (a device-memory counter inside the workspace, for monitoring).
+ * Rows whose threshold estimate kept fewer than k candidates (or more than the record area
+ * holds) and were selected from a full pass since the workspace was first used (a device-memory
+ * counter inside the workspace, for monitoring).
  */
 const uint32_t *pqhsa_decode_rescan_counter(void *workspace);
 

@@ -109,9 +109,10 @@ class PQHSAEngine:
                 self.values_buf[b, :, ln].copy_(values[b])
 
     # ------------------------------------------------------------------ index
-    def _effective_lists(self) -> int:
-        smallest = min((self.n(b) for b in range(self.B) if self.n(b) > 0), default=1)
-        return max(1, min(self.index_config.num_lists, smallest))
+    def _lists_of(self, count: int) -> int:
+        """Coarse lists a stream of ``count`` keys trains: the configured number, or one per key
+        when there are fewer keys than that (IVFPQIndex.build, pq_hsa/index/ivfpq.py:300)."""
+        return max(1, min(self.index_config.num_lists, int(count)))
 
     def _alloc_index(self, n_need: int, num_lists: int) -> None:
         old = self.index
@@ -149,7 +150,10 @@ class PQHSAEngine:
         self.deferred_pending = False
         self._fused_append = False
         counts = [self.n(b) for b in range(self.B)]
-        lists = self._effective_lists() if coarse is None else int(coarse.shape[-2])
+        # the tables are as wide as the longest sequence needs; a shorter sequence trains its own,
+        # smaller number of lists and the columns it leaves unused are filled with centroids that no
+        # key can be nearest to (DeviceIndex.pad_lists), so every stream keeps the reference's lists
+        lists = self._lists_of(max(counts)) if coarse is None else int(coarse.shape[-2])
         self.index = None
         self._alloc_index(max(counts), lists)
         ic = self.index_config
@@ -164,12 +168,13 @@ class PQHSAEngine:
                 for i in range(0, len(seqs), step):
                     part = seqs[i : i + step]
                     rows = torch.stack([self._retrieval_block(b, n) for b in part]).reshape(-1, n, ops.HEAD_DIM)
-                    c, cb = train_ivfpq_batched(rows, num_lists=lists, coarse_iter=ic.coarse_max_iter,
+                    c, cb = train_ivfpq_batched(rows, num_lists=self._lists_of(n), coarse_iter=ic.coarse_max_iter,
                                                 pq_iter=ic.pq_max_iter, seed=ic.seed, eps=ic.eps)
                     del rows
                     for j, b in enumerate(part):
                         sl = slice(b * self.H, (b + 1) * self.H)
                         self.index.coarse[sl, : c.shape[1]].copy_(c[j * self.H : (j + 1) * self.H])
+                        self.index.pad_lists(sl, c.shape[1])
                         self.index.codebooks[sl].copy_(cb[j * self.H : (j + 1) * self.H])
         else:
             self.index.coarse.copy_(coarse.to(self.device, torch.float32).expand_as(self.index.coarse))
@@ -361,12 +366,14 @@ class PQHSAEngine:
         if self._fused_append:
             self._fused_append = False
             old = [self.n(b) for b in range(self.B)]
+            was = (list(self.indexed_len), list(self.pending))
             self.indexed_len = list(self.lens)
             self.pending = [0] * self.B
             added = [self.n(b) - n0 for b, n0 in enumerate(old)]
             if max(added) > 1 or max(self.n(b) for b in range(self.B)) > self.index.n_cap:
-                # not the one-key case after all (or the index must grow first): the separate path
-                self.indexed_len = [ln - 1 for ln in self.lens]
+                # not the one-key case after all (or the index must grow first): the separate path,
+                # from the bookkeeping as it stood (only some sequences may have advanced)
+                self.indexed_len, self.pending = was
                 self._refresh_index_now()
                 added = None
             elif max(added) == 1:

@@ -164,11 +164,14 @@ class DeviceIndex:
     def regroup(cls, sources, n_cap: int) -> "DeviceIndex":
         """A new index whose sequence b is sequence ``seq`` of ``index`` for ``(index, seq) =
         sources[b]``: the rows are copied on the device, nothing is re-encoded.  All sources share
-        KV heads, list count and device; ``n_cap`` is raised to the longest sequence if smaller."""
+        KV heads and device; the new tables are as wide as the widest source's and a sequence from
+        a narrower one leaves the rest unused (``pad_lists``).  ``n_cap`` is raised to the longest
+        sequence if smaller."""
         first = sources[0][0]
-        h, lists = first.kv_heads, first.num_lists
-        if any(ix.kv_heads != h or ix.num_lists != lists or ix.device != first.device for ix, _ in sources):
-            raise ValueError("regroup: the source indexes differ in KV heads, list count or device")
+        h = first.kv_heads
+        if any(ix.kv_heads != h or ix.device != first.device for ix, _ in sources):
+            raise ValueError("regroup: the source indexes differ in KV heads or device")
+        lists = max(ix.num_lists for ix, _ in sources)
         n_cap = max(int(n_cap), max(ix.n_host[seq] for ix, seq in sources))
         new = cls(len(sources), h, lists, n_cap, first.device)
         for b, (ix, seq) in enumerate(sources):
@@ -179,12 +182,25 @@ class DeviceIndex:
             skeep = min(ix.s_cap, new.s_cap)
             for name in ("s_codes", "s_list_ids", "s_norms"):
                 getattr(new, name)[dst, :skeep].copy_(getattr(ix, name)[src, :skeep])
-            for name in ("coarse", "codebooks", "vbar", "vsum", "vcount"):
-                getattr(new, name)[dst].copy_(getattr(ix, name)[src])
+            for name in ("coarse", "vbar", "vsum", "vcount"):
+                getattr(new, name)[dst, : ix.num_lists].copy_(getattr(ix, name)[src])
+            new.pad_lists(dst, ix.num_lists)
+            new.codebooks[dst].copy_(ix.codebooks[src])
             new.s_n[b : b + 1].copy_(ix.s_n[seq : seq + 1])
             new.n_sorted_host[b] = ix.n_sorted_host[seq]
         new.set_counts([ix.n_host[seq] for ix, seq in sources])
         return new
+
+    # Every component of an unused coarse centroid.  Keys are indexed by their direction (unit
+    # vectors) and real centroids are means of directions, so a real centroid is within distance 2
+    # of any key and one of these is about 1e5 away: it is never the nearest, its list stays empty
+    # and its per-list sums stay zero.  Products with it stay far inside the fp32 range.
+    PAD_CENTROID = 1.0e4
+
+    def pad_lists(self, rows: slice, used: int) -> None:
+        """Streams ``rows`` use only the first ``used`` coarse lists."""
+        if used < self.num_lists:
+            self.coarse[rows, used:] = self.PAD_CENTROID
 
     @classmethod
     def sample_size(cls, n: int) -> int:

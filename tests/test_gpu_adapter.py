@@ -423,22 +423,26 @@ def test_vllm_hook_extends_a_checkpointed_prefix_when_the_prompt_continues_it(mo
         rt.reset_pq_hsa_layer_state()
 
 
-def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
-    """PQ_HSA_BATCH=1: a ragged decode batch through the hook, once with one engine for the whole
-    batch (the default: appends ride on the decode launches) and once with one sidecar per
-    request (the reference's form); both must agree with each other step by step, and the
-    batch must be rebuilt when a request leaves."""
-    dev = _cuda()
+def _batch_hook(dev, monkeypatch, ctxs, steps, *, share_first_block=False, request_ids=False, lists="64"):
+    """A paged cache holding one synthetic request per entry of ``ctxs`` and a ``run(fused, reqs_at)``
+    that drives the wrapped forward for ``steps + 1`` decode steps over the requests ``reqs_at(step)``
+    names, returning the outputs per step and the runtime's counters.  ``share_first_block``: the
+    first two requests begin with the same 16 tokens and share their first physical block, as under
+    vLLM's prefix caching.  ``request_ids``: the metadata carries a model runner with vLLM's
+    request ids."""
     from pqhsa_release_amd.vllm_backend import pq_hsa_decode_runtime as rt
     from pqhsa_release_amd.vllm_backend import pq_hsa_flashattn_wrap as wrap
 
-    H, G, bs, steps = 2, 4, 16, 6
-    ctxs = [1500, 900, 1203]
+    H, G, bs = 2, 4, 16
     B = len(ctxs)
     probs = [_problem(dev, heads=H, groups=G, ctx=c, extra=steps, seed=50 + i) for i, c in enumerate(ctxs)]
     per_seq = (max(ctxs) + steps + bs - 1) // bs
     perm = torch.randperm(B * per_seq, generator=torch.Generator().manual_seed(3)).to(torch.int32).to(dev)
     table = perm.reshape(B, per_seq).contiguous()
+    if share_first_block:
+        probs[1][0][:, :, :bs] = probs[0][0][:, :, :bs]
+        probs[1][1][:, :, :bs] = probs[0][1][:, :, :bs]
+        table[1, 0] = table[0, 0]
     cache = torch.zeros(2, B * per_seq, bs, H, DIM, dtype=torch.bfloat16, device=dev)
     for b, (keys, values, _) in enumerate(probs):
         pos = torch.arange(ctxs[b], device=dev)
@@ -456,7 +460,7 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
         for k in list(os.environ):
             if k.startswith("PQ_HSA_"):
                 monkeypatch.delenv(k)
-        for k, v in {"PQ_HSA_ENABLE": "1", "PQ_HSA_BATCH": "1", "PQ_HSA_BATCH_FUSED": fused, "PQ_HSA_NUM_LISTS": "64",
+        for k, v in {"PQ_HSA_ENABLE": "1", "PQ_HSA_BATCH": "1", "PQ_HSA_BATCH_FUSED": fused, "PQ_HSA_NUM_LISTS": lists,
                      "PQ_HSA_TOP_FRAC": "0.02", "PQ_HSA_LOCAL": "64", "PQ_HSA_UPD_INTERVAL": "1",
                      "PQ_HSA_FLUSH_INTERVAL": "0"}.items():
             monkeypatch.setenv(k, v)
@@ -476,6 +480,9 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
                 md = types.SimpleNamespace(max_query_len=1, num_actual_tokens=len(reqs), use_cascade=False,
                                            max_seq_len=max(lens), block_table=tb, slot_mapping=slots,
                                            seq_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
+                if request_ids:
+                    md._pq_runner = types.SimpleNamespace(
+                        input_batch=types.SimpleNamespace(req_ids=[f"req-{b}" for b in reqs] + [None]), requests={})
                 k_new = torch.cat([probs[b][0][:, :, ctxs[b] + s - 1] for b in reqs])      # [R, H, D]
                 v_new = torch.cat([probs[b][1][:, :, ctxs[b] + s - 1] for b in reqs])
                 query = torch.cat([probs[b][2][0, :, s].reshape(1, H * G, DIM) for b in reqs])
@@ -488,14 +495,28 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
             wrap.unwrap_forward(Impl)
             rt.reset_pq_hsa_layer_state()
 
+    return run
+
+
+def _close(a, b, what):
+    # the same kernels on the same trained indexes: only bf16 rounding of the output differs
+    assert np.abs(a - b).max() <= 2e-3 + 2.0 ** -7 * np.abs(b).max(), (what, np.abs(a - b).max())
+
+
+def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
+    """PQ_HSA_BATCH=1: a ragged decode batch through the hook, once with one engine for the whole
+    batch (the default: appends ride on the decode launches) and once with one sidecar per
+    request (the reference's form); both must agree with each other step by step, and the
+    batch must be rebuilt when a request leaves."""
+    dev = _cuda()
+    steps = 6
+    run = _batch_hook(dev, monkeypatch, [1500, 900, 1203], steps)
+    close = _close
+
     everyone = lambda s: [0, 1, 2]
     one_leaves = lambda s: [0, 1, 2] if s < 4 else [0, 2]
     one_joins = lambda s: [0, 1] if s < 3 else [0, 1, 2]
     rows_swap = lambda s: [0, 1, 2] if s < 3 else [2, 0, 1]
-
-    def close(a, b, what):
-        # the same kernels on the same trained indexes: only bf16 rounding of the output differs
-        assert np.abs(a - b).max() <= 2e-3 + 2.0 ** -7 * np.abs(b).max(), (what, np.abs(a - b).max())
 
     fused, st_f = run("1", everyone)
     single, st_s = run("0", everyone)
@@ -519,12 +540,54 @@ def test_vllm_hook_batch_mode_one_engine_for_all_requests(monkeypatch):
     for s_, (a, b) in enumerate(zip(joined, single_j)):
         close(a, b, ("one joins", s_))
 
-    # requests change rows: told apart by their first block, their indexes move with them
+    # requests change rows: told apart by the blocks they own, their indexes move with them
     swapped, st_w = run("1", rows_swap)
     assert st_w["pq_batch_group_builds"] == 1 and st_w["pq_batch_regroups"] == 1 and st_w["pq_build_calls"] == 1
     for s_, a in enumerate(swapped):
         want = fused[s_] if s_ < 3 else fused[s_][[2, 0, 1]]
         close(a, want, ("rows swap", s_))
+
+
+@pytest.mark.parametrize("request_ids", [False, True])
+def test_vllm_hook_batch_mode_tells_apart_requests_that_share_their_first_block(monkeypatch, request_ids):
+    """Two live requests with a common prompt prefix share their first physical block (vLLM's
+    prefix caching).  When the batch rows are permuted each request must keep its own index: by
+    vLLM's request ids when the metadata carries the runner, by the blocks a request alone owns
+    otherwise.  Nothing is rebuilt, and every output is what the unpermuted batch gives."""
+    dev = _cuda()
+    steps = 5
+    run = _batch_hook(dev, monkeypatch, [1100, 1100, 700], steps, share_first_block=True, request_ids=request_ids)
+    base, st_b = run("1", lambda s: [0, 1, 2])
+    assert st_b["pq_batch_group_builds"] == 1 and st_b["pq_batch_regroups"] == 0
+    swapped, st_w = run("1", lambda s: [0, 1, 2] if s < 2 else [1, 0, 2])
+    assert st_w["pq_batch_group_builds"] == 1 and st_w["pq_batch_regroups"] == 1 and st_w["pq_build_calls"] == 1
+    for s_, a in enumerate(swapped):
+        _close(a, base[s_] if s_ < 2 else base[s_][[1, 0, 2]], ("shared first block", s_))
+    # requests 0 and 1 are equally long here: had they been confused, 1's queries would have run on 0's index
+    assert np.abs(base[3][0] - base[3][1]).max() > 0.05
+
+
+def test_vllm_hook_batch_mode_with_a_request_shorter_than_the_list_count(monkeypatch):
+    """A request with fewer indexed keys than PQ_HSA_NUM_LISTS joins a running batch and leaves
+    again.  Every stream keeps the list count it would have alone (the short one trains one list
+    per key, the long ones all 64; unused table columns are padded), so the outputs are those of
+    one sidecar per request, and the batch is regrouped, not rebuilt."""
+    dev = _cuda()
+    steps = 6
+    ctxs = [1500, 110, 900]                    # 110 tokens: 42 keys to index with sink 4 and local window 64
+    run = _batch_hook(dev, monkeypatch, ctxs, steps)
+    comes_and_goes = lambda s: [0, 2] if s < 2 else ([0, 2, 1] if s < 5 else [0, 2])   # per-row sidecars keep rows 0, 1
+    fused, st_f = run("1", comes_and_goes)
+    single, _ = run("0", comes_and_goes)
+    assert st_f["pq_batch_group_builds"] == 1 and st_f["pq_batch_regroups"] == 2 and st_f["pq_build_calls"] == 2
+    for s_, (a, b) in enumerate(zip(fused, single)):
+        _close(a, b, ("short request", s_))
+    # and the whole batch built at once, short request included
+    together, st_t = run("1", lambda s: [0, 1, 2])
+    alone, _ = run("0", lambda s: [0, 1, 2])
+    assert st_t["pq_batch_group_builds"] == 1 and st_t["pq_batch_regroups"] == 0
+    for s_, (a, b) in enumerate(zip(together, alone)):
+        _close(a, b, ("short request from the start", s_))
 
 
 def test_deferred_flush_reproduces_the_reference_online_refresh(golden_dir):

@@ -319,6 +319,43 @@ def test_decode_step_selects_from_a_full_pass_when_candidates_outgrow_their_area
     assert int(ws.candidate_counts()[:, : p.G].min()) == p.n(1)   # the scan counted every key of the shorter row
 
 
+def test_decode_step_with_device_lengths_beyond_the_host_bounds_exits_normally():
+    """``full_max`` and ``n_max`` size the launch on the host; the lengths the kernels read live on
+    the device.  When the device-side lengths run ahead of those bounds (a host mirror one step
+    behind) the kernels cut the excess off instead of writing past the areas the launch sized:
+    the step completes, its output is finite, the selection among the scanned keys is intact, and
+    a correctly sized step afterwards gives the oracle's result."""
+    dev = _cuda()
+    p = Problem(lens=[6000, 4100], heads=2, groups=3, lists=32, seed=41)
+    idx = p.device_index(dev)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    k_cap = ops.resolve_topk(p.n_max, 0.03, 0)
+    ws = ops.DecodeWorkspace(idx, p.G, k_cap)
+    q = p.q_tensor()
+    out = torch.empty_like(q)
+    # one row more on the device than the host sized the attention launch for
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local - 1, fraction=0.03,
+                    topk=0, scale=SCALE, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+    for (b, h) in p.index:
+        _, want_idx, _ = p.oracle_step(b, h, 0.03)
+        for g in range(p.G):
+            assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (b, h, g)
+    # a scan sized for fewer keys than the device-side counts say
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
+                    topk=0, scale=SCALE, workspace=ws, n_max=p.n_max - 1500)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    cnt = ws.topk_cnt.cpu().numpy()
+    assert (cnt >= 0).all() and (cnt <= k_cap).all()
+    sel = ws.topk_idx.cpu().numpy().reshape(p.B * p.H * p.G, -1)
+    for r in range(sel.shape[0]):
+        assert (sel[r, : cnt.reshape(-1)[r]] >= 0).all() and (sel[r, : cnt.reshape(-1)[r]] < p.n_max).all()
+    _check_step(p, idx, kv, ws, 0.03)
+
+
 def test_decode_step_on_unsorted_and_partly_sorted_layouts():
     """The same step over (i) an index that was never sorted or sampled (every key is a candidate),
     (ii) a sorted prefix followed by an insertion-order tail, as after appends."""
