@@ -357,10 +357,6 @@ class PQHSAEngine:
         q = q.contiguous()
         if out is None:
             out = torch.empty_like(q)
-        ws = self._ws.get(groups)
-        k_cap = ops.resolve_topk(self.index.n_cap, ac.retrieval_top_fraction, ac.retrieval_topk)
-        if ws is None or ws.k_cap < k_cap:
-            ws = self._ws[groups] = ops.DecodeWorkspace(self.index, groups, k_cap)
         scale = (1.0 / math.sqrt(D)) if ac.scale is None else float(ac.scale)
         append_count, added = None, None
         if self._fused_append:
@@ -383,6 +379,10 @@ class PQHSAEngine:
                 append_count = self._append_counts[key]
             else:
                 added = None
+        ws = self._ws.get(groups)       # looked up only now: an index that had to grow above has dropped the old ones
+        k_cap = ops.resolve_topk(self.index.n_cap, ac.retrieval_top_fraction, ac.retrieval_topk)
+        if ws is None or ws.k_cap < k_cap:
+            ws = self._ws[groups] = ops.DecodeWorkspace(self.index, groups, k_cap)
         full_max = max(self.full_count(b) for b in range(self.B))
         n_max = self.index.n_max + (1 if append_count is not None else 0)
         ops.decode_step(q, out, self.kv, self.index, groups, self.seq_lens, sink=self.sink, full_max=full_max,

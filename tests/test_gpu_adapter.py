@@ -126,7 +126,8 @@ def _problem(dev, *, batch=1, heads=2, groups=4, ctx=1500, extra=40, dtype=torch
 
     k, v, _ = make_layer(ctx + extra, batch=batch, kv_heads=heads, groups=1, seed0=seed, dtype=dtype)
     gen = torch.Generator().manual_seed(seed + 1)
-    q = k[:, :, 100:100 + (extra + 1) * groups].float() + 0.2 * torch.randn(batch, heads, (extra + 1) * groups, DIM,
+    first = min(100, k.shape[2] - (extra + 1) * groups)      # queries near some of the keys
+    q = k[:, :, first:first + (extra + 1) * groups].float() + 0.2 * torch.randn(batch, heads, (extra + 1) * groups, DIM,
                                                                               generator=gen)
     q = q.reshape(batch, heads, extra + 1, groups, DIM).to(dtype)
     return k.to(dev), v.to(dev), q.to(dev)
@@ -187,6 +188,48 @@ def test_gqa_adapter_decode_steps_match_oracle_on_its_own_index():
     res16 = ad.forward(q[:, :, extra].reshape(1, H * G, DIM))
     assert res16.context.dtype == torch.bfloat16
     assert np.abs(res16.context.float().cpu().numpy() - want).max() <= 2e-3 + 2.0 ** -8 * np.abs(want).max()
+
+
+def test_engine_one_sequence_advances_across_a_capacity_growth():
+    """Only one sequence of a batch advances, and its new key no longer fits the index: the step
+    cannot append inside the decode launches and takes the separate path, which must start from
+    the bookkeeping as it stood (the sequence that did not advance has nothing new to index).
+    Counts, codes and the attention of both sequences are checked against the oracle."""
+    dev = _cuda()
+    from pqhsa_release_amd.attention import PQHSAEngine
+
+    H, G, ctx, frac = 2, 2, 1100, 0.03
+    keys, values, q = _problem(dev, batch=2, heads=H, groups=G, ctx=ctx, extra=4)
+    ic, ac = _cfgs(32, frac)
+    eng = PQHSAEngine(ic, ac, batch=2, kv_heads=H, device=dev, growth_margin=0)
+    eng.bind_dense(keys.clone(), values.clone())              # rows beyond a sequence's length are simply not in use yet
+    lens = [ctx, ctx - 40]
+    eng.build(lens)
+    n0 = [eng.n(0), eng.n(1)]
+    assert eng.index.n_cap == n0[0], "the longest sequence fills the index exactly"
+    for step in range(2):                                      # the first step grows the index, the second appends in-launch
+        eng.advance(1, which=[0])
+        lens[0] += 1
+        out = eng.forward(q[:, :, step].reshape(2, H * G, DIM), G)
+        torch.cuda.synchronize()
+        assert eng.index.n_host == [n0[0] + step + 1, n0[1]] and eng.lens == lens
+        tidx, _, _ = eng.last_topk(G)
+        for b in range(2):
+            for h in range(H):
+                n = eng.n(b)
+                ix = _index_of(eng, b * H + h, n)
+                norms, lists, codes = fixed.encode(keys[b, h, 4 : 4 + n].float().cpu().numpy(), ix["coarse"], ix["codebooks"])
+                assert np.array_equal(lists, ix["list_ids"]) and np.array_equal(codes, ix["codes"]), (step, b, h)
+                want_out, want_idx, _ = fixed.decode_step(q[b, h, step].float().cpu().numpy(),
+                                                          keys[b, h, : lens[b]].float().cpu().numpy(),
+                                                          values[b, h, : lens[b]].float().cpu().numpy(), ix, sink=4,
+                                                          local=lens[b] - 4 - n, fraction=frac, scale=SCALE)
+                got = tidx.reshape(2, H, G, -1)[b, h, :, : want_idx.shape[1]].cpu().numpy()
+                for g in range(G):
+                    assert np.array_equal(np.sort(got[g]), np.sort(want_idx[g])), (step, b, h, g)
+                err = np.abs(out[b, h * G : (h + 1) * G].float().cpu().numpy() - want_out).max()
+                assert err <= 2e-3 + 2.0 ** -8 * np.abs(want_out).max(), (step, b, h, err)
+    assert eng.index.n_cap > n0[0]
 
 
 def test_plain_adapter_multi_query_and_state_round_trip():
