@@ -43,15 +43,21 @@ CONFIGS = {
 SINK, LOCAL, FRACTION, LISTS, BLOCK = 4, 64, 0.02, 512, 16
 KERNELS = ["lut_build", "sample_thresh", "scan_emit", "select_final", "attend_partial", "attend_reduce"]
 
-# HBM bytes per launch (read + written) of each kernel, from two rocprofv3 counter runs of this
+# HBM bytes per launch (read + written) of each kernel come from two rocprofv3 counter runs of this
 # script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for a plain
-# 256 MiB device copy (factor 2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE, KiB per dispatch).  Counters
-# cannot be read from inside the timed run, so the figure is carried here per workload; it is
-# reported only for the configuration it was measured on.
-MEASURED_TRAFFIC_BYTES = {
-    2: {"lut_build": 9_637_000, "sample_thresh": 6_699_000, "scan_emit": 69_658_000, "select_final": 14_521_000,
-        "attend_partial": 183_694_000, "attend_reduce": 1_693_000},
-}
+# device copy of known size.  Counters cannot be read from inside the timed run, so the figures
+# are kept in a small JSON file per workload beside the profile summaries, stamped with the git
+# commit of the kernels they were measured on, and are reported together with that stamp.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_step_cfg{cfg}_hbm_traffic.json")
+
+
+def measured_traffic(cfg_id, kernel):
+    try:
+        with open(TRAFFIC_FILE.format(cfg=cfg_id)) as f:
+            rec = json.load(f)
+        return int(rec["bytes_per_launch"][kernel]), rec.get("commit")
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def log(*a):
@@ -256,27 +262,39 @@ def standalone_kernels(layer, reps=20):
     return out
 
 
-def cpu_baseline(layer, seconds=12.0):
-    """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
-    the same inputs and trained index, and scale to the whole layer."""
+def _cpu_stream(layer, b, h):
+    """One (sequence, KV head) stream of the layer on the host, in the form the torch restatement takes."""
     from oracle import torch_ref as tr
     from pqhsa_release_amd import ops
 
-    b = h = 0
-    bh, n, ln, G = 0, layer.n[0], layer.lens[0], layer.G
+    bh, n, ln, G = b * layer.H + h, layer.n[b], layer.lens[b] + layer.t, layer.G
+    n += layer.t
     kk, vv = ops.paged_gather_range(layer.kv, b, 0, ln) if layer.kv.view.paged else (layer.keys[b], layer.values[b])
-    keys, values = kk[h].float().cpu(), vv[h].float().cpu()
+    keys, values = kk[h, :ln].float().cpu(), vv[h, :ln].float().cpu()
     idx = layer.index
     _, lists_by_key, norms_by_key = idx.by_key(bh, n)
     ref = tr.RefIndex(idx.coarse[bh].cpu(), idx.codebooks[bh].cpu(), (lists_by_key.to(torch.int64) & 0xFFFF).cpu(),
                       idx.packed_bytes(bh, n).cpu().clone(), norms_by_key.cpu())
-    vbar = idx.vbar[bh].cpu()
     q = layer.q[b, h * G : (h + 1) * G].float().cpu()
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
-    torch.set_num_threads(cores)
-    args = dict(sink_end=SINK, retrieval_end=SINK + n, index=ref, vbar=vbar, fraction=FRACTION,
+    args = dict(sink_end=SINK, retrieval_end=SINK + n, index=ref, vbar=idx.vbar[bh].cpu(), fraction=FRACTION,
                 scale=1.0 / math.sqrt(128))
+    return q, keys, values, args
+
+
+def host_cores():
+    return min(os.cpu_count() or 1, 16)
+
+
+def cpu_baseline(layer, seconds=12.0):
+    """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
+    the same inputs and trained index, and scale to the whole layer."""
+    from oracle import torch_ref as tr
+
+    b = h = 0
+    n, G = layer.n[0] + layer.t, layer.G
+    q, keys, values, args = _cpu_stream(layer, b, h)
+    cores = host_cores()
+    torch.set_num_threads(cores)
     out = tr.hybrid_forward_many(q, keys, values, **args)
     t0, reps = time.perf_counter(), 0
     while True:
@@ -296,8 +314,8 @@ def cpu_baseline(layer, seconds=12.0):
     torch.set_num_threads(cores)
     got = layer.out[b, h * G : (h + 1) * G].float().cpu()
     err = None if layer.t else float((got - out).abs().max())  # after append steps the device result is for a longer context
-    streams = sum(1 for _ in range(layer.B * layer.H))
-    scale_factor = sum(layer.n) * layer.H / max(n, 1)  # streams weighted by their indexed length
+    streams = layer.B * layer.H
+    scale_factor = sum(layer.n) * layer.H / max(layer.n[0], 1)  # streams weighted by their indexed length
     return {
         "value": per_stream * scale_factor * 1e6,
         "unit": "us/layer",
@@ -309,6 +327,188 @@ def cpu_baseline(layer, seconds=12.0):
         "max_abs_diff_vs_gpu": err,
         "gpu_out_dtype": str(layer.out.dtype).replace("torch.", ""),  # a bf16 output carries 2^-9 relative rounding
     }
+
+
+def cpu_full_layer(layer, reps=3):
+    """The torch-CPU restatement over EVERY stream of the layer, nothing scaled: the layer's
+    time is the sum over its streams (best of ``reps`` passes), and every stream's output is
+    compared with what the GPU wrote for it."""
+    from oracle import torch_ref as tr
+
+    cores = host_cores()
+    torch.set_num_threads(cores)
+    streams = [_cpu_stream(layer, b, h) for b in range(layer.B) for h in range(layer.H)]
+    best, worst = None, 0.0
+    for rep in range(reps + 1):                       # the first pass warms up and checks
+        t0 = time.perf_counter()
+        outs = [tr.hybrid_forward_many(q, k, v, **a) for q, k, v, a in streams]
+        dt = time.perf_counter() - t0
+        if rep == 0:
+            G = layer.G
+            for i, o in enumerate(outs):
+                b, h = divmod(i, layer.H)
+                worst = max(worst, float((layer.out[b, h * G : (h + 1) * G].float().cpu() - o).abs().max()))
+        else:
+            best = dt if best is None else min(best, dt)
+    return {"value": best * 1e6, "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": f"all {len(streams)} streams of the layer, best of {reps} passes",
+            "max_abs_diff_vs_gpu": worst}
+
+
+class Timed:
+    """The resident layers of one configuration and the timing passes over them."""
+
+    def __init__(self, lib, device, cfg_id, *, layers, steps, warmup, appending):
+        self.lib, self.device, self.cfg_id, self.steps, self.warmup = lib, device, cfg_id, steps, warmup
+        self.appending = appending or cfg_id == 4
+        nl = max(1, layers)
+        room = (3 * steps + 4 * warmup + 60 + nl - 1) // nl + 8 if self.appending else 0
+        t0 = time.perf_counter()
+        self.layers = [Layer(cfg_id, 100 + 7919 * i, device, room=room) for i in range(nl)]
+        log(f"setup {time.perf_counter() - t0:.1f}s: {CONFIGS[cfg_id][0]}, {nl} resident layers")
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def run_steps(self, count):
+        for i in range(count):
+            layer = self.layers[i % len(self.layers)]
+            if self.appending:
+                layer.append_step(self.stream)
+            else:
+                layer.call.run(self.stream)
+
+    def logged_run(self, count, only, every=1):
+        """count steps with the HIP-event log on the stream, one step in `every` carrying the
+        records; returns (ms per step, per-kernel ms averaged over the logged steps)."""
+        from pqhsa_release_amd import _lib
+
+        lib = self.lib
+        _lib.check(lib.pqhsa_profile_enable(count), "pqhsa_profile_enable")
+        _lib.check(lib.pqhsa_profile_only(only), "pqhsa_profile_only")
+        _lib.check(lib.pqhsa_profile_every(every), "pqhsa_profile_every")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.run_steps(count)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        kms = (ctypes.c_float * len(KERNELS))()
+        seen = ctypes.c_int32(0)
+        _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
+        assert seen.value == (count + every - 1) // every, (seen.value, count, every)
+        return (t1 - t0) * 1000.0 / count, [float(v) for v in kms]
+
+    def measure(self, event_every):
+        self.run_steps(self.warmup)
+        torch.cuda.synchronize()
+        # untimed survey with every kernel bracketed by events: finds the dominant kernel
+        _, survey = self.logged_run(max(self.warmup, 20), -1)
+        self.survey_us = {name: survey[i] * 1000.0 for i, name in enumerate(KERNELS)}
+        self.dominant_i = max(range(len(KERNELS)), key=lambda i: survey[i])
+        self.dominant = KERNELS[self.dominant_i]
+        # timed region: exactly `steps` steps; the dominant kernel carries two event records on one
+        # step in `event_every`, spread over the whole region: what its roofline figure is measured from
+        self.event_every = max(1, event_every)
+        self.ms_per_step, dom_ms = self.logged_run(self.steps, self.dominant_i, self.event_every)
+        self.dominant_us = dom_ms[self.dominant_i] * 1000.0
+        layer = self.layers[0]
+        ab = self.bytes = layer.algorithmic_bytes()
+        self.algo = {"lut_build": ab["tables"], "sample_thresh": ab["sample"], "scan_emit": ab["scan"],
+                     "select_final": 0, "attend_partial": ab["exact"] + ab["full"], "attend_reduce": ab["bg"]}
+
+    def plain_ms(self):
+        """The same steps with no event at all, to show what the records cost."""
+        self.run_steps(self.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.run_steps(self.steps)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1000.0 / self.steps
+
+    def graph_ms(self):
+        """The same steps replayed from HIP graphs (one per resident layer), or None for steps that
+        append (a captured graph has the key count of its capture in its launch shapes)."""
+        if self.appending:
+            return None
+        for l in self.layers:
+            l.call.capture()
+        for i in range(self.warmup):
+            self.layers[i % len(self.layers)].call.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(self.steps):
+            self.layers[i % len(self.layers)].call.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1000.0 / self.steps
+
+    def roofline(self):
+        nbytes = self.algo[self.dominant]
+        traffic, commit = measured_traffic(self.cfg_id, self.dominant)
+        return {
+            "kernel": self.dominant,
+            "bound": "hbm",
+            "achieved": round(nbytes / 1e3 / self.dominant_us, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(nbytes / 1e3 / self.dominant_us / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "traffic_measured_at_commit": commit,
+            "algorithmic_bytes": nbytes,
+            "launch_us": round(self.dominant_us, 3),
+            "launches_timed": (self.steps + self.event_every - 1) // self.event_every,
+        }
+
+    def kernels(self):
+        out = {}
+        for name in KERNELS:
+            us = self.survey_us[name]
+            out[name] = {"us": round(us, 3), "algo_MB": round(self.algo[name] / 1e6, 3),
+                         "GBps": round(self.algo[name] / 1e3 / us, 1) if us > 0 else None}
+        return out
+
+    def step_frac(self):
+        return round(self.bytes["total"] / 1e3 / (self.ms_per_step * 1000.0) / HBM_PEAK_GBPS, 4)
+
+    def summary(self):
+        """The short per-configuration record of the default run's "configs" object."""
+        r = self.roofline()
+        return {"workload": CONFIGS[self.cfg_id][0], "us_per_layer": round(self.ms_per_step * 1000.0, 3),
+                "steps": self.steps, "resident_layers": len(self.layers), "append_per_step": self.appending,
+                "step_bytes_MB": round(self.bytes["total"] / 1e6, 2), "step_roofline_frac": self.step_frac(),
+                "dominant": {"kernel": r["kernel"], "launch_us": r["launch_us"], "GBps": r["achieved"], "frac": r["frac"]},
+                "kernels_us": {k: round(v, 2) for k, v in self.survey_us.items()},
+                "rescanned_rows": sum(l.ws.rescans() for l in self.layers)}
+
+    def gather_ceiling(self, reps=30):
+        """Rate at which this GPU delivers the very rows the last steps selected (K and V rows of the
+        selected keys of every query row, read through the same addressing as the attention kernel by a
+        kernel that does nothing else), rotating through the resident layers like the timed steps."""
+        from pqhsa_release_amd import ops
+
+        cases = []
+        for l in self.layers:
+            rows = l.B * l.H * l.G
+            idx = l.ws.topk_idx.reshape(rows, -1).clone()
+            cnt = l.ws.topk_cnt.reshape(rows, 1)
+            col = torch.arange(idx.shape[1], device=idx.device).unsqueeze(0)
+            idx = torch.where(col < cnt, idx, idx[:, :1])          # unused tail entries: a valid row again
+            pos = (idx + SINK).reshape(l.B * l.H, -1).to(torch.int32).contiguous()
+            cases.append((l.kv, pos, torch.zeros(ops.PROBE_SLOTS, dtype=torch.int32, device=idx.device)))
+        for kv, pos, checks in cases:
+            ops.gather_probe(kv, pos, checks)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(reps):
+            ops.gather_probe(*cases[i % len(cases)])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1000.0 / reps
+        esz = 4 if self.layers[0].dtype == torch.float32 else 2
+        nbytes = cases[0][1].numel() * 2 * 128 * esz
+        return {"us": round(us, 2), "MB": round(nbytes / 1e6, 2), "GBps": round(nbytes / 1e3 / us, 1)}
+
+    def close(self):
+        self.layers = []
+        torch.cuda.empty_cache()
 
 
 def main():
@@ -330,6 +530,13 @@ def main():
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one device copy of this many MiB after the warm-up (a kernel of known HBM "
                          "traffic, the yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
+    ap.add_argument("--calibrate-gather", action=argparse.BooleanOptionalAction, default=True,
+                    help="time a kernel that only reads the selected K/V rows and report its rate as "
+                         "roofline.random_row_ceiling_GBps (the practical ceiling of the attention kernel)")
+    ap.add_argument("--other-configs", action=argparse.BooleanOptionalAction, default=None,
+                    help="after the main configuration, run short passes over the other configurations and "
+                         "report them under \"configs\" (default: only when --config is the headline one)")
+    ap.add_argument("--other-steps", type=int, default=60)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (every sequence and KV head of the layer is on it); "
@@ -342,104 +549,23 @@ def main():
     lib = _lib.load()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    t_setup = time.perf_counter()
-    appending = args.append or args.config == 4
-    nl = max(1, args.layers)
-    room = (3 * args.steps + 4 * args.warmup + 60 + nl - 1) // nl + 8 if appending else 0
-    layers = [Layer(args.config, 100 + 7919 * i, device, room=room) for i in range(nl)]
-    log(f"setup {time.perf_counter() - t_setup:.1f}s: {CONFIGS[args.config][0]}, {len(layers)} resident layers")
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def run_steps(count, offset=0):
-        for i in range(count):
-            layer = layers[(i + offset) % len(layers)]
-            if appending:
-                layer.append_step(stream)
-            else:
-                layer.call.run(stream)
-
-    run_steps(args.warmup)
-    torch.cuda.synchronize()
+    run = Timed(lib, device, args.config, layers=args.layers, steps=args.steps, warmup=args.warmup, appending=args.append)
     if args.calibrate_copy_mib > 0:
+        run.run_steps(args.warmup)
         src = torch.empty(args.calibrate_copy_mib * 262144, dtype=torch.float32, device=device).normal_()
         dst = torch.empty_like(src)
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    run.measure(args.event_every)
+    ms_per_step = run.ms_per_step
+    ms_plain = run.plain_ms()
+    ms_graph = run.graph_ms()
 
-    def logged_run(count, only, every=1):
-        """count steps with the HIP-event log on the stream, one step in `every` carrying the
-        records; returns (ms per step, per-kernel ms averaged over the logged steps)."""
-        _lib.check(lib.pqhsa_profile_enable(count), "pqhsa_profile_enable")
-        _lib.check(lib.pqhsa_profile_only(only), "pqhsa_profile_only")
-        _lib.check(lib.pqhsa_profile_every(every), "pqhsa_profile_every")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        run_steps(count)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        kms = (ctypes.c_float * len(KERNELS))()
-        seen = ctypes.c_int32(0)
-        _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
-        assert seen.value == (count + every - 1) // every, (seen.value, count, every)
-        return (t1 - t0) * 1000.0 / count, [float(v) for v in kms]
-
-    # untimed survey with every kernel bracketed by events: finds the dominant kernel
-    _, survey = logged_run(max(args.warmup, 20), -1)
-    dominant_i = max(range(len(KERNELS)), key=lambda i: survey[i])
-    dominant = KERNELS[dominant_i]
-    # timed region: exactly --steps steps; the dominant kernel carries two event records on one
-    # step in --event-every, spread over the whole region: what its roofline figure is measured from
-    ms_per_step, dom_ms = logged_run(args.steps, dominant_i, max(1, args.event_every))
-    # the same steps with no event at all, to show what the records cost
-    run_steps(args.warmup)
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    run_steps(args.steps)
-    torch.cuda.synchronize()
-    ms_plain = (time.perf_counter() - t2) * 1000.0 / args.steps
-
-    # the same steps replayed from HIP graphs (one per resident layer): what a serving loop that
-    # captures its steady state would see
-    ms_graph = None
-    if not appending:  # (a captured graph has the key count of its capture baked into its launch shapes)
-        for l in layers:
-            l.call.capture()
-        for i in range(args.warmup):
-            layers[i % len(layers)].call.replay()
-        torch.cuda.synchronize()
-        t3 = time.perf_counter()
-        for i in range(args.steps):
-            layers[i % len(layers)].call.replay()
-        torch.cuda.synchronize()
-        ms_graph = (time.perf_counter() - t3) * 1000.0 / args.steps
-
-    layer = layers[0]
-    ab = layer.algorithmic_bytes()
-    kus = {name: survey[i] * 1000.0 for i, name in enumerate(KERNELS)}
-    algo = {"lut_build": ab["tables"], "sample_thresh": ab["sample"], "scan_emit": ab["scan"],
-            "select_final": 0, "attend_partial": ab["exact"] + ab["full"], "attend_reduce": ab["bg"]}
-    kernels = {}
-    for name in KERNELS:
-        us = kus[name]
-        kernels[name] = {"us": round(us, 3), "algo_MB": round(algo[name] / 1e6, 3),
-                         "GBps": round(algo[name] / 1e3 / us, 1) if us > 0 else None}
-    dom_us = dom_ms[dominant_i] * 1000.0
-    dom_bytes = algo[dominant]
-    roofline = {
-        "kernel": dominant,
-        "bound": "hbm",
-        "achieved": round(dom_bytes / 1e3 / dom_us, 1),
-        "peak": HBM_PEAK_GBPS,
-        "unit": "GB/s",
-        "frac": round(dom_bytes / 1e3 / dom_us / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(args.config, {}).get(dominant),
-        "algorithmic_bytes": dom_bytes,
-        "launch_us": round(dom_us, 3),
-        "launches_timed": (args.steps + max(1, args.event_every) - 1) // max(1, args.event_every),
-    }
-    scan_us = kus["scan_emit"]
+    layer = run.layers[0]
+    ab = run.bytes
+    scan_us = run.survey_us["scan_emit"]
     result = {
         "metric": "decode attn us/layer at 128K ctx (8 KV heads); LUT-scan HBM GB/s vs peak",
         "value": round(ms_per_step * 1000.0, 3),
@@ -456,30 +582,56 @@ def main():
         "config": {"workload": CONFIGS[args.config][0], "batch": layer.B, "kv_heads": layer.H,
                    "gqa_group": layer.G, "context": layer.lens if len(set(layer.lens)) > 1 else layer.lens[0],
                    "num_lists": LISTS, "top_fraction": FRACTION, "sink": SINK, "local_window": LOCAL,
-                   "kv_dtype": str(layer.dtype).replace("torch.", ""), "resident_layers": len(layers)},
-        "roofline": roofline,
+                   "kv_dtype": str(layer.dtype).replace("torch.", ""), "resident_layers": len(run.layers)},
+        "roofline": run.roofline(),
         "tokens_per_s": round(layer.B / (MODEL_LAYERS * ms_per_step / 1000.0), 1),
         "step_bytes_MB": round(ab["total"] / 1e6, 2),
-        "step_roofline_frac": round(ab["total"] / 1e3 / (ms_per_step * 1000.0) / HBM_PEAK_GBPS, 4),
+        "step_roofline_frac": run.step_frac(),
         "lut_scan": {"us": round(scan_us, 3), "algo_MB": round(ab["scan"] / 1e6, 3),
                      "GBps": round(ab["scan"] / 1e3 / scan_us, 1) if scan_us > 0 else None,
                      "frac_of_peak": round(ab["scan"] / 1e3 / scan_us / HBM_PEAK_GBPS, 4) if scan_us > 0 else None},
-        "kernels": kernels,
-        "kernel_sum_us": round(sum(kus.values()), 3),
+        "kernels": run.kernels(),
+        "kernel_sum_us": round(sum(run.survey_us.values()), 3),
         "ms_per_step_without_event_log": round(ms_plain, 6),
         "ms_per_step_graph_replay": None if ms_graph is None else round(ms_graph, 6),
-        "append_per_step": appending,
-        "selection": {"k": math.ceil(layer.n[0] * FRACTION), "rescanned_rows": sum(l.ws.rescans() for l in layers),
+        "append_per_step": run.appending,
+        "selection": {"k": math.ceil(layer.n[0] * FRACTION), "rescanned_rows": sum(l.ws.rescans() for l in run.layers),
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},
+        "decode_workspace_MB": round(layer.ws.bytes / 1e6, 2),
     }
     if args.standalone:
         result["standalone"] = standalone_kernels(layer)
+    if args.calibrate_gather:
+        g = run.gather_ceiling()
+        result["roofline"]["random_row_ceiling_GBps"] = g["GBps"]
+        result["roofline"]["random_row_probe"] = g
+        att = result["kernels"]["attend_partial"]
+        if att["GBps"]:
+            result["roofline"]["attend_frac_of_random_row_ceiling"] = round(att["GBps"] / g["GBps"], 4)
     copy_gbps = copy_bandwidth(device)
     result["hbm_copy_GBps"] = round(copy_gbps, 1)
     result["roofline"]["frac_of_copy"] = round(result["roofline"]["achieved"] / copy_gbps, 4)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(layer, args.cpu_seconds)
+    others = args.other_configs if args.other_configs is not None else args.config == 2
+    if others:
+        del layer
+        run.close()
+        result["configs"] = {}
+        for cfg in (c for c in sorted(CONFIGS) if c != args.config):
+            side = Timed(lib, device, cfg, layers=2, steps=args.other_steps, warmup=10, appending=False)
+            side.measure(args.event_every)
+            rec = side.summary()
+            if not args.no_cpu and cfg in (0, 1) and not side.appending:
+                side.layers[0].call.run(side.stream)           # the output the CPU pass is compared with
+                torch.cuda.synchronize()
+                rec["cpu_baseline"] = cpu_full_layer(side.layers[0])
+                result["cpu_baseline"].setdefault("full_layers", {})[f"cfg{cfg}"] = rec["cpu_baseline"]
+            result["configs"][f"cfg{cfg}"] = rec
+            log(f"cfg{cfg}: {rec['us_per_layer']} us/layer, step roofline {rec['step_roofline_frac']}")
+            side.close()
+            del side
     print(json.dumps(result), flush=True)
 
 

@@ -313,6 +313,20 @@ int pqhsa_paged_gather_at(const pqhsa_kv_view *kv, int32_t H, int32_t seq,
                           void *stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): reads the K and V rows at the given token
+ * positions and folds every 32-bit word read into checksums, nothing else.  positions is i32
+ * [B*H, per_stream] (device); stream (b, h) reads rows positions[b*H + h, :] of sequence b, KV
+ * head h, through the same addressing as the attention kernel.  It shows the rate at which this
+ * GPU delivers scattered 256- or 512-byte rows, the ceiling to hold the exact-attention kernel
+ * against.  checks is u32 [PQHSA_PROBE_SLOTS] (device), zeroed by the caller; the XOR of all its
+ * entries afterwards is the XOR of all words read.  Every position must be a valid token of its
+ * sequence: the kernel does not check them.
+ */
+#define PQHSA_PROBE_SLOTS 4096
+int pqhsa_gather_probe(const pqhsa_kv_view *kv, int32_t B, int32_t H, const int32_t *positions,
+                       int64_t per_stream, uint32_t *checks, void *stream);
+
+/*
  * Per-kernel timing of pqhsa_decode_step with HIP events recorded on the caller's stream and
  * read back only at collect time (the sync-free event log of the reference,
  * benchmarks/cuda_event_log.py:49-88).  pqhsa_profile_enable creates events for up to

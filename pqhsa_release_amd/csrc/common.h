@@ -113,22 +113,6 @@ __device__ inline int64_t row_offset(const KvView &v, int b, int h, int64_t pos)
     return (int64_t)b * v.stride_seq + (int64_t)h * v.stride_head + pos * v.stride_tok;
 }
 
-// ---- the rows every query attends to in full: the sink prefix and the local window ----------------
-// A sequence of `len` cached tokens with n indexed keys: tokens [0, sink_end) and
-// [sink_end + n, len).  `full_max` is the caller's hard upper bound on their number (it sized the
-// row lists); rows beyond it are left out.
-struct FullRows {
-    int sink_end, local_start, count;
-    __device__ inline int64_t position(int i) const { return i < sink_end ? i : local_start + (i - sink_end); }
-};
-__device__ inline FullRows full_rows(int len, int n, int sink, int full_max) {
-    FullRows f;
-    f.sink_end = min(sink, len);
-    f.local_start = f.sink_end + n;
-    f.count = min(f.sink_end + max(len - f.local_start, 0), full_max);
-    return f;
-}
-
 // ---- typed 8-element row slices ---------------------------------------------------------
 // Load elements [8*j, 8*j + 8) of a 128-element row as floats.
 template <int DT>

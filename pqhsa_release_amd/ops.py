@@ -572,3 +572,25 @@ def paged_gather_at(kv: KvSource, seq: int, positions: torch.Tensor):
         _lib.check(rc, "pqhsa_paged_gather_at")
     shape = (*positions.shape, HEAD_DIM)
     return out_k.reshape(shape), out_v.reshape(shape)
+
+
+PROBE_SLOTS = 4096
+
+
+def gather_probe(kv: KvSource, positions: torch.Tensor, checks: torch.Tensor | None = None) -> torch.Tensor:
+    """Read the K and V rows at token ``positions`` (int32 ``[B*H, count]``, every entry a valid token
+    of its sequence) and return the per-workgroup checksums (int32 ``[4096]``; their XOR is the XOR
+    of all 32-bit words read).  A measurement aid: timed, it gives the rate at which the GPU
+    delivers scattered rows of this cache (``pqhsa_gather_probe``)."""
+    _need_cuda(positions)
+    if positions.dtype != torch.int32 or positions.ndim != 2 or positions.shape[0] != kv.batch * kv.kv_heads \
+            or not positions.is_contiguous():
+        raise ValueError("positions must be a contiguous int32 [B*H, count] tensor")
+    if checks is None:
+        checks = torch.zeros(PROBE_SLOTS, dtype=torch.int32, device=positions.device)
+    elif checks.dtype != torch.int32 or checks.numel() != PROBE_SLOTS or not checks.is_cuda:
+        raise ValueError(f"checks must be a device int32 [{PROBE_SLOTS}] tensor")
+    rc = _lib.load().pqhsa_gather_probe(kv.ref(), kv.batch, kv.kv_heads, positions.data_ptr(), positions.shape[1],
+                                        checks.data_ptr(), _stream())
+    _lib.check(rc, "pqhsa_gather_probe")
+    return checks

@@ -376,6 +376,33 @@ def test_decode_step_on_unsorted_and_partly_sorted_layouts():
     assert ws2.rescans() == 0
 
 
+@pytest.mark.parametrize("layout", ["dense", "5d", "4d"])
+def test_gather_probe_reads_the_rows_it_is_given(layout):
+    """The measurement kernel behind the scattered-row ceiling reads exactly the K and V rows at the
+    listed token positions (same addressing as the attention kernel, block table included): the
+    XOR of its checksums equals the XOR of every 32-bit word of those rows."""
+    dev = _cuda()
+    p = Problem(lens=[1500, 900], heads=2, groups=2, lists=16, dtype=torch.bfloat16 if layout != "dense" else torch.float32,
+                seed=43)
+    kv = ops.kv_contiguous(*p.dense_kv()) if layout == "dense" else ops.kv_paged(*p.paged_kv(layout))
+    gen = torch.Generator().manual_seed(7)
+    count = 777
+    pos = torch.stack([torch.randint(0, p.lens[bh // p.H], (count,), generator=gen) for bh in range(p.B * p.H)])
+    checks = ops.gather_probe(kv, pos.to(torch.int32).to(dev))
+    torch.cuda.synchronize()
+    got = 0
+    for x in checks.cpu().numpy().view(np.uint32):
+        got ^= int(x)
+    keys, values = p.dense_kv()
+    want = 0
+    for bh in range(p.B * p.H):
+        b, h = divmod(bh, p.H)
+        for t in (keys, values):
+            words = t[b, h][pos[bh].to(dev)].contiguous().view(torch.int32).cpu().numpy().view(np.uint32)
+            want ^= int(np.bitwise_xor.reduce(words.reshape(-1)))
+    assert got == want
+
+
 def test_hybrid_attend_paged_alone_matches_oracle():
     """The stand-alone attention entry point, fed the oracle's own selection and per-list masses."""
     dev = _cuda()
