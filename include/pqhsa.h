@@ -331,16 +331,16 @@ int pqhsa_gather_probe(const pqhsa_kv_view *kv, int32_t B, int32_t H, const int3
  * read back only at collect time (the sync-free event log of the reference,
  * benchmarks/cuda_event_log.py:49-88).  pqhsa_profile_enable creates events for up to
  * max_steps decode steps; pqhsa_profile_collect synchronises the recorded events, writes the
- * average milliseconds of the 6 kernels (lut_build, sample_thresh, scan_emit, select_final,
- * attend_partial, attend_reduce) and the number of steps seen, and turns profiling off.
+ * average milliseconds of the 5 kernels (lut_build, sample_thresh, scan_emit, select_final,
+ * attend) and the number of steps seen, and turns profiling off.
  * pqhsa_profile_only(kernel), called after enable, restricts the log to the two events around
  * one kernel (-1: all), so that a timed run carries two event records per step instead of
- * seven; the other entries of kernel_ms are then 0.  pqhsa_profile_every(stride), also after
+ * six; the other entries of kernel_ms are then 0.  pqhsa_profile_every(stride), also after
  * enable, logs one decode step in `stride` (the first, then every stride-th): a timed run then
  * carries the event records on a sample of its steps only, and `steps` counts the logged ones.
  * Not thread-safe; meant for benchmarks.
  */
-#define PQHSA_PROFILE_KERNELS 6
+#define PQHSA_PROFILE_KERNELS 5
 int pqhsa_profile_enable(int32_t max_steps);
 int pqhsa_profile_only(int32_t kernel);
 int pqhsa_profile_every(int32_t stride);

@@ -8,8 +8,9 @@
 // exp(logit - chunk max) * V in fp32.  It also takes a slice of the IVF lists and multiplies
 // their background masses with the lists' mean values, so the mean-value table is read once
 // per query row, spread over all splits.
-// attend_reduce_kernel: grid (G, BH).  Folds the split partials under the final row maximum,
-// rescales the two background parts from their reference logits, and normalises.
+// The workgroup of a query row that finishes last folds the row's split partials under the final
+// row maximum, rescales the background from its reference logit, normalises and writes the
+// output row (fold_row_if_last): the step needs no further launch.
 #include <cfloat>
 
 #include "common.h"
@@ -19,7 +20,7 @@ namespace pqhsa {
 constexpr int kAttThreads = 256;
 constexpr int kGroupLanes = 16;                     // lanes per K/V row
 constexpr int kGroups = kAttThreads / kGroupLanes;  // rows in flight per pass
-constexpr int kPartWidth = 4 + 3 * kD;              // m, l, mass0, mass1, acc[128], bg0[128], bg1[128]
+constexpr int kPartWidth = 4 + 2 * kD;              // m, l, list-mass sum, (unused), acc[128], background[128]
 constexpr int kMaxChunk = 2048;
 constexpr int kMaxSplits = 64;
 
@@ -39,11 +40,12 @@ struct AttendArgs {
     float scale;
     int splits;
     float *partials;          // [BH*G, splits, kPartWidth]
-    // background: two per-list mass tables, element (bh, l, g) at bh*mass_bh + l*mass_l + g*mass_g,
-    // each relative to its own reference logit ref[bh*ref_stride + g]
-    const float *mass0, *mass1;
+    uint32_t *arrive;         // [BH*G] workgroups of a query row that have stored their partial; zero at launch
+    // background: per-list mass table, element (bh, l, g) at bh*mass_bh + l*mass_l + g*mass_g,
+    // relative to the reference logit ref[bh*ref_stride + g]
+    const float *mass0;
     int64_t mass_bh, mass_l, mass_g;
-    const float *ref0, *ref1;
+    const float *ref0;
     int ref_stride;
     const float *vbar;        // [BH, L, 128]
     int L;
@@ -99,14 +101,101 @@ struct RawSlice {
     }
 };
 
+PQHSA_TRACE_DECL(trace_attend)
+// Folding the partials of one query row: run by the workgroup of the row that stores its partial
+// last.  Partials are written and read with device-scope accesses (publish / peek: they go past
+// the caches that are private to a part of the chip), every workgroup waits for its stores to
+// complete and then takes a ticket from the row's arrival counter; the one that draws the last
+// ticket folds all partials under the row's maximum, with the background term, into the output
+// row.  No cache-wide write-back or invalidation is needed this way (a device-scope fence per
+// workgroup made the kernel several times slower).  The counter is back at zero when the kernel
+// ends.
+constexpr int kFoldLanes = kAttThreads / kD;  // splits folded side by side
+
+__device__ inline void publish(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline float peek(const float *p) {
+    return __hip_atomic_load(const_cast<float *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int QDT>
+__device__ inline void fold_row_if_last(const AttendArgs &a, size_t orow, int b, int h, int g, int bh) {
+    __shared__ int last_s;
+    __shared__ float head_s[2];                 // row maximum, sum of the background list masses
+    __shared__ float acc_s[kFoldLanes][kD];
+    __shared__ float den_s[kFoldLanes];
+    const int tid = threadIdx.x;
+    __builtin_amdgcn_s_waitcnt(0);  // this thread's stores of the partial have completed before the ticket is drawn
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t ticket = atomicAdd(&a.arrive[orow], 1u);
+        last_s = ticket + 1u == (uint32_t)a.splits;
+        if (last_s) a.arrive[orow] = 0u;
+    }
+    __syncthreads();
+    if (!last_s) return;
+    const int d = tid & (kD - 1), sl = tid / kD;
+    const int n = a.n_idx[b];
+    if (a.n_commit_dst && g == 0 && h == 0 && tid == 0) a.n_commit_dst[b] = a.n_commit_src[b];
+    const float *part = a.partials + orow * a.splits * kPartWidth;
+    const float r0 = (n > 0 && a.mass0) ? a.ref0[(size_t)bh * a.ref_stride + g] : -INFINITY;
+    // the first wave takes one split per lane (at most 64 splits): maximum and mass sum
+    if (tid < kWave) {
+        float m = -INFINITY, ms0 = 0.0f;
+        if (tid < a.splits) {
+            m = peek(part + tid * kPartWidth);
+            ms0 = peek(part + tid * kPartWidth + 2);
+        }
+        m = wave_max(m);
+        ms0 = wave_sum(ms0);
+        if (tid == 0) { head_s[0] = m; head_s[1] = ms0; }
+    }
+    __syncthreads();
+    float m = head_s[0];
+    const float ms0 = head_s[1];
+    // the background only matters (and only bounds the maximum) when it holds any weight
+    if (ms0 != 0.0f && r0 > -INFINITY) m = fmaxf(m, r0);
+    const size_t qesz = QDT == PQHSA_F32 ? 4 : 2;
+    char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
+    if (m == -INFINITY) {  // nothing to attend to
+        if (sl == 0) store1<QDT>(orow_p, d, 0.0f);
+        return;
+    }
+    const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
+    float acc = 0.0f, den = 0.0f;
+#pragma unroll 4
+    for (int s = sl; s < a.splits; s += kFoldLanes) {  // independent loads: several splits in flight at once
+        const float *p = part + s * kPartWidth;
+        const float pm = peek(p);
+        const float w = pm == -INFINITY ? 0.0f : __expf(pm - m);
+        den = __builtin_fmaf(peek(p + 1), w, den);
+        acc = __builtin_fmaf(peek(p + 4 + d), w, acc);
+        acc = __builtin_fmaf(peek(p + 4 + kD + d), f0, acc);
+    }
+    acc_s[sl][d] = acc;
+    if (d == 0) den_s[sl] = den;
+    __syncthreads();
+    if (sl != 0) return;
+#pragma unroll
+    for (int r = 1; r < kFoldLanes; ++r) {
+        acc += acc_s[r][d];
+        den += den_s[r];
+    }
+    den += ms0 * f0;
+    den = fmaxf(den, FLT_MIN);
+    store1<QDT>(orow_p, d, acc / den);
+}
+
+
 template <int KDT, int QDT>
 __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs a) {
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z);
+    PQHSA_TRACE_MARK(trace_attend, trace_wg, 0);
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[kGroups][kD];
     __shared__ float red_m[kGroups];
     __shared__ float red_l[kGroups];
-    __shared__ __align__(16) float bg_s[2][kAttThreads / (kD / 4)][kD];
-    __shared__ float ms_s[2][kAttThreads / (kD / 4)];
+    __shared__ __align__(16) float bg_s[kAttThreads / (kD / 4)][kD];
+    __shared__ float ms_s[kAttThreads / (kD / 4)];
     const int tid = threadIdx.x;
     const int split = blockIdx.x, g = blockIdx.y, bh = blockIdx.z;
     const int b = bh / a.H, h = bh % a.H;
@@ -152,20 +241,17 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     const int bl = tid / kBgLanes, bd = (tid % kBgLanes) * 4;
     const float *vb = a.vbar + (size_t)bh * a.L * kD;
     const float *m0 = a.mass0 ? a.mass0 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
-    const float *m1 = a.mass1 ? a.mass1 + (size_t)bh * a.mass_bh + (size_t)g * a.mass_g : nullptr;
     float4 bv[kBgU];
-    float bw0[kBgU], bw1[kBgU];
+    float bw0[kBgU];
     auto bg_fetch = [&](int first) {
 #pragma unroll
         for (int u = 0; u < kBgU; ++u) {
             const int l = first + bl + u * kBgRows;
             bv[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             bw0[u] = 0.0f;
-            bw1[u] = 0.0f;
             if (l < l_hi) {
                 bv[u] = *reinterpret_cast<const float4 *>(vb + (size_t)l * kD + bd);
                 if (m0) bw0[u] = m0[(size_t)l * a.mass_l];
-                if (m1) bw1[u] = m1[(size_t)l * a.mass_l];
             }
         }
     };
@@ -226,43 +312,38 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
 
     // ---- background arithmetic, while the first K/V rows are on their way ---------------------
     {
-        float4 b0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), b1 = b0;
-        float s0 = 0.0f, s1 = 0.0f;
+        float4 b0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float s0 = 0.0f;
         for (int first = l_lo; first < l_hi; first += kBgU * kBgRows) {
             if (first != l_lo) bg_fetch(first);
 #pragma unroll
             for (int u = 0; u < kBgU; ++u) {
                 b0.x = __builtin_fmaf(bw0[u], bv[u].x, b0.x); b0.y = __builtin_fmaf(bw0[u], bv[u].y, b0.y);
                 b0.z = __builtin_fmaf(bw0[u], bv[u].z, b0.z); b0.w = __builtin_fmaf(bw0[u], bv[u].w, b0.w);
-                b1.x = __builtin_fmaf(bw1[u], bv[u].x, b1.x); b1.y = __builtin_fmaf(bw1[u], bv[u].y, b1.y);
-                b1.z = __builtin_fmaf(bw1[u], bv[u].z, b1.z); b1.w = __builtin_fmaf(bw1[u], bv[u].w, b1.w);
                 s0 += bw0[u];
-                s1 += bw1[u];
             }
         }
-        *reinterpret_cast<float4 *>(&bg_s[0][bl][bd]) = b0;
-        *reinterpret_cast<float4 *>(&bg_s[1][bl][bd]) = b1;
-        if (bd == 0) { ms_s[0][bl] = s0; ms_s[1][bl] = s1; }
+        *reinterpret_cast<float4 *>(&bg_s[bl][bd]) = b0;
+        if (bd == 0) ms_s[bl] = s0;
         __syncthreads();
         if (tid < kD) {
-            float t0 = 0.0f, t1 = 0.0f;
+            float t0 = 0.0f;
 #pragma unroll
-            for (int r = 0; r < kBgRows; ++r) { t0 += bg_s[0][r][tid]; t1 += bg_s[1][r][tid]; }
-            part[4 + kD + tid] = t0;
-            part[4 + 2 * kD + tid] = t1;
+            for (int r = 0; r < kBgRows; ++r) t0 += bg_s[r][tid];
+            publish(part + 4 + kD + tid, t0);
         }
         if (tid == 0) {
-            float t0 = 0.0f, t1 = 0.0f;
+            float t0 = 0.0f;
 #pragma unroll
-            for (int r = 0; r < kBgRows; ++r) { t0 += ms_s[0][r]; t1 += ms_s[1][r]; }
-            part[2] = t0;
-            part[3] = t1;
+            for (int r = 0; r < kBgRows; ++r) t0 += ms_s[r];
+            publish(part + 2, t0);
         }
     }
 
     if (cnt <= 0) {
-        if (tid == 0) { part[0] = -INFINITY; part[1] = 0.0f; }
-        if (tid < kD) part[4 + tid] = 0.0f;
+        if (tid == 0) { publish(part, -INFINITY); publish(part + 1, 0.0f); }
+        if (tid < kD) publish(part + 4 + tid, 0.0f);
+        fold_row_if_last<QDT>(a, orow, b, h, g, bh);
         return;
     }
 
@@ -326,83 +407,18 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         float s = 0.0f;
 #pragma unroll
         for (int r = 0; r < kGroups; ++r) s += red[r][tid];
-        part[4 + tid] = s;
+        publish(part + 4 + tid, s);
     }
     if (tid == 0) {
         float l = 0.0f;
 #pragma unroll
         for (int r = 0; r < kGroups; ++r) l += red_l[r];
-        part[0] = m;
-        part[1] = l;
+        publish(part, m);
+        publish(part + 1, l);
     }
-}
-
-constexpr int kRedLanes = 4;  // split partials are folded four at a time (512 threads)
-
-template <int QDT>
-__global__ __launch_bounds__(kD * kRedLanes) void attend_reduce_kernel(AttendArgs a) {
-    __shared__ float head_s[3];                 // row maximum, mass sums of the two background parts
-    __shared__ float acc_s[kRedLanes][kD];
-    __shared__ float den_s[kRedLanes];
-    const int tid = threadIdx.x;
-    const int d = tid & (kD - 1), sl = tid / kD;
-    const int g = blockIdx.x, bh = blockIdx.y;
-    const int b = bh / a.H, h = bh % a.H;
-    const size_t orow = (size_t)bh * a.G + g;
-    const int n = a.n_idx[b];
-    if (a.n_commit_dst && g == 0 && h == 0 && tid == 0) a.n_commit_dst[b] = a.n_commit_src[b];
-    const float *part = a.partials + orow * a.splits * kPartWidth;
-    const float r0 = (n > 0 && a.mass0) ? a.ref0[(size_t)bh * a.ref_stride + g] : -INFINITY;
-    const float r1 = (n > 0 && a.mass1) ? a.ref1[(size_t)bh * a.ref_stride + g] : -INFINITY;
-    // the first wave takes one split per lane (at most 64 splits): maximum and mass sums
-    if (tid < kWave) {
-        float m = -INFINITY, ms0 = 0.0f, ms1 = 0.0f;
-        if (tid < a.splits) {
-            m = part[tid * kPartWidth];
-            ms0 = part[tid * kPartWidth + 2];
-            ms1 = part[tid * kPartWidth + 3];
-        }
-        m = wave_max(m);
-        ms0 = wave_sum(ms0);
-        ms1 = wave_sum(ms1);
-        if (tid == 0) { head_s[0] = m; head_s[1] = ms0; head_s[2] = ms1; }
-    }
-    __syncthreads();
-    float m = head_s[0];
-    const float ms0 = head_s[1], ms1 = head_s[2];
-    // a background part only matters (and only bounds the maximum) when it holds any weight
-    if (ms0 != 0.0f && r0 > -INFINITY) m = fmaxf(m, r0);
-    if (ms1 != 0.0f && r1 > -INFINITY) m = fmaxf(m, r1);
-    const size_t qesz = QDT == PQHSA_F32 ? 4 : 2;
-    char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
-    if (m == -INFINITY) {  // nothing to attend to
-        if (sl == 0) store1<QDT>(orow_p, d, 0.0f);
-        return;
-    }
-    const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
-    const float f1 = (ms1 != 0.0f && r1 > -INFINITY) ? __expf(r1 - m) : 0.0f;
-    float acc = 0.0f, den = 0.0f;
-#pragma unroll 4
-    for (int s = sl; s < a.splits; s += kRedLanes) {  // independent loads: several splits in flight at once
-        const float *p = part + s * kPartWidth;
-        const float w = p[0] == -INFINITY ? 0.0f : __expf(p[0] - m);
-        den = __builtin_fmaf(p[1], w, den);
-        acc = __builtin_fmaf(p[4 + d], w, acc);
-        acc = __builtin_fmaf(p[4 + kD + d], f0, acc);
-        acc = __builtin_fmaf(p[4 + 2 * kD + d], f1, acc);
-    }
-    acc_s[sl][d] = acc;
-    if (d == 0) den_s[sl] = den;
-    __syncthreads();
-    if (sl != 0) return;
-#pragma unroll
-    for (int r = 1; r < kRedLanes; ++r) {
-        acc += acc_s[r][d];
-        den += den_s[r];
-    }
-    den += ms0 * f0 + ms1 * f1;
-    den = fmaxf(den, FLT_MIN);
-    store1<QDT>(orow_p, d, acc / den);
+    PQHSA_TRACE_MARK(trace_attend, trace_wg, 1);
+    fold_row_if_last<QDT>(a, orow, b, h, g, bh);
+    PQHSA_TRACE_MARK(trace_attend, trace_wg, 2);
 }
 
 // Stand-alone form only: the caller's masses cover every indexed key of the row, so the
@@ -411,12 +427,14 @@ __global__ __launch_bounds__(kAttThreads) void subtract_selected_kernel(const fl
                                                                         const int32_t *topk_idx, const float *topk_val,
                                                                         const int32_t *topk_cnt, int64_t k_cap,
                                                                         const uint16_t *key_lists, int64_t key_stride,
-                                                                        int G, int L, float *mass_adj) {
+                                                                        int G, int L, float *mass_adj,
+                                                                        uint32_t *arrive) {
     extern __shared__ __align__(16) unsigned char smem[];
     float *ms = reinterpret_cast<float *>(smem);
     const int tid = threadIdx.x;
     const int g = blockIdx.x, bh = blockIdx.y;
     const size_t orow = (size_t)bh * G + g;
+    if (tid == 0) arrive[orow] = 0u;  // the attention launch that follows counts its workgroups per row from zero
     for (int l = tid; l < L; l += kAttThreads) ms[l] = list_mass[orow * L + l];
     __syncthreads();
     const float rm = row_max[orow];
@@ -453,6 +471,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     if (BH == 0) return PQHSA_OK;
     PQHSA_REQUIRE(a.G >= 1 && a.G <= 16, "attend: G=%d outside [1, 16]", a.G);
     PQHSA_REQUIRE(a.L <= 4096, "attend: num_lists=%d too large", a.L);
+    PQHSA_REQUIRE(a.arrive != nullptr, "attend: no arrival counters");
     a.splits = min(pick_splits(BH * a.G, rows_max), splits_room(BH * a.G, (int)a.k_cap));
     a.full_guess = rows_max > (int)a.k_cap ? rows_max - (int)a.k_cap : 0;
     const int chunk = (rows_max + a.splits - 1) / a.splits;
@@ -484,26 +503,24 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
         return PQHSA_EINVAL;
     }
 #undef PQHSA_ATT
-    int rc = check_launch("attend_partial");
-    if (rc) return rc;
-    if (mark) profile_mark(kProfReduce, stream);
-    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(attend_reduce_kernel<DT>, dim3(a.G, BH), dim3(kD * kRedLanes), 0, stream, a));
     if (mark) profile_mark(kProfKernels, stream);
-    return check_launch("attend_reduce");
+    return check_launch("attend");
 }
 
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
-                  float *partials, const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream) {
+                  float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
+                  hipStream_t stream) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
     a.topk_idx = topk_idx; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
     a.partials = partials;
+    a.arrive = arrive;
     const int64_t L = index->num_lists;
-    a.mass0 = mass; a.mass1 = nullptr; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
-    a.ref0 = ref_val; a.ref1 = nullptr; a.ref_stride = GP;
+    a.mass0 = mass; a.mass_bh = L * GP; a.mass_l = GP; a.mass_g = 1;
+    a.ref0 = ref_val; a.ref_stride = GP;
     a.vbar = index->vbar; a.L = index->num_lists;
     a.n_commit_src = n_commit_src; a.n_commit_dst = n_commit_dst;
     return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream);
@@ -514,7 +531,8 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
 using namespace pqhsa;
 
 extern "C" size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t num_lists) {
-    return attend_partials_bytes(B * H * G, 1 << 20) + (size_t)B * H * G * num_lists * sizeof(float) + 512;
+    return attend_partials_bytes(B * H * G, 1 << 20) + (size_t)B * H * G * num_lists * sizeof(float) +
+           (size_t)B * H * G * sizeof(uint32_t) + 1024;
 }
 
 extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
@@ -537,9 +555,11 @@ extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *o
     char *w = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
     float *partials = reinterpret_cast<float *>(w);
     float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G, 1 << 20));
+    uint32_t *arrive = reinterpret_cast<uint32_t *>(
+        (reinterpret_cast<uintptr_t>(mass_adj + (size_t)BH * G * L) + 255) & ~(uintptr_t)255);
     hipLaunchKernelGGL(subtract_selected_kernel, dim3(G, BH), dim3(kAttThreads), (size_t)L * sizeof(float), stream,
                        list_mass, row_max, topk_idx, topk_val, topk_cnt, (int64_t)k_cap, key_lists, key_list_stride, G,
-                       L, mass_adj);
+                       L, mass_adj, arrive);
     rc = check_launch("subtract_selected");
     if (rc) return rc;
     AttendArgs a = {};
@@ -547,8 +567,9 @@ extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *o
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
     a.topk_idx = topk_idx; a.topk_cnt = topk_cnt; a.k_cap = k_cap; a.scale = scale;
     a.partials = partials;
-    a.mass0 = mass_adj; a.mass1 = nullptr; a.mass_bh = (int64_t)G * L; a.mass_l = 1; a.mass_g = L;
-    a.ref0 = row_max; a.ref1 = nullptr; a.ref_stride = G;
+    a.arrive = arrive;
+    a.mass0 = mass_adj; a.mass_bh = (int64_t)G * L; a.mass_l = 1; a.mass_g = L;
+    a.ref0 = row_max; a.ref_stride = G;
     a.vbar = index->vbar; a.L = L;
     return launch_attend(a, q_dtype, kv->dtype, BH, full_max + k_cap, false, stream);
 }

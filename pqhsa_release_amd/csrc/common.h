@@ -24,7 +24,7 @@ int check_launch(const char *what);
 int launch_fill_zero(void *p, size_t bytes, hipStream_t stream);  // clears with a kernel (graph-capturable)
 // Records the next profiling event on `stream` when profiling is enabled (no-op otherwise).
 void profile_mark(int slot, hipStream_t stream);
-enum { kProfLut = 0, kProfSample, kProfEmit, kProfSelect, kProfAttend, kProfReduce, kProfKernels };
+enum { kProfLut = 0, kProfSample, kProfEmit, kProfSelect, kProfAttend, kProfKernels };
 
 #define PQHSA_REQUIRE(cond, ...)            \
     do {                                    \

@@ -29,14 +29,15 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
-                  float *partials, const int32_t *n_commit_src, int32_t *n_commit_dst, hipStream_t stream);
+                  float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
+                  hipStream_t stream);
 size_t attend_partials_bytes(int rows, int k_cap);
 
 static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Carve {
     float *qnorm, *lut, *ls;
-    uint32_t *emit_count, *rescans;
+    uint32_t *emit_count, *rescans, *arrive;
     float *mass;
     size_t zero_words;
     uint32_t *thr_key;
@@ -68,6 +69,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
     const size_t z0 = off;  // everything from here to zero_words is cleared at the start of a step
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
+    c.arrive = reinterpret_cast<uint32_t *>(take(BH * G * 4));  // attention workgroups arrived per query row
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
     c.qnorm = reinterpret_cast<float *>(take(rows * 4));
@@ -174,7 +176,7 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
                             topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
-                         topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials,
+                         topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials, c.arrive,
                          append_count ? c.n_after : nullptr,
                          append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
 }

@@ -817,7 +817,7 @@ def test_event_log_counts_steps_and_samples_them():
                             fraction=0.02, topk=0, scale=SCALE, workspace=ws)
 
     def collect():
-        kms = (ctypes.c_float * 6)()
+        kms = (ctypes.c_float * 5)()
         seen = ctypes.c_int32(-1)
         _lib.check(lib.pqhsa_profile_collect(kms, ctypes.byref(seen)), "pqhsa_profile_collect")
         return seen.value, [float(v) for v in kms]
