@@ -643,6 +643,9 @@ struct SampleArgs {
     AppendFinish append;       // count != NULL: one more workgroup per stream completes the step's append
 };
 
+// Standard deviations of the sampling noise by which the expected number of keys above the
+// threshold exceeds k.
+constexpr double kMarginSigmas = 5.0;
 constexpr int kSampleRegsMax = 32;  // sampled keys per thread: at most 32768 per row
 
 // R sampled keys per thread (s_cap <= R * 1024, chosen by the host).  The sampled keys are
@@ -700,7 +703,7 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
     const int k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
     // expected sampled keys among the top max(k, 1), plus the margin
     const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
-    const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
+    const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
     const double want_d = ceil(x * x) + 1.0;
     if (ns <= 0 || want_d >= (double)ns) {
         // sample too small to say anything: every key is a candidate and no background sum is formed
@@ -1462,7 +1465,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
         const double ns = (double)(index->s_cap < n_max ? index->s_cap : n_max);
         const int kmax = resolve_k((int)n_max, select->fraction, select->topk);
         const double ks = (double)(kmax > 1 ? kmax : 1) * ns / (double)(n_max > 1 ? n_max : 1);
-        const double x = 0.5 * (7.0 + sqrt(49.0 + 4.0 * ks));
+        const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
         s.expected_candidates = (int64_t)((ceil(x * x) + 1.0) * 1.125 * ((double)n_max / (ns > 1.0 ? ns : 1.0)) * 1.12) + 64;
     }
     rc = launch_select_final(s, streams, stream);
