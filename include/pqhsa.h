@@ -109,7 +109,14 @@ typedef struct pqhsa_select {
     double fraction;
     int32_t topk;
     int32_t k_cap; /* row stride of topk_idx / topk_val; >= the largest k of the batch */
+    int32_t flags; /* 0, or PQHSA_SELECT_GENERAL_PATH */
+    int32_t reserved;
 } pqhsa_select;
+
+/* pqhsa_decode_step serves short contexts (at most 16 384 indexed keys per sequence, at most 256
+ * query rows in the batch, no append in the step) with one kernel, one workgroup per query row;
+ * the results are the same.  This flag keeps such a step on the general five-kernel path. */
+#define PQHSA_SELECT_GENERAL_PATH 1
 
 const char *pqhsa_version(void);
 const char *pqhsa_last_error(void);

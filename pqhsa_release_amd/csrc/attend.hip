@@ -54,15 +54,6 @@ struct AttendArgs {
     int32_t *n_commit_dst;        // [B]
 };
 
-// sum over the 16 lanes of a row group (one DPP row), returned in each of them
-__device__ inline float group_sum16(float v) {
-    v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));
-    v += __int_as_float(dpp_move<kDppXor2>(__float_as_int(v)));
-    v += __int_as_float(dpp_move<kDppHalfMirror>(__float_as_int(v)));
-    v += __int_as_float(dpp_move<kDppMirror>(__float_as_int(v)));
-    return v;
-}
-
 // One lane's 8 elements of a 128-element row as loaded (16 bytes for 2-byte types, 32 for fp32),
 // converted to floats only when the row is used: a row in flight costs 4 (or 8) registers.
 template <int DT>

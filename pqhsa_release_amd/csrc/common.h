@@ -240,6 +240,15 @@ constexpr int kDppBcast31 = 0x143;     // lane 31 to rows 2 and 3
 constexpr int kDppWaveShl1 = 0x130;    // lane i reads lane i+1 of the wave (0 for the last lane)
 constexpr int kDppWaveShr1 = 0x138;    // lane i reads lane i-1 of the wave (0 for lane 0)
 
+// sum over the 16 lanes of a row group (one DPP row), returned in each of them
+__device__ inline float group_sum16(float v) {
+    v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppXor2>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppHalfMirror>(__float_as_int(v)));
+    v += __int_as_float(dpp_move<kDppMirror>(__float_as_int(v)));
+    return v;
+}
+
 // sum over the wave, returned in every lane (the order of the additions differs from wave_sum)
 __device__ inline float wave_total(float v) {
     v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));

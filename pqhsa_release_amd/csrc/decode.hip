@@ -26,6 +26,11 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        void *pairs, uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                        const AppendFinish *append, hipStream_t stream);
+bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap);
+int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
+                 const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const pqhsa_select *select, float scale,
+                 float eps, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, uint32_t *emit_count,
+                 hipStream_t stream);
 int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
@@ -148,6 +153,12 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     if (!topk_idx) topk_idx = c.topk_idx;
     if (!topk_val) topk_val = c.topk_val;
     if (!topk_cnt) topk_cnt = c.topk_cnt;
+
+    // Short contexts without an append: one launch, one workgroup per query row.
+    if (!append_count && !(select->flags & PQHSA_SELECT_GENERAL_PATH) &&
+        decode_small_fits(index->batch * index->kv_heads, G, n_max, index->num_lists, select->k_cap))
+        return decode_small(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, n_max, full_max + select->k_cap, select,
+                            scale, eps, topk_idx, topk_val, topk_cnt, c.emit_count, stream);
 
     // with an append, the first launch also encodes the new keys and publishes the new counts;
     // every later kernel of the step reads those, and the last one stores them into the index

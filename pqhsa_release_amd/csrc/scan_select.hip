@@ -23,6 +23,8 @@
 // (one barrier per bit) for inputs the histogram does not resolve: a crowded range, or a wanted
 // rank outside the sampled window.  A row whose estimate kept fewer than k candidates is
 // re-scanned in full by its select workgroup, so the result is always the exact top-k.
+#include <cfloat>
+
 #include "common.h"
 #include "encode_row.h"
 #include "scan_common.h"
@@ -31,6 +33,7 @@ namespace pqhsa {
 
 PQHSA_TRACE_DECL(trace_sample)
 PQHSA_TRACE_DECL(trace_select)
+PQHSA_TRACE_DECL(trace_small)
 
 template <int GP, int MODE, int SRC>
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(ScanArgs a) {
@@ -823,11 +826,14 @@ struct SelectOut {
     uint32_t k_cap;
     float *mx;               // LDS [L] (NULL: no background)
     float ref1;              // reference of the losers' weights: the k-th logit
+    int32_t *lds_idx = nullptr;  // LDS copy of the selected indices, for a kernel that goes on to use them (room lds_cap)
+    uint32_t lds_cap = 0u;
     __device__ inline void winner(uint32_t at, uint32_t key, uint32_t where) const {
         if (at < k_cap) {
             out_idx[at] = (int32_t)where;
             if (out_val) out_val[at] = key_to_float(key);
         }
+        if (at < lds_cap) lds_idx[at] = (int32_t)where;
     }
     __device__ inline void loser(uint32_t key, uint32_t list) const {
         if (mx) atomicAdd(&mx[list], __expf(key_to_float(key) - ref1));
@@ -840,7 +846,7 @@ template <int R>
 __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
                                      int k, SelectOut out, uint32_t (*red)[kSelWaves],
                                      uint32_t *wsum, SelScratch *ss, float *ref1_out, uint32_t lo_hint = 0u,
-                                     uint32_t hi_hint = 0u) {
+                                     uint32_t hi_hint = 0u, bool lo_exact = false) {
     const int tid = threadIdx.x;
     int step = 0;
     bool exact = false;
@@ -858,7 +864,10 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         // With a hint of where the keys lie (the threshold they passed, the largest sampled key and
         // an eighth of the span on top) the smallest and largest key need not be found first.
         // Keys outside the hinted span fall into the first or last range, which keeps the ranges
-        // in key order, so the selection stays exact whatever the hint.
+        // in key order, so the selection stays exact whatever the hint.  A caller that KNOWS the
+        // k-th largest key to lie above lo_hint (lo_exact) has the keys at or below it left out of
+        // the histogram: they cannot be selected, and thousands of them in one range would
+        // serialise on its counter.
         if (hinted) {
             const uint32_t span = hi_hint - lo_hint;
             lo_key = lo_hint;
@@ -871,9 +880,9 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
         uint32_t bucket[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            bucket[r] = key[r] == 0u ? 0xffffffffu
+            bucket[r] = (key[r] == 0u || (lo_exact && hinted && key[r] <= lo_key)) ? 0xffffffffu
                         : key[r] <= lo_key ? 0u : min((key[r] - lo_key) >> shift, (uint32_t)kSelBins - 1u);
-            if (key[r] != 0u) atomicAdd(&ss->hist[bucket[r]], 1u);
+            if (bucket[r] != 0xffffffffu) atomicAdd(&ss->hist[bucket[r]], 1u);
         }
         if (tid == 0) ss->bin = 0xffffffffu;
         __syncthreads();
@@ -1414,6 +1423,429 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     else if (a.expected_candidates <= 16 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<16>, grid, block, lds, stream, a);
     else hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
     return check_launch("select_final");
+}
+
+// ---- short contexts: the whole step of one query row in one workgroup ---------------------------
+// With a few thousand keys per stream the five launches of the general path cost more in launch
+// and memory round trips than in work.  Here one 1024-thread workgroup per query row does it
+// all: the row's tables (the same fused multiply-add chains as the table-building kernel, the
+// coarse centroids staged through LDS in tiles of 256 lists), the logits of every stored key
+// (up to R per thread, kept in registers), the exact top-k among them with the selection
+// routine of the general path (the losers' weights go to per-list sums in LDS, relative to the
+// k-th logit), and the attention over sink, window and selected rows merged with the per-list
+// background.  Results are those of the general path: same logits bit for bit, same selection
+// rule, same softmax terms.
+constexpr int kSmallTile = 256;
+constexpr int kSmallRow = kD + 4;  // floats per staged centroid row
+
+struct SmallArgs {
+    const char *q;
+    char *out;
+    int q_dtype;
+    KvView kv;
+    int H, G, GP;
+    const int32_t *seq_lens;  // [B]
+    const int32_t *n_arr;     // [B]
+    int sink;
+    const uint32_t *codes;
+    const uint16_t *list_ids;
+    const float *norms;
+    const int32_t *pos;
+    int64_t n_cap;
+    const float *coarse, *codebooks, *vbar;
+    int L;
+    float eps, scale;
+    double fraction;
+    int topk;
+    int32_t *topk_idx;
+    float *topk_val;
+    int32_t *topk_cnt;
+    int k_cap;
+    int rows_max;          // full_max + k_cap: the rows the host sized the step for
+    int sel_cap;           // room for selected indices in LDS (>= k_cap)
+    uint32_t *emit_count;  // [BH, GP]: keys considered per row (all of them here), for monitoring
+};
+
+__device__ inline void store1_any(int dtype, char *row, int d, float x) {
+    if (dtype == PQHSA_F32) store1<PQHSA_F32>(row, d, x);
+    else if (dtype == PQHSA_BF16) store1<PQHSA_BF16>(row, d, x);
+    else store1<PQHSA_F16>(row, d, x);
+}
+
+template <int KDT, int R>
+__global__ __launch_bounds__(kSelThreads) void decode_small_kernel(SmallArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ __align__(16) uint32_t red[2][kSelWaves];
+    __shared__ uint32_t wsum[2 * kSelWaves];
+    __shared__ SelScratch ss;
+    __shared__ __align__(16) float qh[kD];
+    __shared__ float lut_s[kM * kCodes];
+    __shared__ float qn_s;
+    __shared__ float fin_s[4];
+    const int tid = threadIdx.x;
+    const int g = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / a.H, h = bh % a.H;
+    const size_t orow = (size_t)bh * a.G + g;
+    const int L = a.L;
+    float(*cs)[kSmallRow] = reinterpret_cast<float(*)[kSmallRow]>(smem);    // [kSmallTile][132]: rows 16-byte aligned, conflict-free
+    float *ls_s = reinterpret_cast<float *>(smem) + kSmallTile * kSmallRow;  // [L] query-to-centroid products
+    float *mx = ls_s + L;                                                   // [L] background weight per list
+    int32_t *sel_s = reinterpret_cast<int32_t *>(mx + L);                   // [sel_cap] the selected keys
+    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 0);
+
+    // ---- 1. the row's tables --------------------------------------------------------------------
+    float4 tile[8];  // a tile is 256 x 128 floats: eight float4 per thread
+    auto fetch_tile = [&](int l0) {
+        const int nl = min(kSmallTile, L - l0);
+        const float4 *c4 = reinterpret_cast<const float4 *>(a.coarse + ((size_t)bh * L + l0) * kD);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = tid + u * kSelThreads;
+            tile[u] = i < nl * (kD / 4) ? c4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    };
+    fetch_tile(0);
+    const size_t qesz = a.q_dtype == PQHSA_F32 ? 4 : 2;
+    const char *qrow = a.q + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
+    float4 cw[kSub / 4];
+    if (tid < kD) {
+        qh[tid] = load1_any(a.q_dtype, qrow, tid);
+        const float4 *w4 = reinterpret_cast<const float4 *>(a.codebooks + ((size_t)bh * kM * kCodes + tid) * kSub);
+#pragma unroll
+        for (int e = 0; e < kSub / 4; ++e) cw[e] = w4[e];
+    }
+    const int n = max(0, min(min(a.n_arr[b], (int)a.n_cap), R * kSelThreads));
+    const int len = a.seq_lens[b];
+    for (int l = tid; l < L; l += kSelThreads) mx[l] = 0.0f;
+    for (int i = tid; i < kSelBins; i += kSelThreads) ss.hist[i] = 0u, ss.cont_key[i] = 0u;
+    if (tid == 0) ss.cont_count = 0u;
+    __syncthreads();
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 1);
+    if (tid == 0) {
+        float ss2 = 0.0f;
+        for (int d = 0; d < kD; ++d) ss2 = __builtin_fmaf(qh[d], qh[d], ss2);
+        const float nq = sqrtf(ss2);
+        qn_s = nq < a.eps ? a.eps : nq;
+    }
+    __syncthreads();
+    const float qn = qn_s;
+    if (tid < kD) qh[tid] = qh[tid] / qn;
+    __syncthreads();
+    if (tid < kM * kCodes) {
+        const int m = tid / kCodes;
+        const float w[kSub] = {cw[0].x, cw[0].y, cw[0].z, cw[0].w, cw[1].x, cw[1].y, cw[1].z, cw[1].w,
+                               cw[2].x, cw[2].y, cw[2].z, cw[2].w, cw[3].x, cw[3].y, cw[3].z, cw[3].w};
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kSub; ++j) acc = __builtin_fmaf(qh[m * kSub + j], w[j], acc);
+        lut_s[tid] = acc;
+    }
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 2);
+    // the coarse centroids, a tile at a time: thread l of the first 256 takes list l of the tile
+    auto stage_tile = [&]() {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = tid + u * kSelThreads;
+            *reinterpret_cast<float4 *>(&cs[i / (kD / 4)][(i % (kD / 4)) * 4]) = tile[u];
+        }
+    };
+    auto products = [&](int l0) {
+        if (tid < kSmallTile && l0 + tid < L) {
+            float acc = 0.0f;
+#pragma unroll 8
+            for (int d4 = 0; d4 < kD / 4; ++d4) {  // the chain runs over d in order, four elements per LDS read
+                const float4 c = *reinterpret_cast<const float4 *>(&cs[tid][4 * d4]);
+                const float4 qq = *reinterpret_cast<const float4 *>(&qh[4 * d4]);
+                acc = __builtin_fmaf(qq.x, c.x, acc);
+                acc = __builtin_fmaf(qq.y, c.y, acc);
+                acc = __builtin_fmaf(qq.z, c.z, acc);
+                acc = __builtin_fmaf(qq.w, c.w, acc);
+            }
+            ls_s[l0 + tid] = acc;
+        }
+    };
+    int l0 = 0;
+    for (; l0 + kSmallTile < L; l0 += kSmallTile) {  // all tiles but the last: the next one travels meanwhile
+        stage_tile();
+        __syncthreads();
+        fetch_tile(l0 + kSmallTile);
+        products(l0);
+        __syncthreads();
+    }
+    stage_tile();
+    __syncthreads();
+    // the stored keys of the row: key p = r * 1024 + tid in slot r, requested while the last tile is used
+    const size_t base = (size_t)bh * a.n_cap;
+    uint32_t code[R], lid[R], where[R];
+    float kn[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int p = r * kSelThreads + tid;
+        const bool ok = p < n;
+        code[r] = ok ? a.codes[base + p] : 0u;
+        lid[r] = ok ? a.list_ids[base + p] : 0u;
+        kn[r] = ok ? a.norms[base + p] : 0.0f;
+        where[r] = ok ? (a.pos ? (uint32_t)a.pos[base + p] : (uint32_t)p) : 0u;
+    }
+    products(l0);
+    __syncthreads();
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 3);
+
+    // ---- 2. logits of all stored keys, exact top-k, background weights ----------------------------
+    const int k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
+    uint32_t key[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int p = r * kSelThreads + tid;
+        if (lid[r] >= (uint32_t)L) lid[r] = 0u;
+        key[r] = p < n ? max(order_key(score_one(lut_s, ls_s, code[r], lid[r], qn, kn[r], a.scale)), 1u) : 0u;
+    }
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 4);
+    float ref1 = -INFINITY;
+    if (n > 0) {  // (uniform over the workgroup)
+        SelectOut out;
+        out.out_idx = a.topk_idx + orow * a.k_cap;
+        out.out_val = a.topk_val ? a.topk_val + orow * a.k_cap : nullptr;
+        out.k_cap = (uint32_t)a.k_cap;
+        out.mx = mx;
+        out.ref1 = 0.0f;
+        out.lds_idx = sel_s;
+        out.lds_cap = (uint32_t)a.sel_cap;
+        // All keys of the row are candidates here, and the k-th largest lies far out in the tail of
+        // a wide span.  A first histogram, over the keys within four exponent steps of the largest
+        // only, finds the range that holds it; the selection proper then works between that
+        // range's lower edge and the largest key and leaves the keys below out of its histogram.
+        // (If the window holds fewer than k keys the selection runs over the whole span.)
+        uint32_t lo_hint = 0u, hi_hint = 0u;
+        if (k > 0) {
+            uint32_t lo_key, hi_key;
+            block_min_max<0u>(key, wsum, lo_key, hi_key);
+            constexpr uint32_t kWindow = 1u << 25;
+            const uint32_t wbase = hi_key > kWindow ? max(hi_key - kWindow, lo_key) : lo_key;
+            const uint32_t range = hi_key >= wbase ? hi_key - wbase : 0u;
+            const int shift = range < (uint32_t)kSelBins ? 0 : (31 - __clz(range)) - 9;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (key[r] != 0u && key[r] >= wbase) atomicAdd(&ss.cont_key[min((key[r] - wbase) >> shift, (uint32_t)kSelBins - 1u)], 1u);
+            if (tid == 0) ss.bin = 0xffffffffu;
+            __syncthreads();
+            if (tid < kWave) find_from_top_1024(ss.cont_key, (uint32_t)k, &ss.bin, &ss.above);
+            __syncthreads();
+            const uint32_t bin = ss.bin;  // (this histogram lives in an array the selection only writes after its own barriers)
+            __syncthreads();              // ... but it sets ss.bin again right away: everyone reads it first
+            const uint32_t edge = bin < (uint32_t)kSelBins ? wbase + (bin << shift) : 0u;
+            if (edge > 1u && hi_key > edge) {  // keys equal to the edge must stay above the hint
+                lo_hint = edge - 1u;
+                hi_hint = hi_key;
+            }
+        }
+        select_loaded<R>(key, where, lid, (uint32_t)n, k, out, red, wsum, &ss, &ref1, lo_hint, hi_hint, lo_hint != 0u);
+    }
+    if (tid == 0) {
+        a.topk_cnt[orow] = k;
+        if (a.emit_count) a.emit_count[(size_t)bh * a.GP + g] = (uint32_t)n;
+    }
+    __syncthreads();  // the selected indices (global memory, this workgroup's own stores) and mx are complete
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 5);
+
+    // ---- 3. attention over sink, window and selected rows, merged with the background -------------
+    constexpr int kGroups = kSelThreads / 16;
+    constexpr int kBgParts = kSelThreads / (kD / 4);   // 32 threads cover a mean-value row with float4 loads
+    float *red_acc = reinterpret_cast<float *>(smem);  // [kGroups][128] (the tile area is free now)
+    float *red_m = red_acc + kGroups * kD;             // [kGroups]
+    float *red_l = red_m + kGroups;                    // [kGroups]
+    float *bg_s = red_l + kGroups;                     // [kBgParts][128]
+    float *ms_s = bg_s + kBgParts * kD;                // [kBgParts]
+    const int lane16 = tid & 15, grp = tid >> 4;
+    const int sink_end = min(a.sink, len);
+    const int local_start = sink_end + n;
+    const int F = sink_end + max(len - local_start, 0);
+    const int total = min(F + min(k, a.sel_cap), a.rows_max);  // (device-side lengths beyond what the host sized the step for are cut)
+    float qv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[e] = load1_any(a.q_dtype, qrow, lane16 * 8 + e);
+    const size_t kesz = KDT == PQHSA_F32 ? 4 : 2;
+    float m_g = -INFINITY, l_g = 0.0f;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    constexpr int U = 4;
+    for (int r0 = grp; r0 < total; r0 += kGroups * U) {
+        float kf[U][8], vf[U][8];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = r0 + u * kGroups;
+            ok[u] = r < total;
+            if (ok[u]) {
+                const int64_t pos = r < sink_end ? r : (r < F ? local_start + (r - sink_end) : sink_end + sel_s[r - F]);
+                const int64_t off = row_offset(a.kv, b, h, pos) * (int64_t)kesz;
+                load8<KDT>(a.kv.k_base + off, lane16, kf[u]);
+                load8<KDT>(a.kv.v_base + off, lane16, vf[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!ok[u]) continue;  // uniform over the 16 lanes of the group
+            float x = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x = __builtin_fmaf(kf[u][e], qv[e], x);
+            x = group_sum16(x) * a.scale;
+            const float m_new = fmaxf(m_g, x);
+            const float keep = __expf(m_g - m_new);  // 0 for the first row (m_g = -inf)
+            const float p = __expf(x - m_new);
+            l_g = __builtin_fmaf(l_g, keep, p);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(acc[e], keep, p * vf[u][e]);
+            m_g = m_new;
+        }
+    }
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 6);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red_acc[grp * kD + lane16 * 8 + e] = acc[e];
+    if (lane16 == 0) { red_m[grp] = m_g; red_l[grp] = l_g; }
+    {
+        // background: sum over the lists of weight x mean value; thread (d4, part) takes four elements
+        // of lists part, part + 32, ...; up to 16 loads per thread, all requested before the first is used
+        const int d4 = (tid & (kD / 4 - 1)) * 4, part = tid / (kD / 4);
+        const float *vb = a.vbar + (size_t)bh * L * kD + d4;
+        float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float msum = 0.0f;
+        if (n > 0) {
+            for (int l0 = part; l0 < L; l0 += 16 * kBgParts) {
+                float4 v[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int l = l0 + u * kBgParts;
+                    v[u] = l < L ? *reinterpret_cast<const float4 *>(vb + (size_t)l * kD) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int l = l0 + u * kBgParts;
+                    const float w = l < L ? mx[l] : 0.0f;
+                    t.x = __builtin_fmaf(w, v[u].x, t.x); t.y = __builtin_fmaf(w, v[u].y, t.y);
+                    t.z = __builtin_fmaf(w, v[u].z, t.z); t.w = __builtin_fmaf(w, v[u].w, t.w);
+                    msum += w;
+                }
+            }
+        }
+        *reinterpret_cast<float4 *>(&bg_s[part * kD + d4]) = t;
+        if (d4 == 0) ms_s[part] = msum;
+    }
+    __syncthreads();
+    if (tid < kWave) {  // one group per lane: row maximum
+        float m = red_m[tid];
+        m = wave_max(m);
+        float ms = tid < kBgParts ? ms_s[tid] : 0.0f;
+        ms = wave_sum(ms);
+        if (tid == 0) { fin_s[0] = m; fin_s[1] = ms; }
+    }
+    __syncthreads();
+    if (tid < kD) {
+        float m = fin_s[0];
+        const float ms = fin_s[1];
+        const bool bg_on = ms != 0.0f && ref1 > -INFINITY;
+        if (bg_on) m = fmaxf(m, ref1);
+        char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
+        if (m == -INFINITY) {  // nothing to attend to
+            store1_any(a.q_dtype, orow_p, tid, 0.0f);
+        } else {
+            float num = 0.0f, den = 0.0f;
+            for (int gi = 0; gi < kGroups; ++gi) {
+                const float mg = red_m[gi];
+                const float w = mg == -INFINITY ? 0.0f : __expf(mg - m);
+                num = __builtin_fmaf(red_acc[gi * kD + tid], w, num);
+                den = __builtin_fmaf(red_l[gi], w, den);
+            }
+            if (bg_on) {
+                const float f0 = __expf(ref1 - m);
+                float bgv = 0.0f;
+#pragma unroll
+                for (int part = 0; part < kBgParts; ++part) bgv += bg_s[part * kD + tid];
+                num = __builtin_fmaf(bgv, f0, num);
+                den = __builtin_fmaf(ms, f0, den);
+            }
+            den = fmaxf(den, FLT_MIN);
+            store1_any(a.q_dtype, orow_p, tid, num / den);
+        }
+    }
+    PQHSA_TRACE_MARK(trace_small, trace_wg, 7);
+}
+
+// whether the short-context kernel serves a step of this shape
+bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap) {
+    // (one workgroup per query row; tables and selected indices in LDS: 135 KB tile + 8 L + 4 k_cap bytes)
+    return streams > 0 && (int64_t)streams * G <= 256 && n_max <= 16 * kSelThreads && L <= 1024 && k_cap <= 2048;
+}
+
+template <int KDT>
+static int launch_decode_small_kdt(const SmallArgs &a, int streams, int64_t n_max, size_t lds, hipStream_t stream) {
+    const dim3 grid(a.G, streams), block(kSelThreads);
+#define PQHSA_SMALL(RV)                                                                                          \
+    {                                                                                                            \
+        auto kern = decode_small_kernel<KDT, RV>;                                                                \
+        static size_t raised[64] = {}; /* per device: the LDS limit already set for this instantiation */       \
+        int dev = 0;                                                                                             \
+        (void)hipGetDevice(&dev);                                                                                \
+        if (dev < 0 || dev >= 64 || raised[dev] < lds) {                                                         \
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)lds) != hipSuccess) {                                                   \
+                set_error("decode_step: cannot raise the LDS limit to %zu bytes", lds);                          \
+                return PQHSA_ELAUNCH;                                                                            \
+            }                                                                                                    \
+            if (dev >= 0 && dev < 64) raised[dev] = lds;                                                         \
+        }                                                                                                        \
+        hipLaunchKernelGGL(kern, grid, block, lds, stream, a);                                                   \
+    }
+    if (n_max <= 8 * kSelThreads) PQHSA_SMALL(8)
+    else PQHSA_SMALL(16)
+#undef PQHSA_SMALL
+    return PQHSA_OK;
+}
+
+int launch_decode_small(SmallArgs a, int kv_dtype, int streams, int64_t n_max, hipStream_t stream) {
+    a.sel_cap = a.k_cap;
+    const size_t lds = (size_t)kSmallTile * kSmallRow * sizeof(float) + 2 * (size_t)a.L * sizeof(float) +
+                       (size_t)a.sel_cap * sizeof(int32_t);
+    int rc;
+    if (kv_dtype == PQHSA_F32) rc = launch_decode_small_kdt<PQHSA_F32>(a, streams, n_max, lds, stream);
+    else if (kv_dtype == PQHSA_BF16) rc = launch_decode_small_kdt<PQHSA_BF16>(a, streams, n_max, lds, stream);
+    else if (kv_dtype == PQHSA_F16) rc = launch_decode_small_kdt<PQHSA_F16>(a, streams, n_max, lds, stream);
+    else {
+        set_error("decode_step: unsupported K/V dtype %d", kv_dtype);
+        return PQHSA_EINVAL;
+    }
+    if (rc) return rc;
+    return check_launch("decode_small");
+}
+
+// the whole step through the short-context kernel (the caller has checked decode_small_fits)
+int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
+                 const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const pqhsa_select *select, float scale,
+                 float eps, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, uint32_t *emit_count,
+                 hipStream_t stream) {
+    SmallArgs a = {};
+    a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.q_dtype = q_dtype;
+    a.kv = make_view(kv);
+    a.H = index->kv_heads; a.G = G; a.GP = GP;
+    a.seq_lens = seq_lens; a.n_arr = index->n_idx; a.sink = sink;
+    a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = index->pos;
+    a.n_cap = index->n_cap;
+    a.coarse = index->coarse; a.codebooks = index->codebooks; a.vbar = index->vbar; a.L = index->num_lists;
+    a.eps = eps; a.scale = scale; a.fraction = select->fraction; a.topk = select->topk;
+    a.topk_idx = topk_idx; a.topk_val = topk_val; a.topk_cnt = topk_cnt; a.k_cap = select->k_cap;
+    a.rows_max = rows_max; a.emit_count = emit_count;
+    PQHSA_REQUIRE(q_dtype == PQHSA_F32 || q_dtype == PQHSA_BF16 || q_dtype == PQHSA_F16, "decode_step: unsupported query dtype %d",
+                  q_dtype);
+    profile_mark(kProfLut, stream);   // one kernel: the event log books it under the last slot
+    profile_mark(kProfSample, stream);
+    profile_mark(kProfEmit, stream);
+    profile_mark(kProfSelect, stream);
+    profile_mark(kProfAttend, stream);
+    const int rc = launch_decode_small(a, kv->dtype, index->batch * index->kv_heads, n_max, stream);
+    profile_mark(kProfKernels, stream);
+    return rc;
 }
 
 int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t stream);

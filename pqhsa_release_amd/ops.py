@@ -424,8 +424,10 @@ class DecodeWorkspace:
 def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
                 seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
                 scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None,
-                append_count: torch.Tensor | None = None) -> torch.Tensor:
+                append_count: torch.Tensor | None = None, general_path: bool = False) -> torch.Tensor:
     """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``.
+    Short contexts are served by a single kernel (same results); ``general_path`` keeps such a step
+    on the five-kernel path (``PQHSA_SELECT_GENERAL_PATH``).
     With ``append_count`` (device int32 [B]) the step first appends one key to every sequence whose
     entry is positive (``pqhsa_append_decode_step``): ``n_max`` must count the appended key and the
     caller calls ``index.note_appended`` afterwards."""
@@ -441,6 +443,7 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     sel.fraction = float(fraction) if fraction else 0.0
     sel.topk = int(topk)
     sel.k_cap = workspace.k_cap
+    sel.flags = _lib.SELECT_GENERAL_PATH if general_path else 0
     n_max = index.n_max if n_max is None else int(n_max)
     args = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups, seq_lens.data_ptr(),
             int(sink), n_max, int(full_max), ctypes.byref(sel), float(scale), eps, workspace.topk_idx.data_ptr(),

@@ -39,4 +39,4 @@ def test_struct_layouts_match_the_header():
     # sizes implied by include/pqhsa.h on LP64: pointers and int64 8-byte aligned
     assert ctypes.sizeof(_lib.KvView) == 8 + 8 + 4 + 4 + 8 * 4 + 4 + 4 + 8
     assert ctypes.sizeof(_lib.Index) == 15 * 8 + 2 * 8 + 4 * 3 + 4
-    assert ctypes.sizeof(_lib.Select) == 16
+    assert ctypes.sizeof(_lib.Select) == 24

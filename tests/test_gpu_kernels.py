@@ -161,7 +161,10 @@ def test_topk_radix_on_logit_matrix_with_ties(stride):
     dict(lens=[2200], heads=2, groups=7, lists=48, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
     dict(lens=[1500], heads=1, groups=2, lists=16, dtype=torch.float16, fraction=0.1, kv="dense"),
 ])
-def test_decode_step_topk_bitexact_and_output_close(case):
+@pytest.mark.parametrize("general_path", [False, True])
+def test_decode_step_topk_bitexact_and_output_close(case, general_path):
+    """Both forms of the step against the oracle: the single kernel that serves short contexts
+    (taken by default at these sizes) and the general five-kernel path."""
     dev = _cuda()
     p = Problem(lens=case["lens"], heads=case["heads"], groups=case["groups"], lists=case["lists"],
                 dtype=case["dtype"], seed=13)
@@ -180,7 +183,7 @@ def test_decode_step_topk_bitexact_and_output_close(case):
         q = p.q_tensor().to(q_dtype)
         out = torch.empty_like(q)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                        fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws)
+                        fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws, general_path=general_path)
         torch.cuda.synchronize()
         tol = 1e-4 if case["dtype"] == torch.float32 else 2e-3
         rel = 0.0 if q_dtype == torch.float32 else (2.0 ** -8 if q_dtype == torch.bfloat16 else 2.0 ** -11)
@@ -268,11 +271,12 @@ def test_missing_or_bad_arguments_fail_loudly():
         ops.lut_build(torch.zeros(1, 17, 128, device=dev), idx, 17)         # G too large
 
 
-def _check_step(p, idx, kv, ws, fraction, tol=1e-4):
+def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
+    """(The tests that use this are about the general path's estimate, candidate area and layouts.)"""
     q = p.q_tensor()
     out = torch.empty_like(q)
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
-                    topk=0, scale=SCALE, workspace=ws)
+                    topk=0, scale=SCALE, workspace=ws, general_path=general_path)
     torch.cuda.synchronize()
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
     o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
@@ -335,7 +339,7 @@ def test_decode_step_with_device_lengths_beyond_the_host_bounds_exits_normally()
     out = torch.empty_like(q)
     # one row more on the device than the host sized the attention launch for
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local - 1, fraction=0.03,
-                    topk=0, scale=SCALE, workspace=ws)
+                    topk=0, scale=SCALE, workspace=ws, general_path=True)
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
@@ -344,10 +348,13 @@ def test_decode_step_with_device_lengths_beyond_the_host_bounds_exits_normally()
         for g in range(p.G):
             assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (b, h, g)
     # a scan sized for fewer keys than the device-side counts say
-    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
-                    topk=0, scale=SCALE, workspace=ws, n_max=p.n_max - 1500)
-    torch.cuda.synchronize()
-    assert torch.isfinite(out.float()).all()
+    for general_path in (False, True):   # (the single-kernel form clamps the same way)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local - 1, fraction=0.03,
+                        topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
+                        topk=0, scale=SCALE, workspace=ws, n_max=p.n_max - 1500, general_path=general_path)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all()
     cnt = ws.topk_cnt.cpu().numpy()
     assert (cnt >= 0).all() and (cnt <= k_cap).all()
     sel = ws.topk_idx.cpu().numpy().reshape(p.B * p.H * p.G, -1)
@@ -652,12 +659,15 @@ def test_device_counts_ahead_of_the_host_stay_inside_k_cap():
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
     q = p.q_tensor()
     out = torch.empty_like(q)
-    ops.decode_step(q, out, ops.kv_contiguous(*p.dense_kv()), idx, p.G, p.seq_lens(), sink=p.sink,
-                    full_max=p.sink + p.local, fraction=0.05, topk=0, scale=SCALE, workspace=ws, n_max=small)
-    torch.cuda.synchronize()
-    assert ws.topk_cnt.cpu().tolist() == [k_cap] * p.G
-    got = ws.topk_idx.cpu().numpy()
-    assert ((got >= 0) & (got < n)).all() and bool(torch.isfinite(out).all())
+    for general_path in (False, True):
+        ws.topk_cnt.zero_()
+        ops.decode_step(q, out, ops.kv_contiguous(*p.dense_kv()), idx, p.G, p.seq_lens(), sink=p.sink,
+                        full_max=p.sink + p.local, fraction=0.05, topk=0, scale=SCALE, workspace=ws, n_max=small,
+                        general_path=general_path)
+        torch.cuda.synchronize()
+        assert ws.topk_cnt.cpu().tolist() == [k_cap] * p.G
+        got = ws.topk_idx.cpu().numpy()
+        assert ((got >= 0) & (got < n)).all() and bool(torch.isfinite(out).all())
 
 
 @pytest.mark.parametrize("seed", [1, 2])
@@ -684,8 +694,10 @@ def test_decode_step_random_shapes_match_oracle(seed):
         ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, fraction, 0))
         q = p.q_tensor()
         out = torch.empty_like(q)
+        general_path = rng.random() < 0.5     # else the single kernel for short contexts, where the shape fits it
+        what = what + (general_path,)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                        fraction=fraction, topk=0, scale=SCALE, workspace=ws)
+                        fraction=fraction, topk=0, scale=SCALE, workspace=ws, general_path=general_path)
         torch.cuda.synchronize()
         tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
         o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
@@ -697,12 +709,13 @@ def test_decode_step_random_shapes_match_oracle(seed):
             for g in range(p.G):
                 assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (what, b, h, g)
             assert (np.abs(o[b, h] - want_out) <= tol + rel * np.abs(want_out)).all(), (what, b, h)
-        if finalize:  # (an index that was never sampled makes every key a candidate: long rows then take the full pass)
+        if finalize and general_path:  # (an index that was never sampled makes every key a candidate: long rows then take the full pass)
             assert ws.rescans() == 0, what
 
 
+@pytest.mark.parametrize("general_path", [False, True])
 @pytest.mark.parametrize("groups,lists,lens", [(16, 64, [2600]), (12, 256, [5000, 1700]), (9, 512, [7000])])
-def test_decode_step_wide_groups_and_many_lists(groups, lists, lens):
+def test_decode_step_wide_groups_and_many_lists(groups, lists, lens, general_path):
     """Query groups of 9 to 16 rows (padded to 16 in the kernels) and list counts up to the
     headline configuration's 512, against the oracle."""
     dev = _cuda()
@@ -713,7 +726,7 @@ def test_decode_step_wide_groups_and_many_lists(groups, lists, lens):
     q = p.q_tensor().float()
     out = torch.empty_like(q)
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.05,
-                    topk=0, scale=SCALE, workspace=ws)
+                    topk=0, scale=SCALE, workspace=ws, general_path=general_path)
     torch.cuda.synchronize()
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
     o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
@@ -814,7 +827,7 @@ def test_event_log_counts_steps_and_samples_them():
     def steps(count):
         for _ in range(count):
             ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                            fraction=0.02, topk=0, scale=SCALE, workspace=ws)
+                            fraction=0.02, topk=0, scale=SCALE, workspace=ws, general_path=True)
 
     def collect():
         kms = (ctypes.c_float * 5)()
