@@ -183,6 +183,21 @@ int pqhsa_lut_scan(const pqhsa_index *index, int32_t G, int32_t n_max, const flo
                    int64_t logit_stride, void *stream);
 
 /*
+ * The scan's other output, stand-alone: per-list background mass of every query row in one pass
+ * over the index, without writing a logit:
+ *   list_mass[bh, l, g] = sum over the stream's stored keys of list l of exp(logit - ref[bh, g])
+ * list_mass is f32 [BH, num_lists, padded_groups(G)] (cleared by the call, accumulated with float
+ * atomics; the weights of 64 neighbouring keys are summed per list as differences of one prefix
+ * sum, so a list's mass is accurate to about 1e-7 of the row's total, not of itself), ref f32
+ * [BH, padded_groups(G)] (a reference logit per row, e.g. the row maximum; a non-finite entry is
+ * taken as 0).  Counterpart of the list-mass output of the reference's
+ * pq_scan_only (pq_hsa/kernels/cuda/pq_fused_h20.cu:3826-3839).
+ */
+int pqhsa_lut_scan_mass(const pqhsa_index *index, int32_t G, int32_t n_max, const float *qnorm,
+                        const float *lut, const float *list_scores, float scale, const float *ref,
+                        float *list_mass, void *stream);
+
+/*
  * Exact top-k of each row of a logit matrix [rows, stride] by radix selection on the fp32
  * bit pattern (no sort); ties at the k boundary go to the lowest index; the k winners are
  * written (in no particular order) with their logits.  n[r] and k[r] are per-row device

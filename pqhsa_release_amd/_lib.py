@@ -118,6 +118,8 @@ SIGNATURES = {
     "pqhsa_profile_collect": (ctypes.c_int, [c_void_p, c_void_p]),
     "pqhsa_paged_gather_at": (ctypes.c_int, [_P(KvView), c_int32, c_int32, c_void_p, c_int64, c_void_p, c_void_p,
                                              c_void_p]),
+    "pqhsa_lut_scan_mass": (ctypes.c_int, [_P(Index), c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                                           c_void_p, c_void_p]),
     "pqhsa_gather_probe": (ctypes.c_int, [_P(KvView), c_int32, c_int32, c_void_p, c_int64, c_void_p, c_void_p]),
 }
 

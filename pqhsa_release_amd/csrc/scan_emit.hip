@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
         for (int i = tid; i < L * GP; i += TH) mass_s[i] = 0.0f;
 #pragma unroll
     for (int g = 0; g < GP; ++g) {
-        const uint32_t tk = a.thr_key[(size_t)bh * GP + g];
+        const uint32_t tk = a.thr_key ? a.thr_key[(size_t)bh * GP + g] : 0xffffffffu;  // no thresholds: no candidates
         const float rv = a.ref_val[(size_t)bh * GP + g];
         // keys below that of the lowest finite float are not keys of ordered floats: such a
         // threshold keeps every key of the index (its logits are finite)
@@ -410,3 +410,33 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t
 }
 
 }  // namespace pqhsa
+
+using namespace pqhsa;
+
+namespace pqhsa {
+int launch_fill_zero(void *p, size_t bytes, hipStream_t stream);
+}
+
+extern "C" int pqhsa_lut_scan_mass(const pqhsa_index *index, int32_t G, int32_t n_max, const float *qnorm, const float *lut,
+                                   const float *list_scores, float scale, const float *ref, float *list_mass,
+                                   void *stream_v) {
+    PQHSA_REQUIRE(index && qnorm && lut && list_scores && ref && list_mass, "lut_scan_mass: NULL argument");
+    PQHSA_REQUIRE(G >= 1 && G <= 16, "lut_scan_mass: G=%d outside [1, 16]", G);
+    PQHSA_REQUIRE(index->n_cap % 8 == 0 && index->n_cap > 0, "lut_scan_mass: n_cap=%lld must be a positive multiple of 8",
+                  (long long)index->n_cap);
+    PQHSA_REQUIRE(n_max >= 0 && n_max <= index->n_cap, "lut_scan_mass: n_max=%d outside [0, n_cap]", n_max);
+    PQHSA_REQUIRE(index->num_lists >= 1 && index->num_lists <= 4096, "lut_scan_mass: num_lists=%d", index->num_lists);
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const int GP = padded_groups(G);
+    const int streams = index->batch * index->kv_heads;
+    if (streams == 0) return PQHSA_OK;
+    int rc = launch_fill_zero(list_mass, (size_t)streams * index->num_lists * GP * sizeof(float), stream);
+    if (rc) return rc;
+    ScanArgs a = {};
+    a.qnorm = qnorm; a.lut = lut; a.list_scores = list_scores; a.scale = scale; a.L = index->num_lists;
+    a.n_div = index->kv_heads; a.G = G;
+    a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = nullptr;
+    a.n_cap = index->n_cap; a.n_arr = index->n_idx;
+    a.thr_key = nullptr; a.ref_val = ref; a.mass = list_mass;
+    return launch_scan_emit(a, GP, streams, n_max, stream);
+}

@@ -367,6 +367,23 @@ def lut_scan(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scale: fl
     return logits
 
 
+def lut_scan_mass(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scale: float, ref: torch.Tensor) -> torch.Tensor:
+    """Per-list background mass of every query row, ``[BH, L, padded G]``: the sum over each list's
+    stored keys of ``exp(logit - ref[bh, g])`` (``ref`` float32 ``[BH, padded G]``), in one pass over
+    the index without writing logits (``pqhsa_lut_scan_mass``)."""
+    lib = _lib.load()
+    _need_cuda(ref)
+    bh = index.batch * index.kv_heads
+    gp = int(lib.pqhsa_padded_groups(groups))
+    if ref.dtype != torch.float32 or tuple(ref.shape) != (bh, gp) or not ref.is_contiguous():
+        raise ValueError(f"ref must be a contiguous float32 [{bh}, {gp}] tensor")
+    mass = torch.empty(bh, index.num_lists, gp, dtype=torch.float32, device=index.device)
+    rc = lib.pqhsa_lut_scan_mass(index.ref(), groups, int(index.n_max), qnorm.data_ptr(), lut.data_ptr(),
+                                 list_scores.data_ptr(), float(scale), ref.data_ptr(), mass.data_ptr(), _stream())
+    _lib.check(rc, "pqhsa_lut_scan_mass")
+    return mass
+
+
 def topk_radix(logits: torch.Tensor, n, k):
     """Exact top-k of each row of ``logits [rows, stride]``; ``n``/``k`` per row.  Returns
     (indices int32 [rows, k_cap], values f32 [rows, k_cap]), the selected keys in no particular order."""

@@ -206,6 +206,39 @@ def test_decode_step_topk_bitexact_and_output_close(case, general_path):
         print(f"decode_step {case['dtype']} q={q_dtype}: max abs err {worst:.3e}")
 
 
+def test_stand_alone_scan_list_mass_matches_the_logits():
+    """pqhsa_lut_scan_mass: per-list sums of exp(logit - reference) in one pass over the index, against
+    the same sums formed in float64 from the oracle's logits (the scan's logits are the oracle's bit
+    for bit; the sums are float atomics, compared to 1e-5)."""
+    dev = _cuda()
+    p = Problem(lens=[5000, 2300], heads=2, groups=3, lists=32, seed=71)
+    idx = p.device_index(dev)
+    qnorm, lut, ls = ops.lut_build(p.q_tensor(), idx, p.G)
+    gp = qnorm.shape[-1] if qnorm.ndim > 1 else qnorm.numel() // (p.B * p.H)
+    ref = torch.zeros(p.B * p.H, gp, dtype=torch.float32, device=dev)
+    want = {}
+    for (b, h), ix in p.index.items():
+        _, _, logits = p.oracle_step(b, h, 0.02)                      # [G, n]
+        bh = b * p.H + h
+        for g in range(p.G):
+            ref[bh, g] = float(logits[g].max())
+        lists = ix["list_ids"].astype(np.int64)
+        w = np.exp(logits.astype(np.float64) - logits.max(axis=1, keepdims=True).astype(np.float64))
+        m = np.zeros((p.L, p.G))
+        for g in range(p.G):
+            np.add.at(m[:, g], lists, w[g])
+        want[bh] = m
+    mass = ops.lut_scan_mass(idx, p.G, qnorm, lut, ls, SCALE, ref)
+    torch.cuda.synchronize()
+    got = mass.cpu().numpy()
+    for bh, m in want.items():
+        # (the weights of a wave's keys are summed per list as differences of one prefix sum over its
+        # lanes: absolute accuracy about 1e-7 of the row's mass, which is what a softmax needs)
+        for g in range(p.G):
+            np.testing.assert_allclose(got[bh, :, g], m[:, g], rtol=1e-5, atol=5e-7 * m[:, g].sum())
+        assert (got[bh, :, p.G:] == 0).all()                          # padded rows of the group carry nothing
+
+
 def test_decode_step_all_selected_equals_dense_attention():
     dev = _cuda()
     p = Problem(lens=[600], heads=1, groups=2, lists=16, seed=17)
