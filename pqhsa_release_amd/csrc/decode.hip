@@ -37,6 +37,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
                   float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
                   hipStream_t stream);
 size_t attend_partials_bytes(int rows, int k_cap);
+size_t attend_arrive_bytes(int rows);
 
 static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -74,7 +75,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.rescans = reinterpret_cast<uint32_t *>(take(256));  // running counter, never cleared by a step
     const size_t z0 = off;  // everything from here to zero_words is cleared at the start of a step
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
-    c.arrive = reinterpret_cast<uint32_t *>(take(BH * G * 4));  // attention workgroups arrived per query row
+    c.arrive = reinterpret_cast<uint32_t *>(take(attend_arrive_bytes((int)(BH * G))));  // attention: arrival flags and tickets per query row
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
     c.zero_words = (off - z0) / 4;
     c.qnorm = reinterpret_cast<float *>(take(rows * 4));
