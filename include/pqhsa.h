@@ -304,6 +304,17 @@ const uint32_t *pqhsa_decode_rescan_counter(void *workspace);
 const uint32_t *pqhsa_decode_candidate_counts(void *workspace);
 
 /*
+ * Number of kernel launches pqhsa_decode_step makes for a step of this shape: 1 when the
+ * short-context kernel serves it (no append, PQHSA_SELECT_GENERAL_PATH not set, at most 16 384
+ * indexed keys per stream, at most 256 query rows, at most 1 024 lists, k_cap at most 2 048), else
+ * PQHSA_PROFILE_KERNELS.  With one launch the event log books the whole step under its last slot
+ * and the other slots hold only the cost of recording an event.  No counterpart in the
+ * reference; for benchmarks and monitors that label per-kernel times.
+ */
+int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t G, int32_t n_max, const pqhsa_select *select,
+                                   int32_t appending);
+
+/*
  * Hybrid exact attention alone, given the selection and the per-list masses:
  *   list_mass f32 [BH, G, L] = sum over ALL the list's indexed keys of exp(logit - row_max),
  *   row_max f32 [BH, G] (the maximum approximate logit of the row),

@@ -123,6 +123,14 @@ extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace) {
     return reinterpret_cast<const uint32_t *>(base + 256);  // the second block of the carve-up
 }
 
+extern "C" int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t G, int32_t n_max,
+                                              const pqhsa_select *select, int32_t appending) {
+    if (!index || !select) return 0;
+    const bool small = !appending && !(select->flags & PQHSA_SELECT_GENERAL_PATH) &&
+                       decode_small_fits(index->batch * index->kv_heads, G, n_max, index->num_lists, select->k_cap);
+    return small ? 1 : PQHSA_PROFILE_KERNELS;
+}
+
 static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
                             const pqhsa_index *index, int32_t G, const int32_t *seq_lens, int32_t sink,
                             int32_t n_max, int32_t full_max, const pqhsa_select *select, float scale, float eps,
@@ -156,8 +164,7 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     if (!topk_cnt) topk_cnt = c.topk_cnt;
 
     // Short contexts without an append: one launch, one workgroup per query row.
-    if (!append_count && !(select->flags & PQHSA_SELECT_GENERAL_PATH) &&
-        decode_small_fits(index->batch * index->kv_heads, G, n_max, index->num_lists, select->k_cap))
+    if (pqhsa_decode_step_launches(index, G, n_max, select, append_count != nullptr) == 1)
         return decode_small(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, n_max, full_max + select->k_cap, select,
                             scale, eps, topk_idx, topk_val, topk_cnt, c.emit_count, stream);
 

@@ -48,7 +48,7 @@ struct ScanArgs {
     uint2 *emit_pairs;        // [rows, emit_cap] (key, retrieval-local index)
     uint16_t *emit_aux;       // [rows, emit_cap] list id of the candidate (NULL: none)
     int64_t emit_cap;
-    float *mass;              // [BH, L, GP] accumulated with atomics (NULL: none)
+    float *mass;              // [BH, L, GP] accumulated with atomics (required by the decode step's scan)
     int stage_cap;            // candidates one wave stages in LDS per row before it writes straight to memory
     int tile_windows;         // the decode step's scan: 256-key windows per workgroup
 };

@@ -42,8 +42,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
     const size_t table_bytes = ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;
     unsigned char *after = smem + table_bytes;
     float *mass_s = reinterpret_cast<float *>(after);                      // [L][GP]
-    const bool want_mass = a.mass != nullptr;
-    const size_t mass_bytes = want_mass ? table_bytes : 0;
+    const size_t mass_bytes = table_bytes;
     uint32_t *wcnt_s = reinterpret_cast<uint32_t *>(after + mass_bytes);   // [waves][GP]
     uint32_t *base_s = wcnt_s + kWaves * 16;                           // [waves][GP]
     uint2 *stage_s = reinterpret_cast<uint2 *>(base_s + kWaves * 16);  // [waves][GP][stage_cap]
@@ -131,8 +130,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
     float nref2[GP];    // -reference * log2(e); -inf for padded rows so that their weights are 0
     uint32_t wcnt[GP];  // candidates this wave has staged per row (wave-uniform)
     constexpr float kLog2e = 1.4426950408889634f;
-    if (want_mass)
-        for (int i = tid; i < L * GP; i += TH) mass_s[i] = 0.0f;
+    for (int i = tid; i < L * GP; i += TH) mass_s[i] = 0.0f;
 #pragma unroll
     for (int g = 0; g < GP; ++g) {
         const uint32_t tk = a.thr_key ? a.thr_key[(size_t)bh * GP + g] : 0xffffffffu;  // no thresholds: no candidates
@@ -202,21 +200,29 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
                 for (int g = 0; g < GP; ++g) s[j][g] = -INFINITY;
             }
         }
-        uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
+        // The comparisons stay lane masks in scalar registers: whether the wave has any candidate is
+        // their union, and the per-lane bit sets are only built for the few windows that have one.
+        bool cand[4][GP];
         float e[4][GP];
-        bool any = false;
+        unsigned long long any = 0ull;
 #pragma unroll
         for (int g = 0; g < GP; ++g) {
-            emit_mask[g] = 0u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const bool cand = s[j][g] >= thr_f[g];
-                if (cand) emit_mask[g] |= 1u << j;
-                if (want_mass) e[j][g] = cand ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
+                cand[j][g] = s[j][g] >= thr_f[g];
+                any |= __ballot(cand[j][g]);
+                e[j][g] = cand[j][g] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
             }
-            any |= emit_mask[g] != 0u;
         }
-        if (__ballot(any) != 0ull) {  // wave-uniform
+        if (any != 0ull) {  // wave-uniform
+            uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
+#pragma unroll
+            for (int g = 0; g < GP; ++g) {
+                emit_mask[g] = 0u;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (cand[j][g]) emit_mask[g] |= 1u << j;
+            }
             // slot of every candidate inside its wave, per row: prefix sums of the lanes' counts,
             // two rows to a 32-bit word
             uint32_t excl[GP], tot[GP];
@@ -282,7 +288,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
         // One prefix sum over the lanes gives every run's total as a difference of two prefix
         // values: the last lane of a run adds its prefix, the first lane takes back the prefix of
         // the lane before it.  (Unordered keys only make more runs.)
-        if (want_mass) {
+        {
             const bool simple = lid[0] == lid[3] && lid[0] == lid[1] && lid[0] == lid[2];
             const int prev = dpp_move<kDppWaveShr1>((int)lid[0]);
             const int nxt = dpp_move<kDppWaveShl1>((int)lid[0]);
@@ -328,7 +334,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
         for (int w = 0; w < kWaves; ++w) total += wcnt_s[w * GP + tid];
         at = total ? atomicAdd(&a.emit_count[(size_t)bh * GP + tid], total) : 0u;
     }
-    if (want_mass) {
+    {
         float *dst = a.mass + (size_t)bh * L * GP;
         for (int i = tid; i < L * GP; i += TH) {
             const float v = mass_s[i];
@@ -367,6 +373,7 @@ static int emit_stage_cap(int GP) {
 
 int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t stream) {
     if (streams == 0 || n_max <= 0) return PQHSA_OK;
+    PQHSA_REQUIRE(a.mass, "scan_emit: no list-mass output");
     a.stage_cap = emit_stage_cap(GP);
     // about four workgroups per compute unit (256 units) over the launch, at least two windows per wave
     const int64_t windows = (n_max + kWaveKeys - 1) / kWaveKeys;
@@ -377,7 +384,7 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t
     a.tile_windows = (int)((windows + tiles - 1) / tiles);
     tiles = (windows + a.tile_windows - 1) / a.tile_windows;
     const size_t tbl = ((size_t)a.L * GP * sizeof(float) + 15) & ~(size_t)15;
-    size_t lds = tbl + (a.mass ? tbl : 0) + 2 * kScanWaves * 16 * sizeof(uint32_t) +
+    size_t lds = 2 * tbl + 2 * kScanWaves * 16 * sizeof(uint32_t) +
                  (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint2);
     if (a.emit_aux) lds += (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint16_t);
     PQHSA_REQUIRE(lds <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);

@@ -1742,27 +1742,49 @@ __global__ __launch_bounds__(kSelThreads) void decode_small_kernel(SmallArgs a) 
         if (tid == 0) { fin_s[0] = m; fin_s[1] = ms; }
     }
     __syncthreads();
+    // The fold over the 64 row groups and the 32 background parts, in two levels: eight slices of
+    // 128 threads take eight groups and four parts each, then 128 threads add the eight slices (one
+    // thread per output element over all 64 groups is a chain of 64 dependent LDS round trips).
+    constexpr int kSlices = kSelThreads / kD;
+    float *fold_num = ms_s + kBgParts;                 // [kSlices][128]
+    float *fold_bg = fold_num + kSlices * kD;          // [kSlices][128]
+    float *fold_den = fold_bg + kSlices * kD;          // [kSlices]
+    float m = fin_s[0];
+    const float ms = fin_s[1];
+    const bool bg_on = ms != 0.0f && ref1 > -INFINITY;
+    if (bg_on) m = fmaxf(m, ref1);
+    if (m != -INFINITY) {  // (uniform over the workgroup)
+        const int slice = tid / kD, d = tid % kD;
+        float num = 0.0f, den = 0.0f, bgv = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kGroups / kSlices; ++i) {
+            const int gi = slice * (kGroups / kSlices) + i;
+            const float mg = red_m[gi];
+            const float w = mg == -INFINITY ? 0.0f : __expf(mg - m);
+            num = __builtin_fmaf(red_acc[gi * kD + d], w, num);
+            den = __builtin_fmaf(red_l[gi], w, den);
+        }
+#pragma unroll
+        for (int i = 0; i < kBgParts / kSlices; ++i) bgv += bg_s[(slice * (kBgParts / kSlices) + i) * kD + d];
+        fold_num[slice * kD + d] = num;
+        fold_bg[slice * kD + d] = bgv;
+        if (d == 0) fold_den[slice] = den;
+    }
+    __syncthreads();
     if (tid < kD) {
-        float m = fin_s[0];
-        const float ms = fin_s[1];
-        const bool bg_on = ms != 0.0f && ref1 > -INFINITY;
-        if (bg_on) m = fmaxf(m, ref1);
         char *orow_p = a.out + ((size_t)b * a.H * a.G + (size_t)h * a.G + g) * kD * qesz;
         if (m == -INFINITY) {  // nothing to attend to
             store1_any(a.q_dtype, orow_p, tid, 0.0f);
         } else {
-            float num = 0.0f, den = 0.0f;
-            for (int gi = 0; gi < kGroups; ++gi) {
-                const float mg = red_m[gi];
-                const float w = mg == -INFINITY ? 0.0f : __expf(mg - m);
-                num = __builtin_fmaf(red_acc[gi * kD + tid], w, num);
-                den = __builtin_fmaf(red_l[gi], w, den);
+            float num = 0.0f, den = 0.0f, bgv = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < kSlices; ++sl) {
+                num += fold_num[sl * kD + tid];
+                bgv += fold_bg[sl * kD + tid];
+                den += fold_den[sl];
             }
             if (bg_on) {
                 const float f0 = __expf(ref1 - m);
-                float bgv = 0.0f;
-#pragma unroll
-                for (int part = 0; part < kBgParts; ++part) bgv += bg_s[part * kD + tid];
                 num = __builtin_fmaf(bgv, f0, num);
                 den = __builtin_fmaf(ms, f0, den);
             }

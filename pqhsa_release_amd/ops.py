@@ -475,6 +475,17 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     return out
 
 
+def decode_step_launches(index: DeviceIndex, groups: int, workspace: DecodeWorkspace, *, n_max: int | None = None,
+                         appending: bool = False, general_path: bool = False) -> int:
+    """Kernel launches ``decode_step`` makes for a step of this shape: 1 when the short-context
+    kernel serves it, else 5 (``pqhsa_decode_step_launches``).  No GPU work."""
+    sel = Select()
+    sel.k_cap = workspace.k_cap
+    sel.flags = _lib.SELECT_GENERAL_PATH if general_path else 0
+    n_max = index.n_max if n_max is None else int(n_max)
+    return int(_lib.load().pqhsa_decode_step_launches(index.ref(), groups, n_max, ctypes.byref(sel), int(appending)))
+
+
 class DecodeCall:
     """A decode step with every argument resolved once: ``run()`` is one C call.
 

@@ -40,3 +40,27 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.KvView) == 8 + 8 + 4 + 4 + 8 * 4 + 4 + 4 + 8
     assert ctypes.sizeof(_lib.Index) == 15 * 8 + 2 * 8 + 4 * 3 + 4
     assert ctypes.sizeof(_lib.Select) == 24
+
+
+def test_launch_count_follows_the_short_context_rule():
+    import ctypes
+
+    lib = _lib.load()
+    index, sel = _lib.Index(), _lib.Select()
+    index.batch, index.kv_heads, index.num_lists = 1, 8, 512
+    sel.k_cap = 328
+
+    def launches(groups, n_max, appending=0):
+        return lib.pqhsa_decode_step_launches(ctypes.byref(index), groups, n_max, ctypes.byref(sel), appending)
+
+    assert launches(4, 16384) == 1
+    assert launches(4, 16385) == 5            # more keys than a workgroup holds in registers
+    assert launches(4, 8192, appending=1) == 5
+    assert launches(16, 8192) == 1 and launches(16, 8192) == launches(16, 1)
+    index.batch = 3                           # 3 * 8 * 16 query rows > 256
+    assert launches(16, 8192) == 5
+    index.batch = 1
+    sel.flags = _lib.SELECT_GENERAL_PATH
+    assert launches(4, 8192) == 5
+    sel.flags, sel.k_cap = 0, 2049
+    assert launches(4, 8192) == 5
