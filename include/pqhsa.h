@@ -110,7 +110,9 @@ typedef struct pqhsa_select {
     int32_t topk;
     int32_t k_cap; /* row stride of topk_idx / topk_val; >= the largest k of the batch */
     int32_t flags; /* 0, or PQHSA_SELECT_GENERAL_PATH */
-    int32_t reserved;
+    int32_t n_mean; /* hint: mean number of indexed keys per sequence of the batch; 0 = unknown (n_max is
+                       assumed).  Sizes the scan's tiles so that a ragged batch still fills the chip;
+                       results do not depend on it. */
 } pqhsa_select;
 
 /* pqhsa_decode_step serves short contexts (at most 16 384 indexed keys per sequence, at most 256

@@ -64,7 +64,7 @@ class Index(ctypes.Structure):
 
 class Select(ctypes.Structure):
     _fields_ = [("fraction", ctypes.c_double), ("topk", c_int32), ("k_cap", c_int32), ("flags", c_int32),
-                ("reserved", c_int32)]
+                ("n_mean", c_int32)]
 
 
 SELECT_GENERAL_PATH = 1

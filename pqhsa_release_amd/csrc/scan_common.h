@@ -51,6 +51,7 @@ struct ScanArgs {
     float *mass;              // [BH, L, GP] accumulated with atomics (required by the decode step's scan)
     int stage_cap;            // candidates one wave stages in LDS per row before it writes straight to memory
     int tile_windows;         // the decode step's scan: 256-key windows per workgroup
+    int tile_major;           // ... and whether the grid is (streams, tiles) instead of (tiles, streams)
 };
 
 template <int GP>

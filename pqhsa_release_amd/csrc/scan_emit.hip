@@ -31,7 +31,12 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int bh = blockIdx.y;
+    // (Ragged batches are launched tile-major: the first tiles of all streams are dispatched before
+    // the later ones, which only the longest streams use.  The stream is rotated by the tile index,
+    // so that the tiles of one stream do not all land on the same eighth of the chip: workgroups go
+    // round the eight XCDs by their linear index, and a long stream would overfill its XCD.)
+    const int tile = a.tile_major ? blockIdx.y : blockIdx.x;
+    const int bh = a.tile_major ? (int)((blockIdx.x + blockIdx.y) % gridDim.x) : (int)blockIdx.y;
     const int L = a.L;
     [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
     PQHSA_TRACE_MARK(trace_scan, trace_wg, 0);
@@ -71,10 +76,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
         return k;
     };
     // the workgroup's tile of windows; wave w takes windows w, w + waves, ... of it
-    const int tile_end = ((int)blockIdx.x + 1) * a.tile_windows;
-    int win = (int)blockIdx.x * a.tile_windows + wave;
-    KeyWords cur = fetch(win);
+    const int tile_end = (tile + 1) * a.tile_windows;
+    int win = tile * a.tile_windows + wave;
+    // A tile past the end of its stream has nothing to do.  In a ragged batch (tile-major launch)
+    // there are many: they leave before they ask for anything but the count, so that their slots go
+    // to tiles with work at once.  Otherwise the first window is requested before the count is
+    // looked at, and a tile with work never waits for the count alone.
     const int n = min(a.n_arr[bh / a.n_div], (int)a.n_cap);
+    const bool idle = (int64_t)tile * a.tile_windows * kWaveKeys >= n;
+    if (a.tile_major && idle) return;  // (uniform over the workgroup)
+    KeyWords cur = fetch(win);
 
     float qn[GP];
     {
@@ -97,6 +108,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
                 const int i = tid + u * TH;
                 ls_r[u] = i < nvec ? ls[i] : make_float4(0, 0, 0, 0);
             }
+            if (idle) return;  // (uniform over the workgroup)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int i = tid + u * TH;
@@ -104,6 +116,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
             }
             for (int i = tid + 2 * TH; i < nvec; i += TH) reinterpret_cast<float4 *>(ls_s)[i] = ls[i];
         } else {
+            if (idle) return;  // (uniform over the workgroup)
             const float *ls = a.list_scores + (size_t)bh * L * GP;
             for (int i = tid; i < L * GP; i += TH) ls_s[i] = ls[i];
         }
@@ -371,24 +384,34 @@ static int emit_stage_cap(int GP) {
     return cap < 32 ? 32 : cap;
 }
 
-int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t stream) {
+// n_mean: the mean key count per stream when the caller knows it (0: every stream is taken to hold n_max)
+int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream) {
     if (streams == 0 || n_max <= 0) return PQHSA_OK;
     PQHSA_REQUIRE(a.mass, "scan_emit: no list-mass output");
     a.stage_cap = emit_stage_cap(GP);
-    // about four workgroups per compute unit (256 units) over the launch, at least two windows per wave
+    // About four workgroups WITH WORK per compute unit (256 units) over the launch, at least two
+    // windows per wave.  The grid covers the longest stream; in a ragged batch the tiles past a
+    // stream's end return at once, so the tile size follows the mean length, not the longest.
     const int64_t windows = (n_max + kWaveKeys - 1) / kWaveKeys;
-    int64_t tiles = (1024 + streams - 1) / streams;
-    const int64_t most = (windows + 2 * kScanWaves - 1) / (2 * kScanWaves);
+    if (n_mean <= 0 || n_mean > n_max) n_mean = n_max;
+    const int64_t windows_mean = (n_mean + kWaveKeys - 1) / kWaveKeys;
+    // (a ragged stream's last tile is part full: one tile per stream is set aside for that, so that
+    // the tiles with work still fit the chip at once)
+    const int64_t room = n_mean < n_max && streams < 256 ? 1024 - 2 * streams : 1024;
+    int64_t tiles = (room + streams - 1) / streams;  // ... per stream of mean length
+    if (n_mean < n_max && tiles * streams > room && tiles > 1) --tiles;
+    const int64_t most = (windows_mean + 2 * kScanWaves - 1) / (2 * kScanWaves);
     if (tiles > most) tiles = most;
     if (tiles < 1) tiles = 1;
-    a.tile_windows = (int)((windows + tiles - 1) / tiles);
+    a.tile_windows = (int)((windows_mean + tiles - 1) / tiles);
     tiles = (windows + a.tile_windows - 1) / a.tile_windows;
     const size_t tbl = ((size_t)a.L * GP * sizeof(float) + 15) & ~(size_t)15;
     size_t lds = 2 * tbl + 2 * kScanWaves * 16 * sizeof(uint32_t) +
                  (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint2);
     if (a.emit_aux) lds += (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint16_t);
     PQHSA_REQUIRE(lds <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);
-    dim3 grid((unsigned)tiles, streams);
+    a.tile_major = n_mean < n_max;
+    dim3 grid = a.tile_major ? dim3(streams, (unsigned)tiles) : dim3((unsigned)tiles, streams);
 #define PQHSA_EMIT_CASE(gp)                                                                                 \
     case gp: {                                                                                              \
         auto kern = scan_emit_kernel<gp>;                                                                   \
@@ -445,5 +468,5 @@ extern "C" int pqhsa_lut_scan_mass(const pqhsa_index *index, int32_t G, int32_t 
     a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = nullptr;
     a.n_cap = index->n_cap; a.n_arr = index->n_idx;
     a.thr_key = nullptr; a.ref_val = ref; a.mass = list_mass;
-    return launch_scan_emit(a, GP, streams, n_max, stream);
+    return launch_scan_emit(a, GP, streams, n_max, 0, stream);
 }

@@ -1223,6 +1223,8 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
     // losers' weights join the scan's per-list sums of the row (same reference), unless those have to start over
     float *mass_out = a.mass ? a.mass + (size_t)bh * a.L * a.GP + g : nullptr;
     const float ref0 = mass_out ? a.ref_val[row] : -INFINITY;
+    // (the scan's sum of this thread's first list is requested now and merged at the end: no round trip then)
+    const float scan_mass = (mass_out && tid < a.L) ? mass_out[(size_t)tid * a.GP] : 0.0f;
     // The estimate kept too few keys, or more than the candidate area holds: every stored key of
     // the row becomes a candidate, scored again on each pass of the selection, and the row's
     // background sums start over, relative to the k-th logit.
@@ -1287,7 +1289,7 @@ __global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a)
             const float f = fresh ? 0.0f : __expf(ref0 - ref1);
             for (int l = tid; l < a.L; l += kSelThreads) {
                 float *m = mass_out + (size_t)l * a.GP;
-                *m = fresh ? mx[l] : __builtin_fmaf(*m, f, mx[l]);
+                *m = fresh ? mx[l] : __builtin_fmaf(l == tid ? scan_mass : *m, f, mx[l]);
             }
             if (tid == 0) a.ref_val[row] = ref1;
         }
@@ -1870,7 +1872,7 @@ int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
     return rc;
 }
 
-int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, hipStream_t stream);
+int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream);
 
 // sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
 int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
@@ -1902,7 +1904,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
     a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = emit_cap;
     a.mass = mass;
-    rc = launch_scan_emit(a, GP, streams, n_max, stream);
+    rc = launch_scan_emit(a, GP, streams, n_max, select->n_mean, stream);
     if (rc) return rc;
     profile_mark(kProfSelect, stream);
     // 3. exact selection among the candidates

@@ -213,6 +213,11 @@ class DeviceIndex:
     def n_max(self) -> int:
         return max(self.n_host) if self.n_host else 0
 
+    @property
+    def n_mean(self) -> int:
+        """Mean indexed keys per sequence (host mirror): the hint that sizes the scan's tiles."""
+        return (sum(self.n_host) + len(self.n_host) - 1) // len(self.n_host) if self.n_host else 0
+
     def set_counts(self, counts) -> None:
         """Keys stored per sequence (a fresh encode leaves them in insertion order: nothing is
         sorted, nothing sampled, until ``finalize_layout``)."""
@@ -441,8 +446,11 @@ class DecodeWorkspace:
 def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceIndex, groups: int,
                 seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
                 scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None,
-                append_count: torch.Tensor | None = None, general_path: bool = False) -> torch.Tensor:
+                append_count: torch.Tensor | None = None, general_path: bool = False,
+                n_mean: int | None = None) -> torch.Tensor:
     """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``.
+    ``n_mean`` (default: the index's host-side mean key count) is the hint that sizes the scan's tiles
+    for ragged batches; results do not depend on it.
     Short contexts are served by a single kernel (same results); ``general_path`` keeps such a step
     on the five-kernel path (``PQHSA_SELECT_GENERAL_PATH``).
     With ``append_count`` (device int32 [B]) the step first appends one key to every sequence whose
@@ -461,6 +469,7 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     sel.topk = int(topk)
     sel.k_cap = workspace.k_cap
     sel.flags = _lib.SELECT_GENERAL_PATH if general_path else 0
+    sel.n_mean = index.n_mean if n_mean is None else max(0, min(int(n_mean), 2**31 - 1))
     n_max = index.n_max if n_max is None else int(n_max)
     args = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups, seq_lens.data_ptr(),
             int(sink), n_max, int(full_max), ctypes.byref(sel), float(scale), eps, workspace.topk_idx.data_ptr(),
@@ -513,6 +522,7 @@ class DecodeCall:
         self._sel.fraction = float(fraction) if fraction else 0.0
         self._sel.topk = int(topk)
         self._sel.k_cap = workspace.k_cap
+        self._sel.n_mean = index.n_mean
         self._keep = (q, out, kv, index, seq_lens, workspace, append_count)
         self.n_max = index.n_max if n_max is None else int(n_max)
         self.full_max = int(full_max)

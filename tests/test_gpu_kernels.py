@@ -628,6 +628,35 @@ def test_decode_step_graph_replays_match_eager_runs():
         assert torch.isfinite(junk)
 
 
+def test_ragged_batch_tile_hint_changes_no_result():
+    """The mean-length hint only sizes the scan's tiles (a ragged batch is then launched with the
+    tiles of all streams interleaved and the empty ones leaving at once): whatever it says, the
+    top-k set is the oracle's and the outputs agree."""
+    dev = _cuda()
+    p = Problem(lens=[9000, 2100, 5200, 400], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=71)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    q = p.q_tensor().float()
+    k_cap = ops.resolve_topk(p.n_max, 0.03, 0)
+    ws = ops.DecodeWorkspace(idx, p.G, k_cap)
+    want = {(b, h): p.oracle_step(b, h, 0.03)[1] for (b, h) in p.index}
+    first = None
+    for hint in (None, 0, 1, 300, p.n_max, 10 ** 9):
+        out = torch.empty_like(q)
+        ws.topk_idx.fill_(-1)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
+                        topk=0, scale=SCALE, workspace=ws, general_path=True, n_mean=hint)
+        torch.cuda.synchronize()
+        tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        for (b, h), want_idx in want.items():
+            for g in range(p.G):
+                assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (hint, b, h, g)
+        if first is None:
+            first = out.clone()
+        np.testing.assert_allclose(out.cpu().numpy(), first.cpu().numpy(), atol=2e-6, rtol=1e-5, err_msg=str(hint))
+    assert ws.rescans() == 0
+
+
 def test_fused_append_decode_steps_match_oracle_and_separate_append():
     """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
     the launch that builds the tables, attends over the grown index, and leaves the new count in
