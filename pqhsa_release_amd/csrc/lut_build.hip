@@ -21,12 +21,15 @@ PQHSA_TRACE_DECL(trace_lut)
 
 int lut_list_blocks(int num_lists);
 
-template <int DT>
+// MULTI: a block takes tiles_per_block > 1 tiles (compiled apart, so that the one-tile form keeps its registers)
+template <int DT, bool MULTI>
 __global__ __launch_bounds__(1024) void lut_build_kernel(
     const char *__restrict__ q, int H, int G, int Gp, const float *__restrict__ coarse,
     const float *__restrict__ codebooks, int L, float eps, float *__restrict__ qnorm,
     float *__restrict__ lut, float *__restrict__ list_scores, uint32_t *__restrict__ zero_base,
-    size_t zero_words, AppendFinish ap, int32_t *__restrict__ n_after, unsigned long long *__restrict__ nearest) {
+    size_t zero_words, AppendFinish ap, int32_t *__restrict__ n_after, unsigned long long *__restrict__ nearest,
+    int tiles_per_block_arg) {
+    const int tiles_per_block = MULTI ? tiles_per_block_arg : 1;
     __shared__ float kx[kD];
     __shared__ float kn_s;
     __shared__ float qh[kMaxG][kD];
@@ -40,19 +43,23 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
     [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
     PQHSA_TRACE_MARK(trace_lut, trace_wg, 0);
 
-    // list blocks: their 64 x 128 centroid tile (2048 float4, 8 per thread) is requested before
-    // anything else, so the loads are all in flight while the query rows are normalised
-    const int l0 = ((int)blockIdx.x - 1) * kListsPerBlock;
-    const int nl = blockIdx.x == 0 ? 0 : min(kListsPerBlock, L - l0);
+    // list blocks: a 64 x 128 centroid tile (2048 float4, 8 per thread) is requested before
+    // anything else, so the loads are all in flight while the query rows are normalised.  A block
+    // takes tiles_per_block tiles in turn (more than one in large batches, so that the launch still
+    // fits the chip at once); the next tile travels while the current one is used.
+    int l0 = ((int)blockIdx.x - 1) * tiles_per_block * kListsPerBlock;
+    const int l_end = blockIdx.x == 0 ? 0 : min(l0 + tiles_per_block * kListsPerBlock, L);
     float4 tile[8];
-    if (blockIdx.x != 0) {
-        const float4 *c4 = reinterpret_cast<const float4 *>(coarse + ((size_t)bh * L + l0) * kD);
+    auto fetch_tile = [&](int first) {
+        const int cnt = min(kListsPerBlock, l_end - first);
+        const float4 *c4 = reinterpret_cast<const float4 *>(coarse + ((size_t)bh * L + first) * kD);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = tid + u * nthr;
-            tile[u] = i < nl * (kD / 4) ? c4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            tile[u] = i < cnt * (kD / 4) ? c4[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
-    }
+    };
+    if (blockIdx.x != 0 && l0 < l_end) fetch_tile(l0);
 
     // scratch that the later kernels of a decode step accumulate into starts at zero
     if (zero_words) {
@@ -121,43 +128,53 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         return;
     }
 
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-        const int i = tid + u * nthr;
-        if (i >= kListsPerBlock * (kD / 4)) break;  // wider workgroups need fewer rounds
-        float *dst = &cs[i / (kD / 4)][(i % (kD / 4)) * 4];
-        dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
-    }
-    __syncthreads();
-    PQHSA_TRACE_MARK(trace_lut, trace_wg, 3);
     const int lane = tid % kListsPerBlock;
     const int wave = tid / kListsPerBlock;
-    float *out = list_scores + ((size_t)bh * L + l0) * Gp;
-    for (int g = wave; g < Gp; g += nthr / kListsPerBlock) {
-        if (lane >= nl) continue;
-        float acc = 0.0f;
-        if (g < G) {
-#pragma unroll 8
-            for (int d = 0; d < kD; ++d) acc = __builtin_fmaf(qh[g][d], cs[lane][d], acc);
+    const int tiles_of_stream = (L + kListsPerBlock - 1) / kListsPerBlock;
+    if (l0 < l_end) do {
+        const int nl = min(kListsPerBlock, l_end - l0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = tid + u * nthr;
+            if (i >= kListsPerBlock * (kD / 4)) break;  // wider workgroups need fewer rounds
+            float *dst = &cs[i / (kD / 4)][(i % (kD / 4)) * 4];
+            dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
         }
-        out[(size_t)lane * Gp + g] = acc;
-    }
-    if (appending && wave == 0) {
-        // nearest of this block's centroids to the new key: squared distance chain as in the encode
-        // kernels; its bit pattern orders like the value (>= 0) and the list id breaks ties low
-        unsigned long long key = ~0ull;
-        if (lane < nl) {
-            float d2 = 0.0f;
+        __syncthreads();
+        if constexpr (MULTI) {
+            if (l0 + kListsPerBlock < l_end) fetch_tile(l0 + kListsPerBlock);
+        }
+        PQHSA_TRACE_MARK(trace_lut, trace_wg, 3);
+        float *out = list_scores + ((size_t)bh * L + l0) * Gp;
+        for (int g = wave; g < Gp; g += nthr / kListsPerBlock) {
+            if (lane >= nl) continue;
+            float acc = 0.0f;
+            if (g < G) {
 #pragma unroll 8
-            for (int d = 0; d < kD; ++d) {
-                const float t = kx[d] - cs[lane][d];
-                d2 = __builtin_fmaf(t, t, d2);
+                for (int d = 0; d < kD; ++d) acc = __builtin_fmaf(qh[g][d], cs[lane][d], acc);
             }
-            key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)(l0 + lane);
+            out[(size_t)lane * Gp + g] = acc;
         }
-        key = wave_min_u64(key, kWave);
-        if (lane == 0) nearest[(size_t)bh * (gridDim.x - 1) + (blockIdx.x - 1)] = key;
-    }
+        if (appending && wave == 0) {
+            // nearest of this tile's centroids to the new key: squared distance chain as in the encode
+            // kernels; its bit pattern orders like the value (>= 0) and the list id breaks ties low
+            unsigned long long key = ~0ull;
+            if (lane < nl) {
+                float d2 = 0.0f;
+#pragma unroll 8
+                for (int d = 0; d < kD; ++d) {
+                    const float t = kx[d] - cs[lane][d];
+                    d2 = __builtin_fmaf(t, t, d2);
+                }
+                key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)(l0 + lane);
+            }
+            key = wave_min_u64(key, kWave);
+            if (lane == 0) nearest[(size_t)bh * tiles_of_stream + l0 / kListsPerBlock] = key;
+        }
+        if constexpr (!MULTI) break;
+        l0 += kListsPerBlock;
+        if (l0 < l_end) __syncthreads();  // (uniform; the tile is overwritten by the next one)
+    } while (l0 < l_end);
     PQHSA_TRACE_MARK(trace_lut, trace_wg, 4);
 }
 
@@ -176,17 +193,30 @@ int launch_lut_build(const void *q, int q_dtype, const pqhsa_index *index, int G
         PQHSA_REQUIRE(n_after && nearest, "lut_build: the fused append needs its scratch arrays");
         ap = *append;
     }
-    dim3 grid(1 + lut_list_blocks(index->num_lists), BH);
+    // One tile of 64 lists per block while the launch fits the chip at once (three blocks per
+    // compute unit, by their LDS); in larger batches a block takes several tiles in turn.
+    const int tiles = lut_list_blocks(index->num_lists);
+    int per_block = 1;
+    while (per_block < tiles && (int64_t)BH * (1 + (tiles + per_block - 1) / per_block) > 3 * 256) ++per_block;
+    dim3 grid(1 + (tiles + per_block - 1) / per_block, BH);
     const int threads = Gp * kWave > kLutThreads ? Gp * kWave : kLutThreads;  // a wave per padded query row
-    PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL(lut_build_kernel<DT>, grid, dim3(threads), 0, stream,
-                                                     static_cast<const char *>(q), index->kv_heads, G, Gp,
-                                                     index->coarse, index->codebooks, index->num_lists, eps,
-                                                     qnorm, lut, list_scores, zero_base, zero_words, ap, n_after,
-                                                     nearest));
+    if (per_block == 1) {
+        PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL((lut_build_kernel<DT, false>), grid, dim3(threads), 0, stream,
+                                                          static_cast<const char *>(q), index->kv_heads, G, Gp,
+                                                          index->coarse, index->codebooks, index->num_lists, eps,
+                                                          qnorm, lut, list_scores, zero_base, zero_words, ap, n_after,
+                                                          nearest, 1));
+    } else {
+        PQHSA_DISPATCH_DTYPE(q_dtype, hipLaunchKernelGGL((lut_build_kernel<DT, true>), grid, dim3(threads), 0, stream,
+                                                          static_cast<const char *>(q), index->kv_heads, G, Gp,
+                                                          index->coarse, index->codebooks, index->num_lists, eps,
+                                                          qnorm, lut, list_scores, zero_base, zero_words, ap, n_after,
+                                                          nearest, per_block));
+    }
     return check_launch("lut_build");
 }
 
-// list blocks of one stream in the table-building launch (each takes 64 coarse lists)
+// tiles of 64 coarse lists of one stream in the table-building launch
 int lut_list_blocks(int num_lists) { return (num_lists + kListsPerBlock - 1) / kListsPerBlock; }
 
 }  // namespace pqhsa

@@ -99,6 +99,27 @@ def test_lut_build_and_scan_match_oracle_bitwise(groups, dtype):
         assert np.array_equal(got, want), (b, h, np.abs(got - want).max())
 
 
+def test_lut_build_large_batch_takes_several_tiles_per_block():
+    """With many streams the table-building launch gives a block several 64-list tiles in turn
+    (so that it still fits the chip at once): same bits as the oracle, last partial tile included."""
+    dev = _cuda()
+    batch, heads, groups, lists = 30, 4, 4, 488      # 120 streams x (1 + 8 tiles) blocks would not fit at once
+    idx = ops.DeviceIndex(batch, heads, lists, 64, dev)
+    gen = torch.Generator(device="cpu").manual_seed(91)
+    idx.coarse.copy_(torch.randn(idx.coarse.shape, generator=gen))
+    idx.codebooks.copy_(0.3 * torch.randn(idx.codebooks.shape, generator=gen))
+    q = torch.randn(batch, heads * groups, DIM, generator=gen)
+    qnorm, lut, ls = ops.lut_build(q.to(dev), idx, groups)
+    torch.cuda.synchronize()
+    coarse, books = idx.coarse.cpu().numpy(), idx.codebooks.cpu().numpy()
+    for bh in (0, 1, 57, 118, 119):
+        b, h = divmod(bh, heads)
+        oq, olut, ols = fixed.lut_build(q[b, h * groups : (h + 1) * groups].numpy(), coarse[bh], books[bh])
+        assert np.array_equal(qnorm[bh, :groups].cpu().numpy(), oq), bh
+        assert np.array_equal(lut[bh, :, :, :groups].permute(2, 0, 1).cpu().numpy(), olut), bh
+        assert np.array_equal(ls[bh, :, :groups].T.cpu().numpy(), ols), bh
+
+
 @pytest.mark.parametrize("stride_pad,offset", [(0, 0), (3, 0), (0, 1), (5, 3)])
 def test_lut_scan_row_stride_and_alignment(stride_pad, offset):
     # The scan writes four neighbouring logits as one 16-byte store when the destination allows it;
@@ -657,13 +678,20 @@ def test_ragged_batch_tile_hint_changes_no_result():
     assert ws.rescans() == 0
 
 
-def test_fused_append_decode_steps_match_oracle_and_separate_append():
+@pytest.mark.parametrize("shape", [
+    dict(steps=5, lens=[1805, 1505], heads=2, groups=4, lists=32, every=1),
+    # 64 streams x 13 table blocks: the table-building launch gives a block two tiles of lists, and the
+    # appended key's nearest list is found over the tiles' answers (a sample of the streams is checked)
+    dict(steps=2, lens=[862, 852, 847, 842, 872, 882, 843, 854], heads=8, groups=2, lists=768, every=9),
+], ids=["small", "many_streams"])
+def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
     the launch that builds the tables, attends over the grown index, and leaves the new count in
     device memory.  Checked against the oracle on the same prefix of the context."""
     dev = _cuda()
-    steps, len0 = 5, 1800
-    p = Problem(lens=[len0 + steps, len0 + steps - 300], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=47)
+    steps = shape["steps"]
+    p = Problem(lens=shape["lens"], heads=shape["heads"], groups=shape["groups"], lists=shape["lists"],
+                dtype=torch.bfloat16, seed=47)
     lens0 = [ln - steps for ln in p.lens]
     n0 = [p.n(b) - steps for b in range(p.B)]
     kv = ops.kv_paged(*p.paged_kv("5d"))
@@ -694,6 +722,8 @@ def test_fused_append_decode_steps_match_oracle_and_separate_append():
             codes, lists, norms = idx.by_key(bh, n)
             assert np.array_equal(u32(codes), ix["codes"][:n]) and np.array_equal(u16(lists), ix["list_ids"][:n])
             assert np.array_equal(norms.cpu().numpy(), ix["norms"][:n])
+            if bh % shape["every"]:
+                continue
             _, _, vbar = fixed.value_summaries(p.values[b, h][p.sink : p.sink + n].numpy(), ix["list_ids"][:n], p.L)
             np.testing.assert_allclose(idx.vbar[bh].cpu().numpy(), vbar, rtol=1e-6, atol=1e-6)
             part = {"coarse": ix["coarse"], "codebooks": ix["codebooks"], "codes": ix["codes"][:n],
