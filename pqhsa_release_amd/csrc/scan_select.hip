@@ -1186,8 +1186,11 @@ __device__ inline void select_stream(const Records &src, uint32_t cnt, int k, Se
 // RS > 0: the host expects at most RS * 1024 candidates per row, and the kernel requests that many
 // candidate slots before it knows the count, together with the count itself (one round trip to
 // memory instead of two); slots past the count hold leftovers of earlier steps and are masked.
-template <int RS>
-__global__ __launch_bounds__(kSelThreads) void select_final_kernel(SelectArgs a) {
+// PACK: compiled for two workgroups per compute unit (fewer scalar registers), for batches of
+// more than 256 query rows; with fewer rows the dispatcher would pair workgroups on one unit
+// while others stand idle, so those take the form that fills a unit alone.
+template <int RS, bool PACK = false>
+__global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel(SelectArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ __align__(16) uint32_t red[2][kSelWaves];
     __shared__ uint32_t wsum[2 * kSelWaves];
@@ -1420,6 +1423,10 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     const size_t lds = (size_t)(kM * kCodes + 2 * a.L) * sizeof(float);
     const dim3 grid(a.G, streams), block(kSelThreads);
     if (a.expected_candidates <= 0) hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
+    else if (a.expected_candidates <= 8 * kSelThreads && (int64_t)a.G * streams > 256) {
+        if (a.expected_candidates <= 4 * kSelThreads) hipLaunchKernelGGL((select_final_kernel<4, true>), grid, block, lds, stream, a);
+        else hipLaunchKernelGGL((select_final_kernel<8, true>), grid, block, lds, stream, a);
+    }
     else if (a.expected_candidates <= 4 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<4>, grid, block, lds, stream, a);
     else if (a.expected_candidates <= 8 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<8>, grid, block, lds, stream, a);
     else if (a.expected_candidates <= 16 * kSelThreads) hipLaunchKernelGGL(select_final_kernel<16>, grid, block, lds, stream, a);

@@ -805,6 +805,37 @@ def test_decode_step_random_shapes_match_oracle(seed):
             assert ws.rescans() == 0, what
 
 
+def test_decode_step_batch_of_more_than_256_query_rows():
+    """288 query rows (9 sequences x 8 KV heads x 4): the selection kernel then runs in the form
+    that shares a compute unit between two workgroups, and the short-context kernel does not
+    apply.  A sample of the streams against the oracle, all rows for sane counts."""
+    dev = _cuda()
+    lens = [2400, 1300, 1900, 2100, 900, 1700, 2300, 1100, 1500]
+    p = Problem(lens=lens, heads=8, groups=4, lists=32, dtype=torch.bfloat16, seed=83)
+    idx = p.device_index(dev)
+    kv = ops.kv_paged(*p.paged_kv("5d"))
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.04, 0))
+    q = p.q_tensor().float()
+    out = torch.empty_like(q)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.04,
+                    topk=0, scale=SCALE, workspace=ws)
+    torch.cuda.synchronize()
+    assert ops.decode_step_launches(idx, p.G, ws) == 5
+    tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+    cnt = ws.topk_cnt.cpu().numpy().reshape(p.B, p.H, p.G)
+    o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    for b in range(p.B):
+        assert (cnt[b] == ops.resolve_topk(p.n(b), 0.04, 0)).all(), b
+    for i, (b, h) in enumerate(p.index):
+        if i % 7:
+            continue
+        want_out, want_idx, _ = p.oracle_step(b, h, 0.04)
+        for g in range(p.G):
+            assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (b, h, g)
+        assert np.abs(o[b, h] - want_out).max() <= 2e-3, (b, h)
+    assert ws.rescans() == 0
+
+
 @pytest.mark.parametrize("general_path", [False, True])
 @pytest.mark.parametrize("groups,lists,lens", [(16, 64, [2600]), (12, 256, [5000, 1700]), (9, 512, [7000])])
 def test_decode_step_wide_groups_and_many_lists(groups, lists, lens, general_path):
