@@ -997,6 +997,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
     for (int r = 0; r < R; ++r) {
         const uint32_t p = (uint32_t)r * kSelThreads + tid;
         const bool real = p < cnt;
+        if (__ballot(real) == 0ull) continue;  // (wave-uniform) slots past the count: nothing to place, no weight to leave
         const bool wins = real && k > 0 && key[r] >= tkey;
         if (wins) out.winner(at++, key[r], where[r]);
         if (out.mx) {
