@@ -30,11 +30,13 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
     size_t zero_words, AppendFinish ap, int32_t *__restrict__ n_after, unsigned long long *__restrict__ nearest,
     int tiles_per_block_arg) {
     const int tiles_per_block = MULTI ? tiles_per_block_arg : 1;
-    __shared__ float kx[kD];
+    __shared__ __align__(16) float kx[kD];
     __shared__ float kn_s;
-    __shared__ float qh[kMaxG][kD];
+    __shared__ __align__(16) float qh[kMaxG][kD];
     __shared__ float qn[kMaxG];
-    __shared__ float cs[kListsPerBlock][kD + 1];
+    // a row stride of 132 floats keeps the rows 16-byte aligned and lets the 64 lanes of a wave read
+    // their own row 16 bytes at a time without meeting in a bank (eight lanes x four banks per pass)
+    __shared__ __align__(16) float cs[kListsPerBlock][kD + 4];
 
     const int tid = threadIdx.x;
     const int nthr = blockDim.x;
@@ -137,8 +139,7 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         for (int u = 0; u < 8; ++u) {
             const int i = tid + u * nthr;
             if (i >= kListsPerBlock * (kD / 4)) break;  // wider workgroups need fewer rounds
-            float *dst = &cs[i / (kD / 4)][(i % (kD / 4)) * 4];
-            dst[0] = tile[u].x; dst[1] = tile[u].y; dst[2] = tile[u].z; dst[3] = tile[u].w;
+            *reinterpret_cast<float4 *>(&cs[i / (kD / 4)][(i % (kD / 4)) * 4]) = tile[u];
         }
         __syncthreads();
         if constexpr (MULTI) {
@@ -149,9 +150,16 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
         for (int g = wave; g < Gp; g += nthr / kListsPerBlock) {
             if (lane >= nl) continue;
             float acc = 0.0f;
-            if (g < G) {
+            if (g < G) {  // the chain runs over d in order, four elements per LDS read
 #pragma unroll 8
-                for (int d = 0; d < kD; ++d) acc = __builtin_fmaf(qh[g][d], cs[lane][d], acc);
+                for (int d4 = 0; d4 < kD / 4; ++d4) {
+                    const float4 c = *reinterpret_cast<const float4 *>(&cs[lane][4 * d4]);
+                    const float4 qq = *reinterpret_cast<const float4 *>(&qh[g][4 * d4]);
+                    acc = __builtin_fmaf(qq.x, c.x, acc);
+                    acc = __builtin_fmaf(qq.y, c.y, acc);
+                    acc = __builtin_fmaf(qq.z, c.z, acc);
+                    acc = __builtin_fmaf(qq.w, c.w, acc);
+                }
             }
             out[(size_t)lane * Gp + g] = acc;
         }
@@ -162,9 +170,13 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
             if (lane < nl) {
                 float d2 = 0.0f;
 #pragma unroll 8
-                for (int d = 0; d < kD; ++d) {
-                    const float t = kx[d] - cs[lane][d];
-                    d2 = __builtin_fmaf(t, t, d2);
+                for (int d4 = 0; d4 < kD / 4; ++d4) {
+                    const float4 c = *reinterpret_cast<const float4 *>(&cs[lane][4 * d4]);
+                    const float4 x = *reinterpret_cast<const float4 *>(&kx[4 * d4]);
+                    float t = x.x - c.x; d2 = __builtin_fmaf(t, t, d2);
+                    t = x.y - c.y; d2 = __builtin_fmaf(t, t, d2);
+                    t = x.z - c.z; d2 = __builtin_fmaf(t, t, d2);
+                    t = x.w - c.w; d2 = __builtin_fmaf(t, t, d2);
                 }
                 key = ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)(l0 + lane);
             }
