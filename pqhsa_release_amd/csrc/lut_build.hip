@@ -88,18 +88,22 @@ __global__ __launch_bounds__(1024) void lut_build_kernel(
     }
     __syncthreads();
     PQHSA_TRACE_MARK(trace_lut, trace_wg, 1);
-    if (tid < G) {
+    // (sum of squares: one chain over d in order, the row read 16 bytes at a time)
+    auto norm_of = [](const float *row, float floor_) {
         float ss = 0.0f;
-        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(qh[tid][d], qh[tid][d], ss);
-        float n = sqrtf(ss);
-        qn[tid] = n < eps ? eps : n;
-    }
-    if (appending && tid == kMaxG) {  // one more thread: the new key's norm, same chain as the encode kernels
-        float ss = 0.0f;
-        for (int d = 0; d < kD; ++d) ss = __builtin_fmaf(kx[d], kx[d], ss);
-        float n = sqrtf(ss);
-        kn_s = n < ap.enc.eps ? ap.enc.eps : n;
-    }
+#pragma unroll 8
+        for (int d4 = 0; d4 < kD / 4; ++d4) {
+            const float4 x = *reinterpret_cast<const float4 *>(row + 4 * d4);
+            ss = __builtin_fmaf(x.x, x.x, ss);
+            ss = __builtin_fmaf(x.y, x.y, ss);
+            ss = __builtin_fmaf(x.z, x.z, ss);
+            ss = __builtin_fmaf(x.w, x.w, ss);
+        }
+        const float n = sqrtf(ss);
+        return n < floor_ ? floor_ : n;
+    };
+    if (tid < G) qn[tid] = norm_of(qh[tid], eps);
+    if (appending && tid == kMaxG) kn_s = norm_of(kx, ap.enc.eps);  // one more thread: the new key's norm, same chain as the encode kernels
     __syncthreads();
     for (int i = tid; i < G * kD; i += nthr) {
         int g = i / kD, d = i % kD;

@@ -1532,9 +1532,16 @@ __global__ __launch_bounds__(kSelThreads) void decode_small_kernel(SmallArgs a) 
     if (tid == 0) ss.cont_count = 0u;
     __syncthreads();
     PQHSA_TRACE_MARK(trace_small, trace_wg, 1);
-    if (tid == 0) {
+    if (tid == 0) {  // one chain over d in order, the row read 16 bytes at a time
         float ss2 = 0.0f;
-        for (int d = 0; d < kD; ++d) ss2 = __builtin_fmaf(qh[d], qh[d], ss2);
+#pragma unroll 8
+        for (int d4 = 0; d4 < kD / 4; ++d4) {
+            const float4 x = *reinterpret_cast<const float4 *>(&qh[4 * d4]);
+            ss2 = __builtin_fmaf(x.x, x.x, ss2);
+            ss2 = __builtin_fmaf(x.y, x.y, ss2);
+            ss2 = __builtin_fmaf(x.z, x.z, ss2);
+            ss2 = __builtin_fmaf(x.w, x.w, ss2);
+        }
         const float nq = sqrtf(ss2);
         qn_s = nq < a.eps ? a.eps : nq;
     }
