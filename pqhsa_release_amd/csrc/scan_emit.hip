@@ -400,7 +400,9 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
     const int64_t room = n_mean < n_max && streams < 256 ? 1024 - 2 * streams : 1024;
     int64_t tiles = (room + streams - 1) / streams;  // ... per stream of mean length
     if (n_mean < n_max && tiles * streams > room && tiles > 1) --tiles;
-    const int64_t most = (windows_mean + 2 * kScanWaves - 1) / (2 * kScanWaves);
+    // (a launch that fills at most half the chip anyway goes down to one window per wave)
+    const int64_t one_each = (windows_mean + kScanWaves - 1) / kScanWaves;
+    const int64_t most = one_each * streams <= 512 ? one_each : (windows_mean + 2 * kScanWaves - 1) / (2 * kScanWaves);
     if (tiles > most) tiles = most;
     if (tiles < 1) tiles = 1;
     a.tile_windows = (int)((windows_mean + tiles - 1) / tiles);
