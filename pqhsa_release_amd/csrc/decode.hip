@@ -35,7 +35,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
                   float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
-                  hipStream_t stream);
+                  bool even_rows, hipStream_t stream);
 size_t attend_partials_bytes(int rows, int k_cap);
 size_t attend_arrive_bytes(int rows);
 
@@ -197,7 +197,9 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials, c.arrive,
                          append_count ? c.n_after : nullptr,
-                         append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
+                         append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr,
+                         // rows of about one length (mean key count known and within an eighth of the longest)
+                         select->n_mean > 0 && (int64_t)select->n_mean * 8 >= (int64_t)n_max * 7, stream);
 }
 
 extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
