@@ -51,7 +51,8 @@ struct ScanArgs {
     float *mass;              // [BH, L, GP] accumulated with atomics (required by the decode step's scan)
     int stage_cap;            // candidates one wave stages in LDS per row before it writes straight to memory
     int tile_windows;         // the decode step's scan: 256-key windows per workgroup
-    int tile_major;           // ... and whether the grid is (streams, tiles) instead of (tiles, streams)
+    int tile_major;           // ... and the launch form: 0 grid (tiles, streams), 1 grid (streams, tiles), 2 packed
+    int seqs;                 // ... and the number of sequences (streams / n_div), for the packed form
 };
 
 template <int GP>

@@ -31,12 +31,35 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    // (Ragged batches are launched tile-major: the first tiles of all streams are dispatched before
-    // the later ones, which only the longest streams use.  The stream is rotated by the tile index,
-    // so that the tiles of one stream do not all land on the same eighth of the chip: workgroups go
-    // round the eight XCDs by their linear index, and a long stream would overfill its XCD.)
-    const int tile = a.tile_major ? blockIdx.y : blockIdx.x;
-    const int bh = a.tile_major ? (int)((blockIdx.x + blockIdx.y) % gridDim.x) : (int)blockIdx.y;
+    // Which tile of which stream this workgroup takes.  An even batch is launched as a grid of
+    // (tiles, streams).  A ragged batch is launched PACKED: one row of workgroups covers the tiles
+    // that hold work, sequence after sequence (within a sequence tile-major, so that its streams
+    // alternate), and the workgroups past the last such tile leave at once.  All tiles with work are
+    // then dispatched before any idle one: idle workgroups in between hold up the dispatch of the
+    // ones behind them, and a launch whose tiles with work would have fitted the chip at once took a
+    // second round.  (Workgroups go round the eight XCDs by their linear index, so the packed order
+    // also spreads every stream over all of them.)  Batches of very many sequences are launched
+    // tile-major instead, as a grid of (streams, tiles) with the stream rotated by the tile index.
+    int tile, bh;
+    if (a.tile_major == 2) {
+        int first = 0, b = 0;
+        for (; b < a.seqs; ++b) {
+            const int windows = (min(a.n_arr[b], (int)a.n_cap) + kWaveKeys - 1) / kWaveKeys;
+            const int held = (windows + a.tile_windows - 1) / a.tile_windows * a.n_div;
+            if ((int)blockIdx.x < first + held) break;
+            first += held;
+        }
+        if (b == a.seqs) return;  // (uniform over the workgroup)
+        const int j = blockIdx.x - first;
+        tile = j / a.n_div;
+        bh = b * a.n_div + j % a.n_div;
+    } else if (a.tile_major) {
+        tile = blockIdx.y;
+        bh = (int)((blockIdx.x + blockIdx.y) % gridDim.x);
+    } else {
+        tile = blockIdx.x;
+        bh = blockIdx.y;
+    }
     const int L = a.L;
     [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
     PQHSA_TRACE_MARK(trace_scan, trace_wg, 0);
@@ -78,9 +101,9 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
     // the workgroup's tile of windows; wave w takes windows w, w + waves, ... of it
     const int tile_end = (tile + 1) * a.tile_windows;
     int win = tile * a.tile_windows + wave;
-    // A tile past the end of its stream has nothing to do.  In a ragged batch (tile-major launch)
-    // there are many: they leave before they ask for anything but the count, so that their slots go
-    // to tiles with work at once.  Otherwise the first window is requested before the count is
+    // A tile past the end of its stream has nothing to do.  In a tile-major launch there are many:
+    // they leave before they ask for anything but the count, so that their slots go to tiles with
+    // work at once.  Otherwise the first window is requested before the count is
     // looked at, and a tile with work never waits for the count alone.
     const int n = min(a.n_arr[bh / a.n_div], (int)a.n_cap);
     const bool idle = (int64_t)tile * a.tile_windows * kWaveKeys >= n;
@@ -379,6 +402,9 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
 
 // per-wave, per-row staging capacity: sparse windows are staged, a window that does not fit
 // writes straight to memory, so a small area is enough
+// a packed launch walks the sequences' key counts in every workgroup: only for batches this small
+constexpr int kPackedSeqs = 64;
+
 static int emit_stage_cap(int GP) {
     const int cap = 256 / GP;
     return cap < 32 ? 32 : cap;
@@ -395,11 +421,15 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
     const int64_t windows = (n_max + kWaveKeys - 1) / kWaveKeys;
     if (n_mean <= 0 || n_mean > n_max) n_mean = n_max;
     const int64_t windows_mean = (n_mean + kWaveKeys - 1) / kWaveKeys;
-    // (a ragged stream's last tile is part full: one tile per stream is set aside for that, so that
-    // the tiles with work still fit the chip at once)
-    const int64_t room = n_mean < n_max && streams < 256 ? 1024 - 2 * streams : 1024;
+    // (a ragged stream's last tile is part full: one tile per stream is set aside for that, two in a
+    // tile-major launch, so that the tiles with work still fit the chip at once)
+    const bool ragged = n_mean < n_max;
+    const int seqs = streams / a.n_div;
+    const bool packed = ragged && seqs * a.n_div == streams && seqs <= kPackedSeqs;
+    const int64_t spare = !ragged || streams >= 256 ? 0 : packed ? streams : 2 * streams;
+    const int64_t room = 1024 - spare;
     int64_t tiles = (room + streams - 1) / streams;  // ... per stream of mean length
-    if (n_mean < n_max && tiles * streams > room && tiles > 1) --tiles;
+    if (ragged && tiles * streams > room && tiles > 1) --tiles;
     // (a launch that fills at most half the chip anyway goes down to one window per wave)
     const int64_t one_each = (windows_mean + kScanWaves - 1) / kScanWaves;
     const int64_t most = one_each * streams <= 512 ? one_each : (windows_mean + 2 * kScanWaves - 1) / (2 * kScanWaves);
@@ -412,8 +442,10 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
                  (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint2);
     if (a.emit_aux) lds += (size_t)kScanWaves * GP * a.stage_cap * sizeof(uint16_t);
     PQHSA_REQUIRE(lds <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);
-    a.tile_major = n_mean < n_max;
-    dim3 grid = a.tile_major ? dim3(streams, (unsigned)tiles) : dim3((unsigned)tiles, streams);
+    a.tile_major = packed ? 2 : ragged ? 1 : 0;
+    a.seqs = seqs;
+    dim3 grid = packed ? dim3((unsigned)(tiles * streams))
+                       : ragged ? dim3(streams, (unsigned)tiles) : dim3((unsigned)tiles, streams);
 #define PQHSA_EMIT_CASE(gp)                                                                                 \
     case gp: {                                                                                              \
         auto kern = scan_emit_kernel<gp>;                                                                   \

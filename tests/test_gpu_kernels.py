@@ -649,12 +649,16 @@ def test_decode_step_graph_replays_match_eager_runs():
         assert torch.isfinite(junk)
 
 
-def test_ragged_batch_tile_hint_changes_no_result():
+@pytest.mark.parametrize("lens, heads", [
+    ([9000, 2100, 5200, 400], 2),                                   # packed launch: tiles with work first
+    ([300 + (977 * i) % 2100 for i in range(66)], 1),               # over 64 sequences: tile-major launch
+], ids=["packed", "tile_major"])
+def test_ragged_batch_tile_hint_changes_no_result(lens, heads):
     """The mean-length hint only sizes the scan's tiles (a ragged batch is then launched with the
-    tiles of all streams interleaved and the empty ones leaving at once): whatever it says, the
+    tiles that hold work ahead of the empty ones, which leave at once): whatever it says, the
     top-k set is the oracle's and the outputs agree."""
     dev = _cuda()
-    p = Problem(lens=[9000, 2100, 5200, 400], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=71)
+    p = Problem(lens=lens, heads=heads, groups=4, lists=32, dtype=torch.bfloat16, seed=71)
     idx = p.device_index(dev)
     kv = ops.kv_paged(*p.paged_kv("5d"))
     q = p.q_tensor().float()
