@@ -138,6 +138,20 @@ int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink
                  void *stream);
 
 /*
+ * pqhsa_encode for many rows at once, with the same results bit for bit (same reference
+ * functions: IVFPQIndex.build_with_codebooks, pq_hsa/index/ivfpq.py:350-433, and the re-encode of
+ * IVFPQIndex.online_refresh, ivfpq.py:696-703).  The distances of a key to all coarse centroids
+ * are first estimated by a half-precision matrix product (MFMA) with a proven error bound, which
+ * leaves two lists per key (rarely: all) to be measured in the oracle's fixed fp32 order.
+ * num_lists <= 4096.  workspace: 256-byte aligned device memory of at least
+ * pqhsa_encode_bulk_workspace_bytes(B, H, num_lists, count_max) bytes, used during the call only.
+ */
+size_t pqhsa_encode_bulk_workspace_bytes(int32_t B, int32_t H, int32_t num_lists, int32_t count_max);
+int pqhsa_encode_bulk(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,
+                      const int32_t *slot0, const int32_t *count, int32_t count_max, float eps,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Rebuild vsum / vcount / vbar from the values of all indexed keys
  * (SparseKVCache._build_retrieval_value_summaries, pq_hsa/attention/kv_cache.py:688-728).
  * n_max >= max_b n_idx[b] sizes the launch (<= 0: n_cap).  Three launches: clear, accumulate

@@ -82,6 +82,9 @@ SIGNATURES = {
     "pqhsa_last_error": (ctypes.c_char_p, []),
     "pqhsa_padded_groups": (c_int32, [c_int32]),
     "pqhsa_encode": (ctypes.c_int, [_P(KvView), _P(Index), c_int32, c_void_p, c_void_p, c_int32, c_float, c_void_p]),
+    "pqhsa_encode_bulk_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "pqhsa_encode_bulk": (ctypes.c_int, [_P(KvView), _P(Index), c_int32, c_void_p, c_void_p, c_int32, c_float,
+                                         c_void_p, c_size_t, c_void_p]),
     "pqhsa_value_summaries": (ctypes.c_int, [_P(KvView), _P(Index), c_int32, c_int32, c_void_p]),
     "pqhsa_encode_append": (ctypes.c_int, [_P(KvView), _P(Index), c_int32, c_void_p, c_void_p, c_int32, c_float,
                                            c_void_p]),

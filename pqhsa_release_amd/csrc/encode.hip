@@ -9,10 +9,17 @@
 
 namespace pqhsa {
 
+__device__ inline float lane_value(float v, int lane) {  // lane: the same in every lane of the wave
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
+
 // One thread per key row; coarse centroids pass through LDS in chunks shared by the block.
-template <int DT>
-__global__ __launch_bounds__(kEncThreads, 3) void encode_bulk_kernel(EncodeArgs a) {
-    __shared__ __align__(16) float cs[kCoarseChunk][kD];
+// HINT: the key's nearest list is known to be one of two (a.hints, from the matrix-core estimate of
+// all distances), and only those are measured; a key whose hint says so still measures all lists,
+// from memory.  Either way the list is the first strict minimum of the same fixed-order distances.
+template <int DT, bool HINT>
+__global__ __launch_bounds__(kEncThreads, HINT ? 2 : 3) void encode_bulk_kernel(EncodeArgs a) {
+    __shared__ __align__(16) float cs[HINT ? 1 : kCoarseChunk][kD];
     __shared__ __align__(16) float cb_s[kM * kCodes * kSub];
     const int tid = threadIdx.x;
     const int bh = blockIdx.y;
@@ -55,35 +62,91 @@ __global__ __launch_bounds__(kEncThreads, 3) void encode_bulk_kernel(EncodeArgs 
     int best = 0;
     float bestd = INFINITY;
     const float *cbase = a.coarse + (size_t)bh * a.L * kD;
-    for (int l0 = 0; l0 < a.L; l0 += kCoarseChunk) {
-        const int nl = min(kCoarseChunk, a.L - l0);
-        __syncthreads();
-        for (int i = tid; i < nl * kD / 4; i += kEncThreads)
-            reinterpret_cast<float4 *>(&cs[0][0])[i] = reinterpret_cast<const float4 *>(cbase + (size_t)l0 * kD)[i];
-        __syncthreads();
-        if (valid) {
+    // the fixed-order distance to one centroid row (LDS or memory), 16 elements at a time: the key
+    // row already takes 128 registers, and three waves per SIMD need the rest to stay small
+    auto measure = [&](const float *crow) {
+        float d2 = 0.0f;
+#pragma unroll
+        for (int d16 = 0; d16 < kD / 16; ++d16) {
+            float4 c[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) c[u] = reinterpret_cast<const float4 *>(crow)[4 * d16 + u];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int d = 16 * d16 + 4 * u;
+                float t;
+                t = x[d] - c[u].x; d2 = __builtin_fmaf(t, t, d2);
+                t = x[d + 1] - c[u].y; d2 = __builtin_fmaf(t, t, d2);
+                t = x[d + 2] - c[u].z; d2 = __builtin_fmaf(t, t, d2);
+                t = x[d + 3] - c[u].w; d2 = __builtin_fmaf(t, t, d2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return d2;
+    };
+    if constexpr (HINT) {
+        const uint32_t hint = valid ? a.hints[(size_t)bh * a.hint_stride + j] : 0u;
+        const bool all_lists = valid && (hint >> 31);
+        if (valid && !all_lists) {
+            const int c0 = hint & 0xfff, c1 = (hint >> 12) & 0xfff;
+            const int lo = min(c0, c1), hi = max(c0, c1);  // in index order: the first strict minimum wins
 #pragma unroll 1
-            for (int l = 0; l < nl; ++l) {
+            for (int t = 0; t < 2; ++t) {
+                const int l = t == 0 ? lo : hi;
+                if (l >= a.L || (t == 1 && hi == lo)) continue;
+                const float d2 = measure(cbase + (size_t)l * kD);
+                if (d2 < bestd) { bestd = d2; best = l; }
+            }
+        }
+        // A key that must be measured against every list (about one in a thousand) is taken by its
+        // whole wave: lane i measures lists i, i + 64, ..., with the key's direction read from its
+        // owner's registers, and the wave keeps the smallest distance, lowest list first.
+        const int lane = tid % kWave;
+        for (uint64_t pending = __ballot(all_lists); pending; pending &= pending - 1) {  // wave-uniform
+            const int owner = __ffsll((unsigned long long)pending) - 1;
+            float bd = INFINITY;
+            int bl = 0;
+#pragma unroll 1
+            for (int l = lane; l < a.L; l += kWave) {
+                const float *crow = cbase + (size_t)l * kD;
                 float d2 = 0.0f;
-                // the centroid passes through registers in pieces of 16 elements: the key row already
-                // takes 128 registers, and three waves per SIMD need the rest to stay small
 #pragma unroll
                 for (int d16 = 0; d16 < kD / 16; ++d16) {
                     float4 c[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) c[u] = reinterpret_cast<const float4 *>(&cs[l][0])[4 * d16 + u];
+                    for (int u = 0; u < 4; ++u) c[u] = reinterpret_cast<const float4 *>(crow)[4 * d16 + u];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         const int d = 16 * d16 + 4 * u;
                         float t;
-                        t = x[d] - c[u].x; d2 = __builtin_fmaf(t, t, d2);
-                        t = x[d + 1] - c[u].y; d2 = __builtin_fmaf(t, t, d2);
-                        t = x[d + 2] - c[u].z; d2 = __builtin_fmaf(t, t, d2);
-                        t = x[d + 3] - c[u].w; d2 = __builtin_fmaf(t, t, d2);
+                        t = lane_value(x[d], owner) - c[u].x; d2 = __builtin_fmaf(t, t, d2);
+                        t = lane_value(x[d + 1], owner) - c[u].y; d2 = __builtin_fmaf(t, t, d2);
+                        t = lane_value(x[d + 2], owner) - c[u].z; d2 = __builtin_fmaf(t, t, d2);
+                        t = lane_value(x[d + 3], owner) - c[u].w; d2 = __builtin_fmaf(t, t, d2);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (d2 < bestd) { bestd = d2; best = l0 + l; }
+                if (d2 < bd) { bd = d2; bl = l; }
+            }
+            // (distances are sums of squares: not negative, so they order as their bits; a lane that
+            // found nothing below +inf offers (+inf, list 0), which is what the serial search keeps)
+            const unsigned long long mine = ((unsigned long long)__float_as_uint(bd) << 32) | (uint32_t)bl;
+            const unsigned long long won = wave_min_u64(mine, kWave);
+            if (lane == owner) best = (int)(won & 0xffffffffull);
+        }
+        } else {
+        for (int l0 = 0; l0 < a.L; l0 += kCoarseChunk) {
+            const int nl = min(kCoarseChunk, a.L - l0);
+            __syncthreads();
+            for (int i = tid; i < nl * kD / 4; i += kEncThreads)
+                reinterpret_cast<float4 *>(&cs[0][0])[i] = reinterpret_cast<const float4 *>(cbase + (size_t)l0 * kD)[i];
+            __syncthreads();
+            if (valid) {
+#pragma unroll 1
+                for (int l = 0; l < nl; ++l) {
+                    const float d2 = measure(&cs[l][0]);
+                    if (d2 < bestd) { bestd = d2; best = l0 + l; }
+                }
             }
         }
     }
@@ -252,11 +315,18 @@ int fill_encode_args(EncodeArgs &a, const pqhsa_kv_view *kv, const pqhsa_index *
     return PQHSA_OK;
 }
 
+size_t prefilter_workspace_bytes(int BH, int L, int64_t count_max);
+int launch_prefilter(const EncodeArgs &e, int dtype, int BH, int count_max, void *workspace, size_t workspace_bytes,
+                     const uint32_t **hints, int64_t *hint_stride, hipStream_t stream);
+
 static int launch_encode(const EncodeArgs &a, int dtype, int BH, int count_max, hipStream_t stream) {
     if (BH == 0 || count_max <= 0) return PQHSA_OK;
-    if (count_max >= 64) {
+    if (a.hints) {
         dim3 grid((count_max + kEncThreads - 1) / kEncThreads, BH);
-        PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(encode_bulk_kernel<DT>, grid, dim3(kEncThreads), 0, stream, a));
+        PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((encode_bulk_kernel<DT, true>), grid, dim3(kEncThreads), 0, stream, a));
+    } else if (count_max >= 64) {
+        dim3 grid((count_max + kEncThreads - 1) / kEncThreads, BH);
+        PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((encode_bulk_kernel<DT, false>), grid, dim3(kEncThreads), 0, stream, a));
     } else {
         dim3 grid(count_max, BH);
         PQHSA_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(encode_row_kernel<DT>, grid, dim3(kEncThreads), 0, stream, a));
@@ -275,6 +345,25 @@ extern "C" int pqhsa_encode(const pqhsa_kv_view *kv, const pqhsa_index *index, i
     if (rc) return rc;
     PQHSA_REQUIRE(slot0 && count, "encode: NULL slot0/count");
     return launch_encode(a, kv->dtype, index->batch * index->kv_heads, count_max, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t pqhsa_encode_bulk_workspace_bytes(int32_t B, int32_t H, int32_t num_lists, int32_t count_max) {
+    return prefilter_workspace_bytes(B * H, num_lists, count_max);
+}
+
+extern "C" int pqhsa_encode_bulk(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink, const int32_t *slot0,
+                                 const int32_t *count, int32_t count_max, float eps, void *workspace,
+                                 size_t workspace_bytes, void *stream_v) {
+    EncodeArgs a = {};
+    int rc = fill_encode_args(a, kv, index, sink, slot0, count, eps);
+    if (rc) return rc;
+    PQHSA_REQUIRE(slot0 && count, "encode_bulk: NULL slot0/count");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const int BH = index->batch * index->kv_heads;
+    if (BH == 0 || count_max <= 0) return PQHSA_OK;
+    rc = launch_prefilter(a, kv->dtype, BH, count_max, workspace, workspace_bytes, &a.hints, &a.hint_stride, stream);
+    if (rc) return rc;
+    return launch_encode(a, kv->dtype, BH, count_max, stream);
 }
 
 extern "C" int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,

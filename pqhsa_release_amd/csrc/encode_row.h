@@ -24,6 +24,9 @@ struct EncodeArgs {
     int64_t n_cap;
     float *vsum, *vcount, *vbar;
     const int32_t *n_idx;
+    // bulk encode with list candidates (NULL: every list is measured)
+    const uint32_t *hints;  // [BH, hint_stride] bits 0-11, 12-23: lists to measure; bit 31: measure all
+    int64_t hint_stride;
 };
 
 __device__ inline unsigned long long wave_min_u64(unsigned long long v, int width) {

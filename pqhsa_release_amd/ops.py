@@ -318,12 +318,29 @@ def _i32(values, device) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- index maintenance
-def encode(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: float = EPS) -> None:
-    """Encode ``count[b]`` key rows per sequence starting at index slot ``slot0[b]``."""
+BULK_ENCODE_MIN_ROWS = 1024   # from here on the matrix-core candidate pass pays for its two extra launches
+BULK_ENCODE_MAX_LISTS = 4096
+
+
+def encode(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: float = EPS,
+           bulk: bool | None = None) -> None:
+    """Encode ``count[b]`` key rows per sequence starting at index slot ``slot0[b]``.
+
+    Many rows at once go through ``pqhsa_encode_bulk`` (same results bit for bit; ``bulk`` forces
+    or forbids that path), whose scratch memory is a temporary of this call."""
     lib = _lib.load()
     s0, c = _i32(slot0, index.device), _i32(count, index.device)
-    rc = lib.pqhsa_encode(kv.ref(), index.ref(), int(sink), s0.data_ptr(), c.data_ptr(), int(max(count)), eps,
-                          _stream())
+    cmax = int(max(count))
+    if bulk is None:
+        bulk = cmax >= BULK_ENCODE_MIN_ROWS
+    if bulk and cmax > 0 and index.num_lists <= BULK_ENCODE_MAX_LISTS:
+        need = lib.pqhsa_encode_bulk_workspace_bytes(index.batch, index.kv_heads, index.num_lists, cmax)
+        ws = torch.empty(need, dtype=torch.uint8, device=index.device)
+        rc = lib.pqhsa_encode_bulk(kv.ref(), index.ref(), int(sink), s0.data_ptr(), c.data_ptr(), cmax, eps,
+                                   ws.data_ptr(), need, _stream())
+        _lib.check(rc, "pqhsa_encode_bulk")
+        return
+    rc = lib.pqhsa_encode(kv.ref(), index.ref(), int(sink), s0.data_ptr(), c.data_ptr(), cmax, eps, _stream())
     _lib.check(rc, "pqhsa_encode")
 
 

@@ -49,6 +49,79 @@ def test_encode_bulk_and_row_kernels_match_oracle_bitwise(dtype, paged):
     assert np.array_equal(packed[:, 1] >> 4, (w >> 12) & 15) and np.array_equal(packed[:, 0] & 15, w & 15)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("paged", [None, "5d"])
+def test_encode_with_matrix_core_candidates_matches_oracle_bitwise(dtype, paged):
+    """pqhsa_encode_bulk: the nearest list comes from two candidates of a half-precision matrix
+    product, measured in the oracle's order; 48 lists leave half of the second tile as padding."""
+    dev = _cuda()
+    p = Problem(lens=[900, 517], heads=2, lists=48, dtype=dtype, seed=3)
+    idx = p.device_index(dev, upload_codes=False)
+    kv = ops.kv_paged(*p.paged_kv(paged)) if paged else ops.kv_contiguous(*p.dense_kv())
+    counts = [p.n(b) for b in range(p.B)]
+    ops.encode(kv, idx, p.sink, [0, 0], [c - 300 for c in counts], bulk=True)
+    ops.encode(kv, idx, p.sink, [c - 300 for c in counts], [300, 300], bulk=True)     # a second call, from an offset
+    torch.cuda.synchronize()
+    for (b, h), ix in p.index.items():
+        bh, n = b * p.H + h, p.n(b)
+        assert np.array_equal(u32(idx.codes[bh, :n]), ix["codes"]), (b, h)
+        assert np.array_equal(u16(idx.list_ids[bh, :n]), ix["list_ids"]), (b, h)
+        assert np.array_equal(idx.norms[bh, :n].cpu().numpy(), ix["norms"]), (b, h)
+        assert np.array_equal(idx.pos[bh, :n].cpu().numpy(), np.arange(n)), (b, h)
+
+
+@pytest.mark.parametrize("case", ["clustered", "twin_lists", "wide_tables", "beyond_half_precision", "one_list",
+                                  "odd_keys"])
+def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
+    """The candidate pass never changes a bit of the encode, also where its estimate cannot tell
+    lists apart: centroid rows that are equal or 1e-5 apart (every key near them measures all
+    lists), tables of large values (the error bound grows with them), values beyond fp16 (no bound:
+    all lists for every key), a single list, zero / huge / non-finite keys."""
+    dev = _cuda()
+    gen = torch.Generator().manual_seed(17)
+    B, H, L, n = 2, 2, (1 if case == "one_list" else 200), 6000
+    centres = torch.randn(B, H, L, 128, generator=gen)
+    pick = torch.randint(0, L, (B, H, n), generator=gen)
+    keys = torch.gather(centres, 2, pick.unsqueeze(-1).expand(-1, -1, -1, 128)) + 0.4 * torch.randn(B, H, n, 128, generator=gen)
+    coarse = centres / centres.norm(dim=-1, keepdim=True)
+    if case == "twin_lists":
+        coarse[:, :, 100:150] = coarse[:, :, 0:50]                      # equal rows: the lower id must win
+        coarse[:, :, 150:200] = coarse[:, :, 50:100] + 1e-5 * torch.randn(B, H, 50, 128, generator=gen)
+    if case == "wide_tables":
+        coarse = coarse * 37.0
+    if case == "beyond_half_precision":
+        coarse[:, :, 7, 3] = 5.0e4
+    if case == "odd_keys":
+        keys[:, :, 0] = 0.0
+        keys[:, :, 1] = 1.0e-30
+        keys[:, :, 2] = 1.0e30
+        keys[:, :, 3, 5] = float("inf")
+        keys[:, :, 4, 9] = float("nan")
+        keys[:, :, 5] = coarse[:, :, 11] * 3.0                            # exactly on a centroid's ray
+    keys = keys.to(dev)
+    kv = ops.kv_contiguous(keys, torch.zeros_like(keys))
+    got = []
+    for bulk in (False, True):
+        idx = ops.DeviceIndex(B, H, L, n + 64, dev)
+        idx.coarse.copy_(coarse.reshape(B * H, L, 128))
+        idx.codebooks.copy_(0.1 * torch.randn(B * H, 8, 16, 16, generator=torch.Generator().manual_seed(5)))
+        idx.set_counts([n, n - 777])
+        ops.encode(kv, idx, 0, [0, 0], [n, n - 777], bulk=bulk)
+        torch.cuda.synchronize()
+        got.append((u16(idx.list_ids), u32(idx.codes), idx.norms.cpu().numpy().view(np.uint32)))
+    for b, cnt in enumerate([n, n - 777]):
+        rows = slice(b * H, (b + 1) * H)
+        for name, x, y in zip(("list ids", "codes", "norms"), got[0], got[1]):
+            assert np.array_equal(x[rows, :cnt], y[rows, :cnt]), (case, b, name)
+    if case in ("clustered", "wide_tables"):   # ... and the lists are the nearest ones (float64 check of a sample)
+        lid = got[1][0][0, :512].astype(np.int64)
+        d = keys[0, 0, :512].double().cpu()
+        d = d / d.norm(dim=-1, keepdim=True)
+        dist = torch.cdist(d, coarse[0, 0].double())
+        best = dist.min(dim=1).values
+        assert torch.all(dist[torch.arange(512), torch.from_numpy(lid)] <= best + 1e-5)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_value_summaries_and_append_match_oracle(dtype):
     dev = _cuda()
