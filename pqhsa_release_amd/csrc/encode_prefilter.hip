@@ -11,14 +11,23 @@
 // as well.  The encode kernel then measures only the reported lists in the fixed order (or all of
 // them when the flag is set), so its results do not change by a bit.
 //
-// The bound, for a key direction x (|x| <= 1) and a centroid c with |c| <= cmax:
-//   operands rounded to fp16 (relative 2^-11 each, 2^-25 absolute below the normal range):
-//       |sum x~ c~ - sum x (-2c)| <= 2 |x| |c| (2^-10 + 2^-22) + tiny
-//   fp32 accumulation of 128 exact products and |c|^2:   <= 129 * 2^-24 * (|c|^2 + 2 |c|)
-//   the fixed-order chain itself (t = x - c, acc = fma(t, t, acc)):  <= 130 * 2^-24 * (1 + |c|)^2
+// The operands are scaled by powers of two (directions by 2^10, centroids by 2^4, so every estimate
+// by 2^14): whatever the matrix cores do with fp16 values below the normal range then concerns
+// components below 6e-8 of a direction and 4e-6 of a centroid only.  The bound, for a key direction
+// x (|x| <= 1) and a centroid c with |c| <= cmax, before that scaling:
+//   operands rounded to fp16 (relative 2^-11 each):
+//       |sum x~ c~ - sum x (-2c)| <= 2 |x| |c| (2^-10 + 2^-22)
+//   operand components below the normal range, should they count as zero:
+//       <= 2^-24 * 2 sqrt(128) |c|  +  2^-18 * sqrt(128) |x|
+//   fp32 accumulation of 128 exact products onto |c|^2, rounded or truncated:
+//       <= 300 * 2^-24 * (|c|^2 + 2 |c|)
+//   the direction itself (a reciprocal and a sum in another order than the encode kernel's):
+//       <= 1e-6 * (|c|^2 + 4 |c|)
+//   the fixed-order chain of the encode kernel (t = x - c, acc = fma(t, t, acc)):
+//       <= 130 * 2^-24 * (1 + |c|)^2
 //   the list id stored in the low bits of the estimate: 2^-(23 - bits) * (|c|^2 + 2 |c|)
-// tau() below adds these up, twice (two estimates are compared), with a margin.  A stream whose
-// table holds values that fp16 cannot carry, or no finite bound, has every key flagged.
+// tau() below adds these up, twice (two estimates are compared), with a margin of a quarter.  A
+// stream whose table holds values that fp16 cannot carry, or no finite bound, has every key flagged.
 #include "common.h"
 #include "encode_row.h"
 
@@ -32,6 +41,8 @@ constexpr int kPreChunk = 32;                      // centroids per matrix tile
 constexpr int kPreKeys = 2 * kPreChunk * (kPreThreads / kWave);  // keys per workgroup: two tiles of 32 per wave
 constexpr int kPreSteps = kD / 16;                 // 16 dims per matrix instruction
 constexpr float kPreFar = 3.0e38f;                 // estimate of a padding row: never among the smallest
+constexpr float kKeyScale = 1024.0f, kRowScale = 16.0f;  // powers of two: exact
+constexpr float kEstScale = kKeyScale * kRowScale;
 
 struct PrefilterArgs {
     KvView kv;
@@ -42,8 +53,8 @@ struct PrefilterArgs {
     const int32_t *count;     // [B]
     const float *coarse;      // [BH, L, 128]
     float eps;
-    half8 *table;             // [BH, chunks, 8 steps, 64 lanes] -2 c in fp16, in the order the lanes load it
-    float *cnorm;             // [BH, chunks * 32] |c|^2 (padding rows: kPreFar)
+    half8 *table;             // [BH, chunks, 8 steps, 64 lanes] -2 c * 2^4 in fp16, in the order the lanes load it
+    float *cnorm;             // [BH, chunks * 32] |c|^2 * 2^14 (padding rows: kPreFar)
     uint32_t *cmax_bits;      // [BH] largest |c| of the stream as float bits (cleared before the table kernel)
     uint32_t *hints;          // [BH, hint_stride]
     int64_t hint_stride;
@@ -64,7 +75,7 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_table_kernel(PrefilterA
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float c = row < a.L ? cbase[(size_t)row * kD + 16 * s + 8 * (lane / kPreChunk) + e] : 0.0f;
-            v[e] = (_Float16)(-2.0f * c);
+            v[e] = (_Float16)(-2.0f * kRowScale * c);
         }
         out[cell] = v;
     }
@@ -76,10 +87,10 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_table_kernel(PrefilterA
                 const float c = cbase[(size_t)row * kD + d];
                 ss = __builtin_fmaf(c, c, ss);
                 // a value fp16 cannot carry (or no number at all) leaves no bound for the stream
-                if (!(fabsf(2.0f * c) <= 60000.0f)) big = INFINITY;
+                if (!(fabsf(2.0f * kRowScale * c) <= 60000.0f)) big = INFINITY;
             }
         }
-        a.cnorm[(size_t)bh * a.chunks * kPreChunk + row] = row < a.L ? ss : kPreFar;
+        a.cnorm[(size_t)bh * a.chunks * kPreChunk + row] = row < a.L ? ss * kEstScale : kPreFar;
         float m = big > 0.0f ? big : sqrtf(ss);
         if (!(m == m)) m = INFINITY;
         cmax_s[tid] = m;
@@ -92,14 +103,15 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_table_kernel(PrefilterA
     }
 }
 
+// how far apart two estimates (as the kernel holds them: scaled by 2^14) of equal fixed-order distances can lie
 __device__ inline float tau(float cmax, int id_bits) {
-    if (!(cmax <= 1.0e4f)) return INFINITY;
+    if (!(cmax <= 1.0e3f)) return INFINITY;
     const float reach = cmax * cmax + 2.0f * cmax;  // largest |estimate|
-    const float operands = cmax * 2.0f * (0x1p-10f + 0x1p-22f) + 64.0f * 0x1p-25f * (1.0f + 2.0f * cmax);
-    const float sums = 129.0f * 0x1p-24f * reach + 1.0e-6f * (2.0f * cmax + reach);  // accumulation, |c|^2, the norm
+    const float operands = cmax * 2.0f * (0x1p-10f + 0x1p-22f) + 0x1p-24f * 23.0f * cmax + 0x1p-18f * 12.0f;
+    const float sums = 300.0f * 0x1p-24f * reach + 1.0e-6f * (reach + 2.0f * cmax);
     const float chain = 130.0f * 0x1p-24f * (1.0f + cmax) * (1.0f + cmax);
     const float packed = ldexpf(reach, id_bits - 23);
-    return 1.25f * 2.0f * (operands + sums + chain + packed);
+    return kEstScale * 1.25f * 2.0f * (operands + sums + chain + packed);
 }
 
 // the three smallest of what a lane has seen (v0 <= v1 <= v2)
@@ -154,11 +166,11 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(Prefi
         ss += __shfl_xor(ss, kPreChunk);
         float nrm = sqrtf(ss);
         if (nrm < a.eps) nrm = a.eps;
-        const float inv = 1.0f / nrm;
+        const float inv = kKeyScale / nrm;
 #pragma unroll
         for (int s = 0; s < kPreSteps; ++s)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) key[nb][s][e] = (_Float16)(f[s][e] * inv);
+            for (int e = 0; e < 8; ++e) key[nb][s][e] = (_Float16)(f[s][e] * inv);  // inv carries the 2^10
     }
     tile_s[tid] = stage[0];
     tile_s[tid + kPreThreads] = stage[1];

@@ -244,27 +244,45 @@ class DeviceIndex:
 
     def finalize_layout(self, seed: int = 0) -> None:
         """Order every stream's stored keys by list id (stable, so keys of a list keep their
-        insertion order) and draw the sampled subset.  Host-side torch ops, off the decode path."""
+        insertion order) and draw the sampled subset: one key from each of ``sample_size(n)``
+        equal strata of the list-ordered keys, the place inside a stratum from an integer hash of
+        (seed, sequence, stratum).  Torch ops on the device, off the decode path; nothing waits
+        for the host.  Sequences of one length that follow each other are ordered in one go."""
         h = self.kv_heads
-        gen = torch.Generator(device="cpu")
-        gen.manual_seed(int(seed))
-        for b, n in enumerate(self.n_host):
-            rows = slice(b * h, (b + 1) * h)
+        b = 0
+        while b < self.batch:
+            n = self.n_host[b]
+            e = b + 1
+            while e < self.batch and self.n_host[e] == n:
+                e += 1
             if n > 0:
-                lids = (self.list_ids[rows, :n].to(torch.int64) & 0xFFFF)
+                rows = slice(b * h, e * h)
+                lids = self.list_ids[rows, :n].to(torch.int32) & 0xFFFF
                 order = torch.argsort(lids, dim=1, stable=True)
                 for t in (self.codes, self.list_ids, self.norms, self.pos):
                     t[rows, :n] = torch.gather(t[rows, :n], 1, order)
                 ns = self.sample_size(n)
-                pick = torch.randperm(n, generator=gen)[:ns].sort().values.to(self.device)
-                self.s_codes[rows, :ns] = self.codes[rows][:, pick]
-                self.s_list_ids[rows, :ns] = self.list_ids[rows][:, pick]
-                self.s_norms[rows, :ns] = self.norms[rows][:, pick]
-            else:
-                ns = 0
-            self.n_sorted_host[b] = n
+                seqs = torch.arange(b, e, device=self.device, dtype=torch.int64).repeat_interleave(h).unsqueeze(1)
+                pick = self._sample_positions(n, ns, int(seed), seqs)                 # [(e - b) * h, ns]
+                self.s_codes[rows, :ns] = torch.gather(self.codes[rows, :n], 1, pick)
+                self.s_list_ids[rows, :ns] = torch.gather(self.list_ids[rows, :n], 1, pick)
+                self.s_norms[rows, :ns] = torch.gather(self.norms[rows, :n], 1, pick)
+            for i in range(b, e):
+                self.n_sorted_host[i] = n
+            b = e
         self.n_sorted.copy_(torch.tensor(self.n_sorted_host, dtype=torch.int32))
         self.s_n.copy_(torch.tensor([self.sample_size(n) if n > 0 else 0 for n in self.n_host], dtype=torch.int32))
+
+    def _sample_positions(self, n: int, ns: int, seed: int, seqs: torch.Tensor) -> torch.Tensor:
+        """Ascending positions in ``[0, n)``, one per stratum ``[i n / ns, (i + 1) n / ns)``; the
+        heads of a sequence share them (``seqs``: the sequence number of every row, ``[rows, 1]``)."""
+        i = torch.arange(ns, device=self.device, dtype=torch.int64).unsqueeze(0)
+        lo, hi = i * n // ns, (i + 1) * n // ns
+        x = (i + 1) * 0x9E3779B1 + (seqs + 1) * 0x85EBCA77 + (seed + 1) * 0xC2B2AE3D
+        x = (x ^ (x >> 15)) * 0x2C1B3C6D & 0xFFFFFFFF
+        x = (x ^ (x >> 12)) * 0x297A2D39 & 0xFFFFFFFF
+        x = x ^ (x >> 15)
+        return lo + x % (hi - lo)
 
     def tail_max(self) -> int:
         return max((n - s for n, s in zip(self.n_host, self.n_sorted_host)), default=0)
@@ -318,7 +336,7 @@ def _i32(values, device) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- index maintenance
-BULK_ENCODE_MIN_ROWS = 1024   # from here on the matrix-core candidate pass pays for its two extra launches
+BULK_ENCODE_MIN_ROWS = 128    # from here on the matrix-core candidate pass pays for its two extra launches
 BULK_ENCODE_MAX_LISTS = 4096
 
 

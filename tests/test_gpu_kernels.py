@@ -71,11 +71,12 @@ def test_encode_with_matrix_core_candidates_matches_oracle_bitwise(dtype, paged)
 
 
 @pytest.mark.parametrize("case", ["clustered", "twin_lists", "wide_tables", "beyond_half_precision", "one_list",
-                                  "odd_keys"])
+                                  "odd_keys", "between_two_lists", "between_three_lists"])
 def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
     """The candidate pass never changes a bit of the encode, also where its estimate cannot tell
     lists apart: centroid rows that are equal or 1e-5 apart (every key near them measures all
-    lists), tables of large values (the error bound grows with them), values beyond fp16 (no bound:
+    lists), keys half way between two or three centroids (distances equal to within 1e-4, far
+    inside the estimate's error), tables of large values (the error bound grows with them), values beyond fp16 (no bound:
     all lists for every key), a single list, zero / huge / non-finite keys."""
     dev = _cuda()
     gen = torch.Generator().manual_seed(17)
@@ -91,6 +92,11 @@ def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
         coarse = coarse * 37.0
     if case == "beyond_half_precision":
         coarse[:, :, 7, 3] = 5.0e4
+    if case in ("between_two_lists", "between_three_lists"):
+        k = 2 if case == "between_two_lists" else 3
+        near = torch.stack([torch.gather(coarse, 2, torch.randint(0, L, (B, H, n), generator=gen).unsqueeze(-1)
+                                         .expand(-1, -1, -1, 128)) for _ in range(k)]).sum(0)
+        keys = 5.0 * near + 1e-4 * torch.randn(B, H, n, 128, generator=gen)
     if case == "odd_keys":
         keys[:, :, 0] = 0.0
         keys[:, :, 1] = 1.0e-30
