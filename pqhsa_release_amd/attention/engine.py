@@ -310,35 +310,38 @@ class PQHSAEngine:
         from the HIP encode kernel; the small per-list means are torch ops on the device."""
         ic, idx = self.index_config, self.index
         lr = ic.online_codebook_lr
-        H, L = self.H, idx.num_lists
-        head = torch.arange(H, device=self.device).unsqueeze(1)
-
-        def new_dirs(b: int) -> torch.Tensor:  # [H, added, 128] directions of sequence b's new keys
-            rows = self._retrieval_block(b, added[b], start=old[b]).float()
-            return rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
+        H, L, M = self.H, idx.num_lists, ops.SUBSPACES
+        dev = self.device
+        # sequences that gained the same number of keys move their tables in one go (all KV heads
+        # and subspaces at once); nothing below waits for the host
+        groups: dict[int, list[int]] = {}
+        for b in range(self.B):
+            if added[b] > 0:
+                groups.setdefault(added[b], []).append(b)
+        batches = []
+        for cnt, seqs in groups.items():
+            rows = torch.cat([self._retrieval_block(b, cnt, start=old[b]).float() for b in seqs])      # [S, cnt, 128]
+            dirs = rows / torch.linalg.vector_norm(rows, dim=-1, keepdim=True).clamp_min(ic.eps)
+            streams = (torch.tensor(seqs, device=dev).unsqueeze(1) * H + torch.arange(H, device=dev)).reshape(-1, 1)
+            first = torch.tensor([old[b] for b in seqs], device=dev).repeat_interleave(H).unsqueeze(1)
+            where = streams * idx.n_cap + first + torch.arange(cnt, device=dev)                           # [S, cnt] flat slots
+            batches.append((dirs, streams, where))
 
         ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # lists of the new rows
-        for b in range(self.B):  # all KV heads of a sequence move their tables in one go
-            if added[b] <= 0:
-                continue
-            sl = slice(old[b], old[b] + added[b])
-            lids = idx.list_ids[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFF
-            _ema_rows(idx.coarse[b * H : (b + 1) * H].view(H * L, D), new_dirs(b).reshape(-1, D),
-                      (lids + head * L).reshape(-1), lr, ic.eps)
+        for dirs, streams, where in batches:
+            lids = idx.list_ids.view(-1)[where].to(torch.int64) & 0xFFFF
+            _ema_rows(idx.coarse.view(-1, D), dirs.reshape(-1, D), (lids + streams * L).reshape(-1), lr, ic.eps)
         ops.encode(self.kv, idx, self.sink, old, added, eps=ic.eps)          # re-assign with moved lists
-        for b in range(self.B):
-            if added[b] <= 0:
-                continue
-            sl = slice(old[b], old[b] + added[b])
-            lids = idx.list_ids[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFF
-            coarse = idx.coarse[b * H : (b + 1) * H]
-            resid = new_dirs(b) - torch.gather(coarse, 1, lids.unsqueeze(-1).expand(-1, -1, D))
-            words = idx.codes[b * H : (b + 1) * H, sl].to(torch.int64) & 0xFFFFFFFF
-            shifts = 4 * torch.arange(ops.SUBSPACES, device=self.device)
-            code = (words.unsqueeze(-1) >> shifts) & 15                           # [H, added, 8]
-            book = (head.unsqueeze(-1) * ops.SUBSPACES + torch.arange(ops.SUBSPACES, device=self.device)) * 16
-            _ema_rows(idx.codebooks[b * H : (b + 1) * H].view(H * ops.SUBSPACES * 16, ops.SUBDIM),
-                      resid.reshape(-1, ops.SUBDIM), (code + book).reshape(-1), lr, ic.eps)
+        shifts = 4 * torch.arange(M, device=dev)
+        for dirs, streams, where in batches:
+            lids = idx.list_ids.view(-1)[where].to(torch.int64) & 0xFFFF
+            centre = idx.coarse.view(-1, D)[(lids + streams * L).reshape(-1)].view_as(dirs)
+            resid = dirs - centre
+            words = idx.codes.view(-1)[where].to(torch.int64) & 0xFFFFFFFF
+            code = (words.unsqueeze(-1) >> shifts) & 15                                                   # [S, cnt, 8]
+            book = (streams.unsqueeze(-1) * M + torch.arange(M, device=dev)) * 16                         # [S, 1, 8]
+            _ema_rows(idx.codebooks.view(-1, ops.SUBDIM), resid.reshape(-1, ops.SUBDIM), (code + book).reshape(-1),
+                      lr, ic.eps)
         new = [o + a for o, a in zip(old, added)]
         idx.reset_layout()
         idx.set_counts(new)
@@ -451,7 +454,7 @@ def _ema_rows(table: torch.Tensor, vectors: torch.Tensor, assign: torch.Tensor, 
     """table[j] <- (1 - lr) * table[j] + lr * mean(vectors assigned to j), for non-empty j."""
     sums = torch.zeros_like(table)
     sums.index_add_(0, assign, vectors.to(table.dtype))
-    counts = torch.bincount(assign, minlength=table.shape[0]).to(table.dtype)
-    filled = counts > 0
-    means = sums[filled] / counts[filled].unsqueeze(1).clamp_min(eps)
-    table[filled] = (1.0 - lr) * table[filled] + lr * means
+    counts = torch.bincount(assign, minlength=table.shape[0]).to(table.dtype).unsqueeze(1)
+    means = sums / counts.clamp_min(eps)
+    # (rows nothing was assigned to keep their bits; no mask is read back by the host)
+    table.copy_(torch.where(counts > 0, (1.0 - lr) * table + lr * means, table))
