@@ -207,13 +207,13 @@ __global__ __launch_bounds__(kD) void value_append_kernel(EncodeArgs a) {
 }
 
 // Rebuild per-list value sums / counts / means in three launches: clear, accumulate, divide.
-// Accumulate: 16 lanes own one value row (8 channels each); every 16-lane group walks 16
+// Accumulate: 16 lanes own one value row (8 channels each); every 16-lane group walks 128
 // consecutive stored keys and hands a run of equal list ids to the list's sum with one atomic
 // add per channel, so on a list-ordered layout most keys cost no atomic at all (an unordered
 // layout pays one set per key).  The sums are exact up to the order of fp32 additions.
 constexpr int kSumThreads = 256;
 constexpr int kSumGroups = kSumThreads / 16;
-constexpr int kSumRun = 16;
+constexpr int kSumRun = 128;  // stored keys one 16-lane group walks
 
 template <int DT>
 __global__ __launch_bounds__(kSumThreads) void value_sums_kernel(EncodeArgs a) {
@@ -224,14 +224,6 @@ __global__ __launch_bounds__(kSumThreads) void value_sums_kernel(EncodeArgs a) {
     const int first = (blockIdx.x * kSumGroups + grp) * kSumRun;
     if (first >= n) return;
     const size_t esz = DT == PQHSA_F32 ? 4 : 2;
-    // lane r of the group fetches list id and token of the group's r-th key
-    int my_list = -1, my_tok = 0;
-    if (first + lane16 < n) {
-        const size_t o = (size_t)bh * a.n_cap + first + lane16;
-        my_list = a.list_ids[o];
-        my_tok = a.pos ? a.pos[o] : first + lane16;  // retrieval-local index of the stored key
-        if (my_list >= a.L) my_list = -1;
-    }
     float *vsum = a.vsum + (size_t)bh * a.L * kD;
     float *vcount = a.vcount + (size_t)bh * a.L;
     float acc[8];
@@ -243,31 +235,41 @@ __global__ __launch_bounds__(kSumThreads) void value_sums_kernel(EncodeArgs a) {
         for (int e = 0; e < 8; ++e) unsafeAtomicAdd(&vsum[(size_t)cur * kD + lane16 * 8 + e], acc[e]);
         if (lane16 == 0) unsafeAtomicAdd(&vcount[cur], run);
     };
-    for (int r0 = 0; r0 < kSumRun; r0 += 4) {
-        int l[4];
-        float f[4][8];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {  // four rows on their way at once
-            l[u] = __shfl(my_list, r0 + u, 16);
-            const int tok = __shfl(my_tok, r0 + u, 16);
-            if (l[u] >= 0) {
-                const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + tok) * esz;
-                load8<DT>(row, lane16, f[u]);
-            }
+    for (int sub = 0; sub < kSumRun && first + sub < n; sub += 16) {
+        // lane r of the group fetches list id and token of the r-th key of this piece of the run
+        int my_list = -1, my_tok = 0;
+        if (first + sub + lane16 < n) {
+            const size_t o = (size_t)bh * a.n_cap + first + sub + lane16;
+            my_list = a.list_ids[o];
+            my_tok = a.pos ? a.pos[o] : first + sub + lane16;  // retrieval-local index of the stored key
+            if (my_list >= a.L) my_list = -1;
         }
+        for (int r0 = 0; r0 < 16; r0 += 4) {
+            int l[4];
+            float f[4][8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if (l[u] < 0) continue;  // past the end of the stream (uniform in the group)
-            if (l[u] != cur) {
-                flush();
-                cur = l[u];
-                run = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+            for (int u = 0; u < 4; ++u) {  // four rows on their way at once
+                l[u] = __shfl(my_list, r0 + u, 16);
+                const int tok = __shfl(my_tok, r0 + u, 16);
+                if (l[u] >= 0) {
+                    const char *row = a.kv.v_base + row_offset(a.kv, b, h, (int64_t)a.sink + tok) * esz;
+                    load8<DT>(row, lane16, f[u]);
+                }
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] += f[u][e];
-            run += 1.0f;
+            for (int u = 0; u < 4; ++u) {
+                if (l[u] < 0) continue;  // past the end of the stream, or no list (uniform in the group)
+                if (l[u] != cur) {
+                    flush();
+                    cur = l[u];
+                    run = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] += f[u][e];
+                run += 1.0f;
+            }
         }
     }
     flush();
