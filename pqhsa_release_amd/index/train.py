@@ -14,6 +14,8 @@ trains on: the same seed then starts the same trajectory here and there, and the
 
 from __future__ import annotations
 
+import functools
+
 import torch
 
 
@@ -101,17 +103,18 @@ def train_ivfpq(keys: torch.Tensor, *, num_lists: int, num_subspaces: int = 8, n
 
 
 class _LazyGenerators:
-    """One generator per stream, all seeded alike, created only for a stream that needs a draw of
-    its own (an empty cluster) and first advanced past the draws every stream shares."""
+    """One generator per problem, seeded as that problem's own call would seed it, created only
+    for a problem that needs a draw of its own (an empty cluster) and first advanced past the
+    draw of the start."""
 
-    def __init__(self, streams: int, seed: int, n: int, shared_perm: bool) -> None:
-        self.gens = [None] * streams
-        self.seed, self.n, self.shared_perm = int(seed), n, shared_perm
+    def __init__(self, seeds: list[int], n: int, shared_perm: bool) -> None:
+        self.gens = [None] * len(seeds)
+        self.seeds, self.n, self.shared_perm = seeds, n, shared_perm
 
     def get(self, s: int) -> torch.Generator:
         if self.gens[s] is None:
             g = torch.Generator(device="cpu")
-            g.manual_seed(self.seed)
+            g.manual_seed(self.seeds[s])
             if self.shared_perm:
                 torch.randperm(self.n, generator=g)
             self.gens[s] = g
@@ -131,27 +134,38 @@ def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int
     return out
 
 
-def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed: int = 0, eps: float = 1e-12):
+@functools.lru_cache(maxsize=64)
+def _seeded_start(n: int, num_clusters: int, seed: int) -> torch.Tensor:
+    """The first ``num_clusters`` entries of the seeded permutation of ``n`` (CPU generator, as the
+    reference draws it).  Kept per (n, clusters, seed): every stream, sequence and layer of one
+    length starts from the same draw, and a permutation of 131 072 takes the CPU about a millisecond."""
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(seed)
+    return torch.randperm(n, generator=gen)[:num_clusters].clone()
+
+
+def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed=0, eps: float = 1e-12):
     """``kmeans_l2`` for ``S`` independent problems of one size, ``vectors [S, N, D]``: the seeded
-    start (one permutation, the same for every problem, as S separate calls with one seed would
-    draw) and the Lloyd iterations run as batched products; a problem whose assignment stops
-    changing keeps its centroids, as the early exit of the per-stream loop does."""
+    start (``seed``: one number for all problems, as S separate calls with one seed would draw,
+    or one per problem) and the Lloyd iterations run as batched products; a problem whose
+    assignment stops changing keeps its centroids, as the early exit of the per-stream loop does."""
     if vectors.ndim != 3:
         raise ValueError(f"vectors must be [S, N, D], got {tuple(vectors.shape)}")
     s, n, dim = vectors.shape
     if n == 0:
         raise ValueError("cannot train k-means with zero vectors")
     dev = vectors.device
-    gen = torch.Generator(device="cpu")
-    gen.manual_seed(int(seed))
-    lazy = _LazyGenerators(s, seed, n, shared_perm=n >= num_clusters)
+    seeds = [int(x) for x in seed] if isinstance(seed, (list, tuple)) else [int(seed)] * s
+    if len(seeds) != s:
+        raise ValueError(f"{len(seeds)} seeds for {s} problems")
+    lazy = _LazyGenerators(seeds, n, shared_perm=n >= num_clusters)
     if n >= num_clusters:
-        centroids = vectors[:, torch.randperm(n, generator=gen)[:num_clusters].to(dev)].clone()
+        start = torch.stack([_seeded_start(n, num_clusters, x) for x in seeds]).to(dev)               # [S, K]
+        centroids = torch.gather(vectors, 1, start.unsqueeze(-1).expand(-1, -1, dim)).clone()
     else:
-        extra = torch.randint(0, n, (num_clusters - n,), generator=gen).to(dev)
-        centroids = torch.cat([vectors, vectors[:, extra]], dim=1).clone()
-        for i in range(s):  # every stream's own generator has made this draw too
-            torch.randint(0, n, (num_clusters - n,), generator=lazy.get(i))
+        # (every problem's own generator makes this draw: a later reseeding continues from it)
+        extra = torch.stack([torch.randint(0, n, (num_clusters - n,), generator=lazy.get(i)) for i in range(s)]).to(dev)
+        centroids = torch.cat([vectors, torch.gather(vectors, 1, extra.unsqueeze(-1).expand(-1, -1, dim))], dim=1).clone()
     assign = torch.zeros(s, n, dtype=torch.long, device=dev)
     live = torch.ones(s, dtype=torch.bool, device=dev)
     offsets = (torch.arange(s, device=dev) * num_clusters).unsqueeze(1)
@@ -163,11 +177,21 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
         live = live & ~same
         if not bool(live.any()):
             break
-        sums = torch.zeros(s * num_clusters, dim, dtype=torch.float32, device=dev)
-        sums.index_add_(0, (assign + offsets).reshape(-1), flat)
-        counts = torch.bincount((assign + offsets).reshape(-1), minlength=s * num_clusters).float()
-        filled = counts > 0
-        sums[filled] /= counts[filled].unsqueeze(1).clamp_min(eps)
+        if num_clusters <= 64:
+            # Few clusters (the 16 codewords of a subspace): row adds from a million keys would
+            # queue up on 16 rows per problem.  The product with the 0/1 membership matrix adds
+            # the same terms without that, and its column sums are the counts.
+            member = (assign.unsqueeze(-1) == torch.arange(num_clusters, device=dev)).float()      # [S, N, K]
+            sums = torch.bmm(member.transpose(1, 2), flat.view(s, n, dim)).reshape(s * num_clusters, dim)
+            counts = member.sum(dim=1).reshape(-1)
+        else:
+            where = (assign + offsets).reshape(-1)
+            sums = torch.zeros(s * num_clusters, dim, dtype=torch.float32, device=dev)
+            sums.index_add_(0, where, flat)
+            counts = torch.zeros(s * num_clusters, dtype=torch.float32, device=dev)
+            counts.index_add_(0, where, torch.ones(1, dtype=torch.float32, device=dev).expand(where.numel()))
+        filled = counts > 0   # (float counts are exact below 2^24 keys per problem)
+        sums = torch.where(filled.unsqueeze(1), sums / counts.unsqueeze(1).clamp_min(eps), sums)
         sums = sums.reshape(s, num_clusters, dim)
         empty = (~filled).reshape(s, num_clusters)
         if bool(empty.any()):
@@ -196,9 +220,9 @@ def train_ivfpq_batched(keys: torch.Tensor, *, num_lists: int, num_subspaces: in
     resid = dirs - torch.gather(coarse, 1, assign.unsqueeze(-1).expand(-1, -1, dirs.shape[2]))
     sub = keys.shape[2] // num_subspaces
     chunks = resid.reshape(resid.shape[0], resid.shape[1], num_subspaces, sub)
-    books = []
-    for m in range(num_subspaces):
-        c, _ = kmeans_l2_batched(chunks[:, :, m].contiguous(), num_codes, max_iter=pq_iter,
-                                 seed=seed + 10_000 + m, eps=eps)
-        books.append(c)
-    return coarse.float().contiguous(), torch.stack(books, dim=1).float().contiguous()
+    # the subspaces of all streams are one batch of problems, each with its own seed
+    streams = resid.shape[0]
+    problems = chunks.permute(0, 2, 1, 3).reshape(streams * num_subspaces, resid.shape[1], sub)
+    books, _ = kmeans_l2_batched(problems, num_codes, max_iter=pq_iter,
+                                 seed=[seed + 10_000 + m for _ in range(streams) for m in range(num_subspaces)], eps=eps)
+    return coarse.float().contiguous(), books.reshape(streams, num_subspaces, num_codes, sub).float().contiguous()
