@@ -85,6 +85,11 @@ def make_stream(ctx, groups, seed, device, dtype):
 class Layer:
     """One layer's resident state: K/V (paged or dense), trained + encoded index, queries."""
 
+    @staticmethod
+    def _now(device):
+        torch.cuda.synchronize(device)
+        return time.perf_counter()
+
     def __init__(self, cfg_id, seed0, device, room=0):
         """``room`` > 0 prepares the layer for that many append + decode steps: the cache holds
         ``room`` more tokens per sequence (already written, as a serving engine writes a token's K/V
@@ -120,6 +125,7 @@ class Layer:
             self.values = torch.zeros_like(self.keys)
             self.kv = ops.kv_contiguous(self.keys, self.values)
         q = torch.empty(B, H * G, 128, dtype=dtype, device=device)
+        train_s, seq_keys = 0.0, []
         for b, ln0 in enumerate(self.lens):
             ln = ln0 + room
             pos = torch.arange(ln, device=device)
@@ -136,18 +142,37 @@ class Layer:
                 q[b, h * G : (h + 1) * G] = qq
                 head_keys.append(k[SINK : SINK + self.n[b]])
                 del k, v
-            # the sequence's KV heads have one length: their indexes train together
-            coarse, books = train_ivfpq_batched(torch.stack(head_keys), num_lists=LISTS, coarse_iter=1, pq_iter=2,
-                                                seed=0)
-            self.index.coarse[b * H : (b + 1) * H, : coarse.shape[1]] = coarse
-            self.index.codebooks[b * H : (b + 1) * H] = books
+            seq_keys.append(torch.stack(head_keys))
             del head_keys
+        # sequences of one length train together, all their KV heads at once (about 2 GB of fp32 keys per call)
+        by_n = {}
+        for b, nb in enumerate(self.n):
+            by_n.setdefault(nb, []).append(b)
+        for nb, seqs in by_n.items():
+            step = max(1, ((1 << 31) // (nb * 128 * 4)) // H)
+            for i in range(0, len(seqs), step):
+                part = seqs[i : i + step]
+                t0 = self._now(device)
+                coarse, books = train_ivfpq_batched(torch.cat([seq_keys[b] for b in part]), num_lists=LISTS,
+                                                    coarse_iter=1, pq_iter=2, seed=0)
+                train_s += self._now(device) - t0
+                for j, b in enumerate(part):
+                    self.index.coarse[b * H : (b + 1) * H, : coarse.shape[1]] = coarse[j * H : (j + 1) * H]
+                    self.index.codebooks[b * H : (b + 1) * H] = books[j * H : (j + 1) * H]
+        del seq_keys
         self.q = q
         self.out = torch.empty_like(q)
         self.index.set_counts(self.n)
+        t0 = self._now(device)
         ops.encode(self.kv, self.index, SINK, [0] * B, self.n)
+        t1 = self._now(device)
         self.index.finalize_layout()
+        t2 = self._now(device)
         ops.value_summaries(self.kv, self.index, SINK)
+        t3 = self._now(device)
+        # wall-clock of the index build's parts for this layer (the device drained around each)
+        self.build_ms = {"train": round(train_s * 1e3, 2), "encode": round((t1 - t0) * 1e3, 2),
+                         "layout": round((t2 - t1) * 1e3, 2), "value_summaries": round((t3 - t2) * 1e3, 2)}
         self.seq_lens = torch.tensor(self.lens, dtype=torch.int32, device=device)
         k_cap = ops.resolve_topk(n_max + room, FRACTION, 0)
         self.ws = ops.DecodeWorkspace(self.index, G, k_cap)
@@ -614,6 +639,7 @@ def main():
                       "candidates_mean": round(float(layer.ws.candidate_counts().float().mean()), 1),
                       "candidates_max": int(layer.ws.candidate_counts().max())},
         "decode_workspace_MB": round(layer.ws.bytes / 1e6, 2),
+        "index_build_ms": run.layers[-1].build_ms,   # of the layer built last (kernels and allocator warm)
     }
     if args.standalone:
         result["standalone"] = standalone_kernels(layer)
