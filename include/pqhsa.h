@@ -152,6 +152,16 @@ int pqhsa_encode_bulk(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t
                       void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The assignment step of index training after its matrix product: for problem p and vector j,
+ * out[p * out_stride + j] = the first k that minimises sq[p, k] - 2 * dots[p, j, k] (a NaN counts
+ * as smallest, as in torch.argmin).  dots [problems, rows, K] and sq [problems, K] contiguous and
+ * 16-byte aligned.  One pass over the products in place of the multiply, subtract and arg-min of
+ * _nearest_centroids_chunked (pq_hsa/index/kmeans.py:108-131), with the same arithmetic.
+ */
+int pqhsa_nearest_from_products(const float *dots, const float *sq, int32_t problems, int64_t rows,
+                                int32_t K, int64_t *out, int64_t out_stride, void *stream);
+
+/*
  * Rebuild vsum / vcount / vbar from the values of all indexed keys
  * (SparseKVCache._build_retrieval_value_summaries, pq_hsa/attention/kv_cache.py:688-728).
  * n_max >= max_b n_idx[b] sizes the launch (<= 0: n_cap).  Three launches: clear, accumulate

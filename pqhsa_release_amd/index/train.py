@@ -130,7 +130,12 @@ def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int
     out = torch.empty(s, n, dtype=torch.long, device=vectors.device)
     for i in range(0, n, chunk):
         v = vectors[:, i : i + chunk].float()
-        out[:, i : i + chunk] = (half_sq - 2.0 * torch.bmm(v, cf.transpose(1, 2))).argmin(dim=2)
+        dots = torch.bmm(v, cf.transpose(1, 2))
+        if dots.is_cuda:  # one pass over the products (same arithmetic, ties to the lowest index)
+            from .. import ops
+            ops.nearest_from_products(dots, half_sq.reshape(s, -1), out[:, i : i + chunk])
+        else:
+            out[:, i : i + chunk] = (half_sq - 2.0 * dots).argmin(dim=2)
     return out
 
 

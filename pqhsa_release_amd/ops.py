@@ -362,6 +362,20 @@ def encode(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: fl
     _lib.check(rc, "pqhsa_encode")
 
 
+def nearest_from_products(dots: torch.Tensor, sq: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[p, j]`` = first argmin over k of ``sq[p, k] - 2 * dots[p, j, k]``; ``dots [P, R, K]``
+    and ``sq [P, K]`` contiguous fp32, ``out`` int64 ``[P, R]`` with unit stride along R (a column
+    slice of a wider tensor is fine)."""
+    _need_cuda(dots, sq, out)
+    p, r, k = dots.shape
+    if (dots.dtype != torch.float32 or sq.dtype != torch.float32 or out.dtype != torch.int64 or not dots.is_contiguous()
+            or not sq.is_contiguous() or tuple(sq.shape) != (p, k) or tuple(out.shape) != (p, r) or (r > 1 and out.stride(1) != 1)):
+        raise ValueError("nearest_from_products: dots [P, R, K] / sq [P, K] contiguous fp32, out [P, R] int64")
+    rc = _lib.load().pqhsa_nearest_from_products(dots.data_ptr(), sq.data_ptr(), p, r, k, out.data_ptr(),
+                                                 out.stride(0) if p > 1 else r, _stream())
+    _lib.check(rc, "pqhsa_nearest_from_products")
+
+
 def value_summaries(kv: KvSource, index: DeviceIndex, sink: int) -> None:
     lib = _lib.load()
     rc = lib.pqhsa_value_summaries(kv.ref(), index.ref(), int(sink), int(index.n_max), _stream())

@@ -128,6 +128,33 @@ def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
         assert torch.all(dist[torch.arange(512), torch.from_numpy(lid)] <= best + 1e-5)
 
 
+@pytest.mark.parametrize("k", [1, 3, 16, 17, 32, 36, 512, 600, 1024, 2000])
+def test_nearest_from_products_is_the_elementwise_argmin(k):
+    """pqhsa_nearest_from_products against the three torch ops it stands for, bit for bit: equal
+    values (lowest index wins), +inf rows, NaNs (the first NaN wins, as in torch.argmin), and an
+    output that is a column slice of a wider tensor."""
+    dev = _cuda()
+    gen = torch.Generator().manual_seed(k)
+    p, r = 3, 1501
+    dots = torch.randn(p, r, k, generator=gen)
+    sq = torch.rand(p, k, generator=gen) * 2.0
+    if k >= 3:
+        dots[:, 5] = dots[:, 5, :1]                                 # whole rows of equal products ...
+        sq[0] = sq[0, 0]                                            # ... and of equal norms: all values equal
+        dots[1, 7, k // 2] = float("-inf")                          # value +inf in the middle
+        dots[1, 8] = float("-inf")                                  # a row of +inf only
+        dots[2, 9, k - 1] = float("nan")
+        dots[2, 10, 1] = float("nan"); dots[2, 10, k - 1] = float("nan")
+        dots[:, 11, k - 1] = dots[:, 11].max(dim=1).values + 1.0    # the minimum in the last place
+    dots, sq = dots.to(dev), sq.to(dev)
+    want = (sq.unsqueeze(1) - 2.0 * dots).argmin(dim=2)
+    wide = torch.full((p, r + 9), -1, dtype=torch.int64, device=dev)
+    ops.nearest_from_products(dots, sq, wide[:, 4 : 4 + r])
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:, 4 : 4 + r], want)
+    assert int((wide[:, :4] != -1).sum()) == 0 and int((wide[:, 4 + r :] != -1).sum()) == 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_value_summaries_and_append_match_oracle(dtype):
     dev = _cuda()
