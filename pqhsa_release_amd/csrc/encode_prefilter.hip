@@ -38,7 +38,8 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int kPreThreads = 256;
 constexpr int kPreChunk = 32;                      // centroids per matrix tile
-constexpr int kPreKeys = 2 * kPreChunk * (kPreThreads / kWave);  // keys per workgroup: two tiles of 32 per wave
+constexpr int kPreTiles = 1;                       // tiles of 32 keys per wave
+constexpr int kPreKeys = kPreTiles * kPreChunk * (kPreThreads / kWave);  // keys per workgroup
 constexpr int kPreSteps = kD / 16;                 // 16 dims per matrix instruction
 constexpr float kPreFar = 3.0e38f;                 // estimate of a padding row: never among the smallest
 constexpr float kKeyScale = 1024.0f, kRowScale = 16.0f;  // powers of two: exact
@@ -121,7 +122,9 @@ __device__ inline void keep3(float x, float &v0, float &v1, float &v2) {
     v0 = fminf(v0, x);
 }
 
-// ---- candidates: two tiles of 32 keys per wave against all tiles of 32 lists ---------------------
+// ---- candidates: a tile of 32 keys per wave against all tiles of 32 lists -------------------------
+// (one tile per wave keeps the kernel at four waves per SIMD; two tiles, with the centroid operand
+// read once for both, ran at two waves per SIMD and 7 % slower)
 template <int DT>
 __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(PrefilterArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -142,11 +145,11 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(Prefi
     stage[1] = table[tid + kPreThreads];
     for (int i = tid; i < a.chunks * kPreChunk; i += kPreThreads) cn_s[i] = a.cnorm[(size_t)bh * a.chunks * kPreChunk + i];
 
-    // this lane's half of its two keys, as directions in fp16
-    half8 key[2][kPreSteps];
+    // this lane's half of its key (of each tile), as a direction in fp16
+    half8 key[kPreTiles][kPreSteps];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-        const int j = j0 + wave * 2 * kPreChunk + nb * kPreChunk + col;
+    for (int nb = 0; nb < kPreTiles; ++nb) {
+        const int j = j0 + wave * kPreTiles * kPreChunk + nb * kPreChunk + col;
         float f[kPreSteps][8];
         float ss = 0.0f;
         if (j < cnt) {
@@ -177,9 +180,9 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(Prefi
     __syncthreads();
 
     const uint32_t id_mask = (1u << a.id_bits) - 1u;
-    float v0[2], v1[2], v2[2];
+    float v0[kPreTiles], v1[kPreTiles], v2[kPreTiles];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) v0[nb] = v1[nb] = v2[nb] = INFINITY;
+    for (int nb = 0; nb < kPreTiles; ++nb) v0[nb] = v1[nb] = v2[nb] = INFINITY;
     for (int c = 0; c < a.chunks; ++c) {
         const half8 *cur = tile_s + (c & 1) * kPreSteps * kWave;
         if (c + 1 < a.chunks) {  // the next tile travels while this one is used
@@ -188,22 +191,24 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(Prefi
         }
         // Accumulator register r of a lane belongs to row 8 (r / 4) + 4 (lane / 32) + r % 4 of the
         // tile and to column lane % 32: it starts from that row's |c|^2.
-        float16v acc[2];
+        float16v acc[kPreTiles];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 n4 = *reinterpret_cast<const float4 *>(cn_s + c * kPreChunk + 8 * q + 4 * half);
             acc[0][4 * q] = n4.x; acc[0][4 * q + 1] = n4.y; acc[0][4 * q + 2] = n4.z; acc[0][4 * q + 3] = n4.w;
         }
-        acc[1] = acc[0];
+#pragma unroll
+        for (int nb = 1; nb < kPreTiles; ++nb) acc[nb] = acc[0];
 #pragma unroll
         for (int s = 0; s < kPreSteps; ++s) {
             const half8 rows = cur[s * kWave + lane];
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(rows, key[0][s], acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(rows, key[1][s], acc[1], 0, 0, 0);
+#pragma unroll
+            for (int nb = 0; nb < kPreTiles; ++nb)
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(rows, key[nb][s], acc[nb], 0, 0, 0);
         }
         const uint32_t id0 = (uint32_t)(c * kPreChunk + 4 * half);
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
+        for (int nb = 0; nb < kPreTiles; ++nb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t id = id0 + (uint32_t)(8 * (r / 4) + r % 4);
@@ -220,14 +225,14 @@ __global__ __launch_bounds__(kPreThreads) void prefilter_candidates_kernel(Prefi
 
     const float reach = tau(__uint_as_float(a.cmax_bits[bh]), a.id_bits);
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < kPreTiles; ++nb) {
         // the other half of the wave has seen the other rows of every tile for the same key
         const float o0 = __shfl_xor(v0[nb], kPreChunk), o1 = __shfl_xor(v1[nb], kPreChunk), o2 = __shfl_xor(v2[nb], kPreChunk);
         keep3(o0, v0[nb], v1[nb], v2[nb]);
         keep3(o1, v0[nb], v1[nb], v2[nb]);
         keep3(o2, v0[nb], v1[nb], v2[nb]);
-        const int j = j0 + wave * 2 * kPreChunk + nb * kPreChunk + col;
-        if (half == nb && j < cnt) {
+        const int j = j0 + wave * kPreTiles * kPreChunk + nb * kPreChunk + col;
+        if (half == nb % 2 && j < cnt) {
             const bool clear = v2[nb] - v0[nb] > reach;  // false for anything that is not a number
             const uint32_t c0 = __float_as_uint(v0[nb]) & id_mask, c1 = __float_as_uint(v1[nb]) & id_mask;
             a.hints[(size_t)bh * a.hint_stride + j] = c0 | (c1 << 12) | (clear ? 0u : 0x80000000u);
