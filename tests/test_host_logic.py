@@ -434,3 +434,48 @@ def test_device_index_regroup_copies_rows_and_counts():
         assert torch.equal(new.s_codes[rows_new, :keep], src.s_codes[rows_old, :keep])
     with pytest.raises(ValueError):
         ops.DeviceIndex.regroup([(a, 0), (ops.DeviceIndex(1, 4, 8, 16, "cpu"), 0)], n_cap=16)
+
+
+def test_sampled_subset_positions_are_one_per_stratum():
+    """DeviceIndex._sample_positions: ascending, distinct, inside [0, n), one per stratum of the
+    list-ordered keys; the heads of a sequence share them, sequences and seeds do not."""
+    from pqhsa_release_amd.ops import DeviceIndex
+
+    holder = types.SimpleNamespace(device=torch.device("cpu"))
+    seqs = torch.tensor([[0], [0], [1]])
+    for n, ns in ((131004, 8192), (5000, 1024), (1000, 1000), (4097, 4096)):
+        pos = DeviceIndex._sample_positions(holder, n, ns, 0, seqs)
+        assert pos.shape == (3, ns) and int(pos.min()) >= 0 and int(pos.max()) < n
+        assert bool((pos[:, 1:] > pos[:, :-1]).all())
+        i = torch.arange(ns)
+        assert bool((pos >= i * n // ns).all()) and bool((pos < (i + 1) * n // ns).all())
+        assert torch.equal(pos[0], pos[1])
+        if n >= 2 * ns:   # strata of one key leave no choice
+            assert not torch.equal(pos[0], pos[2])
+            assert not torch.equal(pos[0], DeviceIndex._sample_positions(holder, n, ns, 1, seqs)[0])
+    # the places inside the strata are spread: no half of a stratum is favoured
+    pos = DeviceIndex._sample_positions(holder, 1 << 20, 8192, 3, seqs[:1])[0]
+    inside = (pos - torch.arange(8192) * 128).float() / 128.0
+    assert 0.45 < float(inside.mean()) < 0.55 and float(inside.std()) > 0.25
+
+
+def test_ema_rows_moves_the_rows_that_got_vectors_and_no_others():
+    """_ema_rows (the table move of the deferred flush): row j becomes (1 - lr) row + lr * mean of
+    the vectors assigned to j; rows without vectors keep their bits (pq.py:117-173)."""
+    from pqhsa_release_amd.attention.engine import _ema_rows
+
+    gen = torch.Generator().manual_seed(9)
+    table = torch.randn(40, 16, generator=gen)
+    vectors = torch.randn(300, 16, generator=gen)
+    assign = torch.randint(0, 40, (300,), generator=gen)
+    assign[assign == 7] = 8                       # row 7 gets nothing
+    before = table.clone()
+    _ema_rows(table, vectors, assign, 0.25, 1e-12)
+    for j in range(40):
+        mine = vectors[assign == j]
+        if mine.shape[0] == 0:
+            assert torch.equal(table[j], before[j])
+        else:
+            want = 0.75 * before[j] + 0.25 * (mine.sum(0) / mine.shape[0])
+            torch.testing.assert_close(table[j], want, rtol=0, atol=1e-6)
+    assert torch.equal(table[7], before[7])
