@@ -71,7 +71,7 @@ def test_encode_with_matrix_core_candidates_matches_oracle_bitwise(dtype, paged)
 
 
 @pytest.mark.parametrize("case", ["clustered", "twin_lists", "wide_tables", "beyond_half_precision", "one_list",
-                                  "odd_keys", "between_two_lists", "between_three_lists"])
+                                  "odd_keys", "between_two_lists", "between_three_lists", "many_lists"])
 def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
     """The candidate pass never changes a bit of the encode, also where its estimate cannot tell
     lists apart: centroid rows that are equal or 1e-5 apart (every key near them measures all
@@ -80,7 +80,7 @@ def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
     all lists for every key), a single list, zero / huge / non-finite keys."""
     dev = _cuda()
     gen = torch.Generator().manual_seed(17)
-    B, H, L, n = 2, 2, (1 if case == "one_list" else 200), 6000
+    B, H, L, n = 2, 2, {"one_list": 1, "many_lists": 4096}.get(case, 200), 6000   # 4096: all 12 bits of a hint's list ids
     centres = torch.randn(B, H, L, 128, generator=gen)
     pick = torch.randint(0, L, (B, H, n), generator=gen)
     keys = torch.gather(centres, 2, pick.unsqueeze(-1).expand(-1, -1, -1, 128)) + 0.4 * torch.randn(B, H, n, 128, generator=gen)
