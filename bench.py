@@ -310,6 +310,56 @@ def host_cores():
     return min(os.cpu_count() or 1, 16)
 
 
+def index_maintenance(device, batch=4, kv_heads=8, groups=4, ctx=131072, appended=256):
+    """Wall-clock of the index work around the decode step, through the adapter a serving engine
+    drives (the device drained around each part): the build after prefill (training + encode +
+    layout + summaries of all streams), ``appended`` one-token appends with the deferred strategy,
+    and the flush that follows them (table moves, re-encode of every key, layout, summaries)."""
+    from pqhsa_release_amd.attention import GQAIVFPQDecodeAttentionAdapter
+    from pqhsa_release_amd.config import IVFPQConfig, SparseAttentionConfig
+
+    ic = IVFPQConfig(num_lists=LISTS, nprobe=8, num_subspaces=8, num_bits=4, residual=True, coarse_max_iter=1,
+                     pq_max_iter=2, kernel_backend="mi355x", direction_normalize=True, seed=0)
+    ac = SparseAttentionConfig(sink_tokens=SINK, local_window=LOCAL, retrieval_top_fraction=FRACTION,
+                               exact_rerank=True, mode="hybrid", hybrid_value_mode="centroid",
+                               index_update_interval=appended, index_update_strategy="deferred",
+                               collect_attention_details=False)
+    gen = torch.Generator(device=device).manual_seed(1)
+    centres = torch.randn(LISTS, 128, device=device, generator=gen)
+
+    def rows(n):
+        pick = torch.randint(0, LISTS, (batch, kv_heads, n), device=device, generator=gen)
+        k = (centres[pick] + 0.3 * torch.randn(batch, kv_heads, n, 128, device=device, generator=gen)).to(torch.bfloat16)
+        return k, torch.randn(batch, kv_heads, n, 128, device=device, generator=gen).to(torch.bfloat16)
+
+    def clock():
+        torch.cuda.synchronize(device)
+        return time.perf_counter()
+
+    keys, values = rows(ctx)
+    adapter = GQAIVFPQDecodeAttentionAdapter(ic, ac, num_query_heads=kv_heads * groups, num_key_value_heads=kv_heads)
+    adapter.build_cache(keys, values)                     # first call: allocations, kernel loading
+    q = torch.randn(batch, kv_heads * groups, 128, device=device, generator=gen)
+    out = {"shape": f"batch {batch} x {kv_heads} KV heads x {ctx} tokens, bf16", "appended_keys_per_flush": appended}
+    for rep in range(2):                                  # the second round is the one reported
+        nk, nv = rows(appended)
+        t0 = clock()
+        for s in range(appended):
+            adapter.append(nk[:, :, s], nv[:, :, s])
+        t1 = clock()
+        adapter.forward(q)
+        t2 = clock()
+        flushed = adapter.apply_pending_index_update()
+        t3 = clock()
+        out.update(append_us_per_key=round((t1 - t0) / appended * 1e6, 1), flush_ms=round((t3 - t2) * 1e3, 2),
+                   flushed=bool(flushed))
+    t0 = clock()
+    adapter.build_cache(keys, values)
+    out["build_ms"] = round((clock() - t0) * 1e3, 2)
+    out["flush_us_per_step"] = round(out["flush_ms"] * 1e3 / appended, 1)
+    return out
+
+
 def cpu_baseline(layer, seconds=12.0):
     """Time the torch-CPU restatement of the reference path on one (sequence, KV head) stream of
     the same inputs and trained index, and scale to the whole layer."""
@@ -577,6 +627,9 @@ def main():
                     help="after the main configuration, run short passes over the other configurations and "
                          "report them under \"configs\" (default: only when --config is the headline one)")
     ap.add_argument("--other-steps", type=int, default=60)
+    ap.add_argument("--index-maintenance", action=argparse.BooleanOptionalAction, default=None,
+                    help="also time the index build and the deferred flush at the cfg 2 shape through the adapter "
+                         "(default: with the default configuration)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (every sequence and KV head of the layer is on it); "
@@ -674,6 +727,14 @@ def main():
             log(f"cfg{cfg}: {rec['us_per_layer']} us/layer, step roofline {rec['step_roofline_frac']}")
             side.close()
             del side
+    maintain = args.index_maintenance if args.index_maintenance is not None else (args.config == 2 and others)
+    if maintain:
+        if not others:
+            del layer
+            run.close()
+        torch.cuda.empty_cache()
+        result["index_maintenance"] = index_maintenance(device)
+        log(f"index maintenance: {result['index_maintenance']}")
     print(json.dumps(result), flush=True)
 
 
