@@ -39,6 +39,7 @@ struct AttendArgs {
     int chunk_cap;            // rows a workgroup's address list in LDS holds: full_max + k_cap are hard bounds
     float scale;
     int splits;
+    int group_xcd;            // launch form, see the kernel
     float *partials;          // [BH*G, splits, kPartWidth]
     uint32_t *arrive;         // [rows, 64] arrival flag of every split of a query row, then [rows] tickets; zero at launch
     size_t rows;              // BH*G
@@ -113,7 +114,7 @@ __device__ inline float peek(const float *p) {
 }
 
 template <int QDT>
-__device__ inline void fold_row_if_last(const AttendArgs &a, size_t orow, int b, int h, int g, int bh) {
+__device__ inline void fold_row_if_last(const AttendArgs &a, size_t orow, int b, int h, int g, int bh, int split) {
     __shared__ int last_s;
     __shared__ float head_s[2];                 // row maximum, sum of the background list masses
     __shared__ float acc_s[kFoldLanes][kD];
@@ -123,7 +124,7 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, size_t orow, int b,
     __syncthreads();
     if (tid < kWave) {  // (at most 64 splits: one flag per lane)
         uint32_t *flags = a.arrive + orow * kMaxSplits;
-        if (tid == 0) __hip_atomic_store(flags + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(flags + split, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __builtin_amdgcn_s_waitcnt(0);  // ... and the flag is visible before the row's flags are read
         const uint32_t set = tid < a.splits ? __hip_atomic_load(flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
         const bool all_set = __ballot(set == 0u) == 0ull;
@@ -195,7 +196,20 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     __shared__ __align__(16) float bg_s[kAttThreads / (kD / 4)][kD];
     __shared__ float ms_s[kAttThreads / (kD / 4)];
     const int tid = threadIdx.x;
-    const int split = blockIdx.x, g = blockIdx.y, bh = blockIdx.z;
+    // grid (splits, G, BH) -- or, group_xcd: one row of workgroups in which the G workgroups that
+    // take the same chunk number of the G query rows of a stream follow each other 8 apart, i.e.
+    // land on one XCD at about the same time (workgroups go round the 8 XCDs by linear index): the
+    // rows of a group select partly the same keys, in about the same order
+    int split, g, bh;
+    if (a.group_xcd) {
+        const int id = blockIdx.x, blk = id / (8 * a.G), in = id % (8 * a.G);
+        const int pair = blk * 8 + in % 8;   // (stream, chunk number)
+        g = in / 8;
+        split = pair % a.splits;
+        bh = pair / a.splits;
+    } else {
+        split = blockIdx.x; g = blockIdx.y; bh = blockIdx.z;
+    }
     const int b = bh / a.H, h = bh % a.H;
     const size_t orow = (size_t)bh * a.G + g;
     // The selected indices of this chunk are requested before the row's counts are known, from
@@ -341,7 +355,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
     if (cnt <= 0) {
         if (tid == 0) { publish(part, -INFINITY); publish(part + 1, 0.0f); }
         if (tid < kD) publish(part + 4 + tid, 0.0f);
-        fold_row_if_last<QDT>(a, orow, b, h, g, bh);
+        fold_row_if_last<QDT>(a, orow, b, h, g, bh, split);
         return;
     }
 
@@ -415,7 +429,7 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         publish(part + 1, l);
     }
     PQHSA_TRACE_MARK(trace_attend, trace_wg, 1);
-    fold_row_if_last<QDT>(a, orow, b, h, g, bh);
+    fold_row_if_last<QDT>(a, orow, b, h, g, bh, split);
     PQHSA_TRACE_MARK(trace_attend, trace_wg, 2);
 }
 
@@ -495,7 +509,8 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
                   kMaxSplits);
     a.chunk_cap = chunk;
     const size_t lds = (size_t)chunk * sizeof(int64_t) + 16;
-    dim3 grid(a.splits, a.G, BH);
+    a.group_xcd = even_rows && (BH * a.splits) % 8 == 0;
+    dim3 grid = a.group_xcd ? dim3(a.splits * a.G * BH) : dim3(a.splits, a.G, BH);
 #define PQHSA_ATT(KD, QD)                                                                              \
     {                                                                                                  \
         auto kern = attend_partial_kernel<KD, QD>;                                                     \
