@@ -27,7 +27,8 @@
 //       <= 130 * 2^-24 * (1 + |c|)^2
 //   the list id stored in the low bits of the estimate: 2^-(23 - bits) * (|c|^2 + 2 |c|)
 // tau() below adds these up, twice (two estimates are compared), with a margin of a quarter.  A
-// stream whose table holds values that fp16 cannot carry, or no finite bound, has every key flagged.
+// centroid row with values that fp16 cannot carry takes no part (it cannot be the nearest); a stream
+// without a finite bound has every key flagged.
 #include "common.h"
 #include "encode_row.h"
 
@@ -56,7 +57,7 @@ struct PrefilterArgs {
     float eps;
     half8 *table;             // [BH, chunks, 8 steps, 64 lanes] -2 c * 2^4 in fp16, in the order the lanes load it
     float *cnorm;             // [BH, chunks * 32] |c|^2 * 2^14 (padding rows: kPreFar)
-    uint32_t *cmax_bits;      // [BH] largest |c| of the stream as float bits (cleared before the table kernel)
+    uint32_t *cmax_bits;      // [BH] largest |c| among the stream's rows that take part, as float bits (0: none; cleared before the table kernel)
     uint32_t *hints;          // [BH, hint_stride]
     int64_t hint_stride;
 };
@@ -64,49 +65,53 @@ struct PrefilterArgs {
 // ---- the centroid table in matrix-operand order -------------------------------------------------
 // Lane l of a wave supplies row l % 32 of the tile and the 8 dims 16 s + 8 (l / 32) .. + 7 of step s.
 __global__ __launch_bounds__(kPreThreads) void prefilter_table_kernel(PrefilterArgs a) {
-    __shared__ float cmax_s[kPreChunk];
+    __shared__ float norm_s[kPreChunk];  // |c| of the tile's rows; negative: the row takes no part
     const int tid = threadIdx.x;
     const int chunk = blockIdx.x, bh = blockIdx.y;
     const float *cbase = a.coarse + (size_t)bh * a.L * kD;
+    // A row with a value fp16 cannot carry (or no number at all) is left out of the estimates: one
+    // of its elements is beyond 1 875, so its fixed-order distance to a direction is above 3.5e6
+    // (or not a number, which never wins), while every row that takes part lies within
+    // (1 + 1 000)^2 of it -- tau() gives up on a stream whose other rows are longer than 1 000.
+    // Padding centroids of sequences with fewer keys than lists are such rows.
+    if (tid < kPreChunk) {
+        const int row = chunk * kPreChunk + tid;
+        float ss = 0.0f;
+        bool plain = row < a.L;
+        if (plain) {
+            for (int d = 0; d < kD; ++d) {
+                const float c = cbase[(size_t)row * kD + d];
+                ss = __builtin_fmaf(c, c, ss);
+                if (!(fabsf(2.0f * kRowScale * c) <= 60000.0f)) plain = false;
+            }
+        }
+        a.cnorm[(size_t)bh * a.chunks * kPreChunk + row] = plain ? ss * kEstScale : kPreFar;
+        norm_s[tid] = plain ? fmaxf(sqrtf(ss), 1.0e-30f) : -1.0f;
+    }
+    __syncthreads();
     half8 *out = a.table + ((size_t)bh * a.chunks + chunk) * kPreSteps * kWave;
     for (int cell = tid; cell < kPreSteps * kWave; cell += kPreThreads) {
         const int s = cell / kWave, lane = cell % kWave;
         const int row = chunk * kPreChunk + lane % kPreChunk;
+        const bool plain = norm_s[lane % kPreChunk] > 0.0f;
         half8 v;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float c = row < a.L ? cbase[(size_t)row * kD + 16 * s + 8 * (lane / kPreChunk) + e] : 0.0f;
+            const float c = plain ? cbase[(size_t)row * kD + 16 * s + 8 * (lane / kPreChunk) + e] : 0.0f;
             v[e] = (_Float16)(-2.0f * kRowScale * c);
         }
         out[cell] = v;
     }
-    if (tid < kPreChunk) {
-        const int row = chunk * kPreChunk + tid;
-        float ss = 0.0f, big = 0.0f;
-        if (row < a.L) {
-            for (int d = 0; d < kD; ++d) {
-                const float c = cbase[(size_t)row * kD + d];
-                ss = __builtin_fmaf(c, c, ss);
-                // a value fp16 cannot carry (or no number at all) leaves no bound for the stream
-                if (!(fabsf(2.0f * kRowScale * c) <= 60000.0f)) big = INFINITY;
-            }
-        }
-        a.cnorm[(size_t)bh * a.chunks * kPreChunk + row] = row < a.L ? ss * kEstScale : kPreFar;
-        float m = big > 0.0f ? big : sqrtf(ss);
-        if (!(m == m)) m = INFINITY;
-        cmax_s[tid] = m;
-    }
-    __syncthreads();
     if (tid == 0) {
-        float m = 0.0f;
-        for (int r = 0; r < kPreChunk; ++r) m = fmaxf(m, cmax_s[r]);
+        float m = 0.0f;  // stays 0 for a tile without a row that takes part
+        for (int r = 0; r < kPreChunk; ++r) m = fmaxf(m, norm_s[r]);
         atomicMax(a.cmax_bits + bh, __float_as_uint(m));  // non-negative floats order as their bits
     }
 }
 
 // how far apart two estimates (as the kernel holds them: scaled by 2^14) of equal fixed-order distances can lie
 __device__ inline float tau(float cmax, int id_bits) {
-    if (!(cmax <= 1.0e3f)) return INFINITY;
+    if (!(cmax > 0.0f && cmax <= 1.0e3f)) return INFINITY;  // no row takes part, or rows too long for the bound
     const float reach = cmax * cmax + 2.0f * cmax;  // largest |estimate|
     const float operands = cmax * 2.0f * (0x1p-10f + 0x1p-22f) + 0x1p-24f * 23.0f * cmax + 0x1p-18f * 12.0f;
     const float sums = 300.0f * 0x1p-24f * reach + 1.0e-6f * (reach + 2.0f * cmax);

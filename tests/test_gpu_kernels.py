@@ -71,13 +71,16 @@ def test_encode_with_matrix_core_candidates_matches_oracle_bitwise(dtype, paged)
 
 
 @pytest.mark.parametrize("case", ["clustered", "twin_lists", "wide_tables", "beyond_half_precision", "one_list",
-                                  "odd_keys", "between_two_lists", "between_three_lists", "many_lists"])
+                                  "odd_keys", "between_two_lists", "between_three_lists", "many_lists",
+                                  "padded_lists"])
 def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
     """The candidate pass never changes a bit of the encode, also where its estimate cannot tell
     lists apart: centroid rows that are equal or 1e-5 apart (every key near them measures all
     lists), keys half way between two or three centroids (distances equal to within 1e-4, far
-    inside the estimate's error), tables of large values (the error bound grows with them), values beyond fp16 (no bound:
-    all lists for every key), a single list, zero / huge / non-finite keys."""
+    inside the estimate's error), tables of large values (the error bound grows with them), a
+    centroid row with a value beyond fp16 and the padding rows of a sequence with fewer keys than
+    lists (such rows take no part in the estimate: they cannot be the nearest), a single list,
+    zero / huge / non-finite keys."""
     dev = _cuda()
     gen = torch.Generator().manual_seed(17)
     B, H, L, n = 2, 2, {"one_list": 1, "many_lists": 4096}.get(case, 200), 6000   # 4096: all 12 bits of a hint's list ids
@@ -92,6 +95,9 @@ def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
         coarse = coarse * 37.0
     if case == "beyond_half_precision":
         coarse[:, :, 7, 3] = 5.0e4
+    if case == "padded_lists":    # a sequence with fewer keys than lists: the unused rows hold the padding centroid
+        coarse[:, :, 150:] = ops.DeviceIndex.PAD_CENTROID
+        coarse[1, :, 3:] = ops.DeviceIndex.PAD_CENTROID
     if case in ("between_two_lists", "between_three_lists"):
         k = 2 if case == "between_two_lists" else 3
         near = torch.stack([torch.gather(coarse, 2, torch.randint(0, L, (B, H, n), generator=gen).unsqueeze(-1)
