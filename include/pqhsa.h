@@ -152,6 +152,23 @@ int pqhsa_encode_bulk(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t
                       void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The assignment step of the coarse k-means in index training, without the matrix of products: for
+ * problem p and row j, out[p * out_stride + j] = the centroid of centroids[p] nearest to the
+ * DIRECTION of vectors[p, j] (the row divided by max(its norm, eps); training hands over unit
+ * directions, for which this is the nearest centroid), ties to the lowest index.  Candidates come
+ * from the half-precision matrix product of pqhsa_encode_bulk, the decision from fixed-order fp32
+ * distances.  vectors [problems, rows, 128] and centroids [problems, num_centroids, 128] fp32,
+ * contiguous, 16-byte aligned; num_centroids <= 4096; workspace 256-byte aligned, of
+ * pqhsa_nearest_rows_workspace_bytes(...) bytes, used during the call only.
+ * Replaces _nearest_centroids_chunked (pq_hsa/index/kmeans.py:108-131) for 128-dimensional
+ * directions; nearly equal distances may fall the other way than in its |c|^2 - 2<v,c> form.
+ */
+size_t pqhsa_nearest_rows_workspace_bytes(int32_t problems, int32_t num_centroids, int32_t rows);
+int pqhsa_nearest_rows(const float *vectors, const float *centroids, int32_t problems, int32_t rows,
+                       int32_t num_centroids, float eps, int64_t *out, int64_t out_stride,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * The assignment step of index training after its matrix product: for problem p and vector j,
  * out[p * out_stride + j] = the first k that minimises sq[p, k] - 2 * dots[p, j, k] (a NaN counts
  * as smallest, as in torch.argmin).  dots [problems, rows, K] and sq [problems, K] contiguous and

@@ -31,7 +31,8 @@ __global__ __launch_bounds__(kEncThreads, HINT ? 2 : 3) void encode_bulk_kernel(
     const int slot = a.slot0[b] + j;
     const size_t esz = DT == PQHSA_F32 ? 4 : 2;
 
-    for (int i = tid; i < kM * kCodes * kSub; i += kEncThreads) cb_s[i] = a.codebooks[(size_t)bh * kM * kCodes * kSub + i];
+    if (!(HINT && a.assign_out))
+        for (int i = tid; i < kM * kCodes * kSub; i += kEncThreads) cb_s[i] = a.codebooks[(size_t)bh * kM * kCodes * kSub + i];
 
     float x[kD];
     float nrm = 1.0f;
@@ -151,6 +152,12 @@ __global__ __launch_bounds__(kEncThreads, HINT ? 2 : 3) void encode_bulk_kernel(
         }
     }
     if (!valid) return;
+    if constexpr (HINT) {
+        if (a.assign_out) {  // the assignment step of index training: the nearest list is all that is asked for
+            a.assign_out[(size_t)bh * a.assign_stride + j] = best;
+            return;
+        }
+    }
 
     const float *cbest = cbase + (size_t)best * kD;
 #pragma unroll
@@ -366,6 +373,50 @@ extern "C" int pqhsa_encode_bulk(const pqhsa_kv_view *kv, const pqhsa_index *ind
     rc = launch_prefilter(a, kv->dtype, BH, count_max, workspace, workspace_bytes, &a.hints, &a.hint_stride, stream);
     if (rc) return rc;
     return launch_encode(a, kv->dtype, BH, count_max, stream);
+}
+
+// slot0 = 0 and count = rows for every problem of pqhsa_nearest_rows
+__global__ void nearest_rows_counts_kernel(int32_t *slot0, int32_t *count, int problems, int rows) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < problems) { slot0[i] = 0; count[i] = rows; }
+}
+
+extern "C" size_t pqhsa_nearest_rows_workspace_bytes(int32_t problems, int32_t num_centroids, int32_t rows) {
+    return prefilter_workspace_bytes(problems, num_centroids, rows) + 2 * (((size_t)problems * sizeof(int32_t) + 255) & ~(size_t)255);
+}
+
+extern "C" int pqhsa_nearest_rows(const float *vectors, const float *centroids, int32_t problems, int32_t rows,
+                                  int32_t num_centroids, float eps, int64_t *out, int64_t out_stride, void *workspace,
+                                  size_t workspace_bytes, void *stream_v) {
+    PQHSA_REQUIRE(vectors && centroids && out && workspace, "nearest_rows: NULL argument");
+    PQHSA_REQUIRE(problems >= 0 && rows >= 0 && num_centroids >= 1 && num_centroids <= 4096,
+                  "nearest_rows: problems=%d rows=%d centroids=%d", problems, rows, num_centroids);
+    PQHSA_REQUIRE(((uintptr_t)vectors & 15) == 0 && ((uintptr_t)centroids & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
+                  "nearest_rows: vectors / centroids not 16-byte aligned or workspace not 256-byte aligned");
+    PQHSA_REQUIRE(workspace_bytes >= pqhsa_nearest_rows_workspace_bytes(problems, num_centroids, rows),
+                  "nearest_rows: workspace of %zu bytes, %zu needed", workspace_bytes,
+                  pqhsa_nearest_rows_workspace_bytes(problems, num_centroids, rows));
+    if (problems == 0 || rows == 0) return PQHSA_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const size_t counts_bytes = ((size_t)problems * sizeof(int32_t) + 255) & ~(size_t)255;
+    int32_t *slot0 = static_cast<int32_t *>(workspace);
+    int32_t *count = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + counts_bytes);
+    hipLaunchKernelGGL(nearest_rows_counts_kernel, dim3((problems + 255) / 256), dim3(256), 0, stream, slot0, count, problems, rows);
+    int rc = check_launch("nearest_rows_counts");
+    if (rc) return rc;
+    EncodeArgs a = {};
+    a.kv.k_base = reinterpret_cast<const char *>(vectors);
+    a.kv.v_base = a.kv.k_base;
+    a.kv.stride_seq = (int64_t)rows * kD; a.kv.stride_head = 0; a.kv.stride_tok = kD; a.kv.stride_block = 0;
+    a.kv.block_table = nullptr; a.kv.block_size = 0; a.kv.max_blocks = 0; a.kv.paged = 0; a.kv.esize = 4;
+    a.H = 1; a.L = num_centroids; a.sink = 0; a.slot0 = slot0; a.count = count;
+    a.coarse = centroids; a.eps = eps;
+    a.n_cap = rows;
+    a.assign_out = out; a.assign_stride = out_stride;
+    rc = launch_prefilter(a, PQHSA_F32, problems, rows, static_cast<char *>(workspace) + 2 * counts_bytes,
+                          workspace_bytes - 2 * counts_bytes, &a.hints, &a.hint_stride, stream);
+    if (rc) return rc;
+    return launch_encode(a, PQHSA_F32, problems, rows, stream);
 }
 
 extern "C" int pqhsa_encode_append(const pqhsa_kv_view *kv, const pqhsa_index *index, int32_t sink,

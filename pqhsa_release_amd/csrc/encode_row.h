@@ -27,6 +27,9 @@ struct EncodeArgs {
     // bulk encode with list candidates (NULL: every list is measured)
     const uint32_t *hints;  // [BH, hint_stride] bits 0-11, 12-23: lists to measure; bit 31: measure all
     int64_t hint_stride;
+    // bulk form only: stop after the nearest list and store it here, [BH, assign_stride] (NULL: encode fully)
+    int64_t *assign_out;
+    int64_t assign_stride;
 };
 
 __device__ inline unsigned long long wave_min_u64(unsigned long long v, int width) {

@@ -121,10 +121,18 @@ class _LazyGenerators:
         return self.gens[s]
 
 
-def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int = 1 << 27) -> torch.Tensor:
-    """``vectors [S, N, D]``, ``centroids [S, K, D]`` -> nearest centroid per vector ``[S, N]``."""
+def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int = 1 << 27,
+                     unit_vectors: bool = False) -> torch.Tensor:
+    """``vectors [S, N, D]``, ``centroids [S, K, D]`` -> nearest centroid per vector ``[S, N]``.
+    ``unit_vectors``: the rows are unit directions (the coarse k-means); on the device, with
+    D = 128, their nearest centroids then come from ``pqhsa_nearest_rows`` (matrix-core candidates,
+    fixed-order fp32 decision) instead of a matrix of all products."""
     s, n, _ = vectors.shape
     cf = centroids.float()
+    if (unit_vectors and vectors.is_cuda and vectors.shape[2] == 128 and vectors.dtype == torch.float32
+            and vectors.is_contiguous() and 1 <= cf.shape[1] <= 4096 and n >= 128):
+        from .. import ops
+        return ops.nearest_rows(vectors, cf.contiguous())
     half_sq = (cf * cf).sum(dim=2).unsqueeze(1)
     chunk = max(1024, budget // max(1, s * cf.shape[1]))
     out = torch.empty(s, n, dtype=torch.long, device=vectors.device)
@@ -149,7 +157,8 @@ def _seeded_start(n: int, num_clusters: int, seed: int) -> torch.Tensor:
     return torch.randperm(n, generator=gen)[:num_clusters].clone()
 
 
-def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed=0, eps: float = 1e-12):
+def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int, seed=0, eps: float = 1e-12,
+                      unit_vectors: bool = False):
     """``kmeans_l2`` for ``S`` independent problems of one size, ``vectors [S, N, D]``: the seeded
     start (``seed``: one number for all problems, as S separate calls with one seed would draw,
     or one per problem) and the Lloyd iterations run as batched products; a problem whose
@@ -176,7 +185,7 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
     offsets = (torch.arange(s, device=dev) * num_clusters).unsqueeze(1)
     flat = vectors.reshape(s * n, dim).float()
     for _ in range(max_iter):
-        nxt = _nearest_batched(vectors, centroids)
+        nxt = _nearest_batched(vectors, centroids, unit_vectors=unit_vectors)
         same = (assign == nxt).all(dim=1)
         assign = torch.where(live.unsqueeze(1), nxt, assign)
         live = live & ~same
@@ -206,7 +215,7 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
                 pick = torch.randint(0, n, (int(empty[i].sum().item()),), generator=lazy.get(i)).to(dev)
                 sums[i][empty[i]] = vectors[i][pick].float()
         centroids = torch.where(live.view(s, 1, 1), sums.to(vectors.dtype), centroids)
-    return centroids, _nearest_batched(vectors, centroids)
+    return centroids, _nearest_batched(vectors, centroids, unit_vectors=unit_vectors)
 
 
 def train_ivfpq_batched(keys: torch.Tensor, *, num_lists: int, num_subspaces: int = 8, num_codes: int = 16,
@@ -221,7 +230,7 @@ def train_ivfpq_batched(keys: torch.Tensor, *, num_lists: int, num_subspaces: in
     norms = torch.linalg.vector_norm(k32, dim=-1).clamp_min(eps)
     dirs = k32 / norms.unsqueeze(-1)
     lists = min(int(num_lists), dirs.shape[1])
-    coarse, assign = kmeans_l2_batched(dirs, lists, max_iter=coarse_iter, seed=seed, eps=eps)
+    coarse, assign = kmeans_l2_batched(dirs, lists, max_iter=coarse_iter, seed=seed, eps=eps, unit_vectors=True)
     resid = dirs - torch.gather(coarse, 1, assign.unsqueeze(-1).expand(-1, -1, dirs.shape[2]))
     sub = keys.shape[2] // num_subspaces
     chunks = resid.reshape(resid.shape[0], resid.shape[1], num_subspaces, sub)

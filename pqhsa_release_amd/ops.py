@@ -362,6 +362,25 @@ def encode(kv: KvSource, index: DeviceIndex, sink: int, slot0, count, *, eps: fl
     _lib.check(rc, "pqhsa_encode")
 
 
+def nearest_rows(vectors: torch.Tensor, centroids: torch.Tensor, *, eps: float = EPS) -> torch.Tensor:
+    """Nearest centroid to the direction of every row: ``vectors [P, R, 128]``, ``centroids
+    [P, K, 128]`` contiguous fp32 -> int64 ``[P, R]`` (``pqhsa_nearest_rows``; K <= 4096)."""
+    _need_cuda(vectors, centroids)
+    p, r, d = vectors.shape
+    k = centroids.shape[1]
+    if (d != HEAD_DIM or tuple(centroids.shape) != (p, k, HEAD_DIM) or vectors.dtype != torch.float32
+            or centroids.dtype != torch.float32 or not vectors.is_contiguous() or not centroids.is_contiguous()):
+        raise ValueError(f"nearest_rows: vectors [P, R, {HEAD_DIM}] and centroids [P, K, {HEAD_DIM}] contiguous fp32")
+    lib = _lib.load()
+    out = torch.empty(p, r, dtype=torch.int64, device=vectors.device)
+    need = lib.pqhsa_nearest_rows_workspace_bytes(p, k, r)
+    ws = torch.empty(need, dtype=torch.uint8, device=vectors.device)
+    rc = lib.pqhsa_nearest_rows(vectors.data_ptr(), centroids.data_ptr(), p, r, k, eps, out.data_ptr(), r,
+                                ws.data_ptr(), need, _stream())
+    _lib.check(rc, "pqhsa_nearest_rows")
+    return out
+
+
 def nearest_from_products(dots: torch.Tensor, sq: torch.Tensor, out: torch.Tensor) -> None:
     """``out[p, j]`` = first argmin over k of ``sq[p, k] - 2 * dots[p, j, k]``; ``dots [P, R, K]``
     and ``sq [P, K]`` contiguous fp32, ``out`` int64 ``[P, R]`` with unit stride along R (a column

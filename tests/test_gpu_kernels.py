@@ -134,6 +134,36 @@ def test_encode_with_matrix_core_candidates_equals_the_full_measurement(case):
         assert torch.all(dist[torch.arange(512), torch.from_numpy(lid)] <= best + 1e-5)
 
 
+@pytest.mark.parametrize("k", [1, 5, 48, 512, 1000])
+def test_nearest_rows_gives_the_nearest_centroid_of_every_direction(k):
+    """pqhsa_nearest_rows (the coarse k-means' assignment step): for unit rows the answer is a
+    nearest centroid by a float64 measurement (to the 1e-6 that fp32 distances can tell apart),
+    equal centroid rows go to the lower index, and a row that is not unit is judged by its
+    direction."""
+    dev = _cuda()
+    gen = torch.Generator().manual_seed(100 + k)
+    p, r = 3, 3001
+    centres = torch.randn(p, k, 128, generator=gen)
+    centres = centres / centres.norm(dim=-1, keepdim=True) * (0.5 + 0.5 * torch.rand(p, k, 1, generator=gen))
+    rows = torch.gather(centres, 1, torch.randint(0, k, (p, r), generator=gen).unsqueeze(-1).expand(-1, -1, 128))
+    rows = rows + 0.2 * torch.randn(p, r, 128, generator=gen)
+    rows = rows / rows.norm(dim=-1, keepdim=True)
+    if k >= 5:
+        centres[:, 4] = centres[:, 1]                    # equal rows: 1 wins over 4
+    rows[:, 7] *= 37.0                                   # not unit: judged by its direction
+    got = ops.nearest_rows(rows.to(dev), centres.to(dev)).cpu()
+    unit = (rows / rows.norm(dim=-1, keepdim=True)).double()
+    dist = torch.cdist(unit, centres.double()) ** 2
+    best = dist.min(dim=2).values
+    mine = torch.gather(dist, 2, got.unsqueeze(-1)).squeeze(-1)
+    assert bool((mine <= best + 1e-6).all())
+    assert int((got == 4).sum()) == 0 or k < 5
+    fp32 = ((centres * centres).sum(-1).unsqueeze(1) - 2.0 * torch.bmm(unit.float(), centres.transpose(1, 2))).argmin(dim=2)
+    if k >= 5:
+        fp32[fp32 == 4] = 1                              # (a product matrix may round the twin columns apart)
+    assert float((got == fp32).float().mean()) > 0.999
+
+
 @pytest.mark.parametrize("k", [1, 3, 16, 17, 32, 36, 512, 600, 1024, 2000])
 def test_nearest_from_products_is_the_elementwise_argmin(k):
     """pqhsa_nearest_from_products against the three torch ops it stands for, bit for bit: equal
