@@ -169,6 +169,18 @@ int pqhsa_nearest_rows(const float *vectors, const float *centroids, int32_t pro
                        void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The assignment step of the codebook k-means in index training: rows of 16 numbers (one subspace
+ * of a residual) against the 16 codewords of their problem, out[p * out_stride + j] = the first
+ * codeword at the smallest fixed-order fp32 distance (the measure of pqhsa_encode's code search).
+ * rows [problems, rows_per_problem, 16] and words [problems, 16, 16] fp32, contiguous, rows
+ * 16-byte aligned.  Replaces _nearest_centroids_chunked (pq_hsa/index/kmeans.py:108-131) for the
+ * subspace problems of ProductQuantizer.train (pq_hsa/index/pq.py:47-95); nearly equal distances
+ * may fall the other way than in its |c|^2 - 2<v,c> form.
+ */
+int pqhsa_nearest_codewords(const float *rows, const float *words, int32_t problems, int64_t rows_per_problem,
+                            int64_t *out, int64_t out_stride, void *stream);
+
+/*
  * The assignment step of index training after its matrix product: for problem p and vector j,
  * out[p * out_stride + j] = the first k that minimises sq[p, k] - 2 * dots[p, j, k] (a NaN counts
  * as smallest, as in torch.argmin).  dots [problems, rows, K] and sq [problems, K] contiguous and

@@ -88,6 +88,7 @@ SIGNATURES = {
     "pqhsa_nearest_rows_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "pqhsa_nearest_rows": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_float, c_void_p, c_int64,
                                           c_void_p, c_size_t, c_void_p]),
+    "pqhsa_nearest_codewords": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_int64, c_void_p]),
     "pqhsa_nearest_from_products": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int64,
                                                    c_void_p]),
     "pqhsa_value_summaries": (ctypes.c_int, [_P(KvView), _P(Index), c_int32, c_int32, c_void_p]),

@@ -57,9 +57,60 @@ __global__ __launch_bounds__(kNearThreads) void nearest_kernel(const float *__re
     if (live && j == 0) out[problem * out_stride + (row - problem * rows_per_problem)] = bi;
 }
 
+// The assignment step of the codebook k-means: rows of kSub = 16 numbers (one subspace of a
+// residual) against the 16 codewords of their problem, by the encode kernel's own measure: the
+// left-to-right chain t = x - c, acc = fma(t, t, acc), first strict minimum.  One thread per row;
+// a workgroup's rows belong to one problem, whose codewords sit in LDS (every lane reads the same
+// word: a broadcast).
+__global__ __launch_bounds__(kNearThreads) void nearest_codeword_kernel(const float *__restrict__ rows, const float *__restrict__ words,
+                                                                        int64_t rows_per_problem, int64_t *__restrict__ out,
+                                                                        int64_t out_stride) {
+    __shared__ __align__(16) float w_s[kCodes * kSub];
+    const int problem = blockIdx.y;
+    const int64_t r = (int64_t)blockIdx.x * kNearThreads + threadIdx.x;
+    for (int i = threadIdx.x; i < kCodes * kSub; i += kNearThreads) w_s[i] = words[(size_t)problem * kCodes * kSub + i];
+    __syncthreads();
+    if (r >= rows_per_problem) return;
+    const float4 *src = reinterpret_cast<const float4 *>(rows + ((size_t)problem * rows_per_problem + r) * kSub);
+    float x[kSub];
+#pragma unroll
+    for (int q = 0; q < kSub / 4; ++q) {
+        const float4 v = src[q];
+        x[4 * q] = v.x; x[4 * q + 1] = v.y; x[4 * q + 2] = v.z; x[4 * q + 3] = v.w;
+    }
+    int best = 0;
+    float bd = INFINITY;
+#pragma unroll 4
+    for (int c = 0; c < kCodes; ++c) {
+        float d2 = 0.0f;
+#pragma unroll
+        for (int e = 0; e < kSub; ++e) {
+            const float t = x[e] - w_s[c * kSub + e];
+            d2 = __builtin_fmaf(t, t, d2);
+        }
+        if (d2 < bd) { bd = d2; best = c; }
+    }
+    out[(size_t)problem * out_stride + r] = best;
+}
+
 }  // namespace pqhsa
 
 using namespace pqhsa;
+
+extern "C" int pqhsa_nearest_codewords(const float *rows, const float *words, int32_t problems, int64_t rows_per_problem,
+                                       int64_t *out, int64_t out_stride, void *stream_v) {
+    PQHSA_REQUIRE(rows && words && out, "nearest_codewords: NULL argument");
+    PQHSA_REQUIRE(problems >= 0 && problems <= 65535 && rows_per_problem >= 0, "nearest_codewords: problems=%d rows=%lld",
+                  problems, (long long)rows_per_problem);
+    PQHSA_REQUIRE(((uintptr_t)rows & 15) == 0, "nearest_codewords: rows not 16-byte aligned");
+    if (problems == 0 || rows_per_problem == 0) return PQHSA_OK;
+    const int64_t blocks = (rows_per_problem + kNearThreads - 1) / kNearThreads;
+    PQHSA_REQUIRE(blocks < (1ll << 31), "nearest_codewords: %lld rows per problem are too many for one launch",
+                  (long long)rows_per_problem);
+    hipLaunchKernelGGL(nearest_codeword_kernel, dim3((unsigned)blocks, problems), dim3(kNearThreads), 0,
+                       static_cast<hipStream_t>(stream_v), rows, words, rows_per_problem, out, out_stride);
+    return check_launch("nearest_codewords");
+}
 
 extern "C" int pqhsa_nearest_from_products(const float *dots, const float *sq, int32_t problems, int64_t rows,
                                            int32_t K, int64_t *out, int64_t out_stride, void *stream_v) {

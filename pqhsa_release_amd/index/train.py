@@ -126,13 +126,19 @@ def _nearest_batched(vectors: torch.Tensor, centroids: torch.Tensor, budget: int
     """``vectors [S, N, D]``, ``centroids [S, K, D]`` -> nearest centroid per vector ``[S, N]``.
     ``unit_vectors``: the rows are unit directions (the coarse k-means); on the device, with
     D = 128, their nearest centroids then come from ``pqhsa_nearest_rows`` (matrix-core candidates,
-    fixed-order fp32 decision) instead of a matrix of all products."""
+    fixed-order fp32 decision) instead of a matrix of all products.  The subspace problems of the
+    codebooks (D = 16 against 16 codewords) likewise go through ``pqhsa_nearest_codewords`` on the
+    device.  Elsewhere: the reference's product form, with the arg-min fused on the device."""
     s, n, _ = vectors.shape
     cf = centroids.float()
     if (unit_vectors and vectors.is_cuda and vectors.shape[2] == 128 and vectors.dtype == torch.float32
             and vectors.is_contiguous() and 1 <= cf.shape[1] <= 4096 and n >= 128):
         from .. import ops
         return ops.nearest_rows(vectors, cf.contiguous())
+    if (vectors.is_cuda and vectors.shape[2] == 16 and cf.shape[1] == 16 and vectors.dtype == torch.float32
+            and vectors.is_contiguous() and s <= 65535):
+        from .. import ops   # the subspace problems of the codebooks: one pass over the rows, no products
+        return ops.nearest_codewords(vectors, cf.contiguous())
     half_sq = (cf * cf).sum(dim=2).unsqueeze(1)
     chunk = max(1024, budget // max(1, s * cf.shape[1]))
     out = torch.empty(s, n, dtype=torch.long, device=vectors.device)

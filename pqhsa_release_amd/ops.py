@@ -381,6 +381,20 @@ def nearest_rows(vectors: torch.Tensor, centroids: torch.Tensor, *, eps: float =
     return out
 
 
+def nearest_codewords(rows: torch.Tensor, words: torch.Tensor) -> torch.Tensor:
+    """``rows [P, R, 16]`` against ``words [P, 16, 16]`` (contiguous fp32): the nearest codeword of
+    every row, int64 ``[P, R]`` (``pqhsa_nearest_codewords``)."""
+    _need_cuda(rows, words)
+    p, r, d = rows.shape
+    if (d != SUBDIM or tuple(words.shape) != (p, CODES, SUBDIM) or rows.dtype != torch.float32
+            or words.dtype != torch.float32 or not rows.is_contiguous() or not words.is_contiguous()):
+        raise ValueError(f"nearest_codewords: rows [P, R, {SUBDIM}] and words [P, {CODES}, {SUBDIM}] contiguous fp32")
+    out = torch.empty(p, r, dtype=torch.int64, device=rows.device)
+    rc = _lib.load().pqhsa_nearest_codewords(rows.data_ptr(), words.data_ptr(), p, r, out.data_ptr(), r, _stream())
+    _lib.check(rc, "pqhsa_nearest_codewords")
+    return out
+
+
 def nearest_from_products(dots: torch.Tensor, sq: torch.Tensor, out: torch.Tensor) -> None:
     """``out[p, j]`` = first argmin over k of ``sq[p, k] - 2 * dots[p, j, k]``; ``dots [P, R, K]``
     and ``sq [P, K]`` contiguous fp32, ``out`` int64 ``[P, R]`` with unit stride along R (a column

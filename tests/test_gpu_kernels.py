@@ -164,6 +164,27 @@ def test_nearest_rows_gives_the_nearest_centroid_of_every_direction(k):
     assert float((got == fp32).float().mean()) > 0.999
 
 
+def test_nearest_codewords_gives_the_nearest_codeword_of_every_row():
+    """pqhsa_nearest_codewords (the codebook k-means' assignment step): a nearest codeword by a
+    float64 measurement for every row, the lower index among equal codewords, the fp32 product
+    form's answer almost everywhere."""
+    dev = _cuda()
+    gen = torch.Generator().manual_seed(31)
+    p, r = 5, 4099
+    words = 0.2 * torch.randn(p, 16, 16, generator=gen)
+    words[:, 9] = words[:, 2]                                        # equal codewords: 2 wins over 9
+    rows = torch.gather(words, 1, torch.randint(0, 16, (p, r), generator=gen).unsqueeze(-1).expand(-1, -1, 16))
+    rows = rows + 0.05 * torch.randn(p, r, 16, generator=gen)
+    got = ops.nearest_codewords(rows.to(dev), words.to(dev)).cpu()
+    dist = torch.cdist(rows.double(), words.double()) ** 2
+    mine = torch.gather(dist, 2, got.unsqueeze(-1)).squeeze(-1)
+    assert bool((mine <= dist.min(dim=2).values + 1e-9).all())
+    assert int((got == 9).sum()) == 0
+    fp32 = ((words * words).sum(-1).unsqueeze(1) - 2.0 * torch.bmm(rows, words.transpose(1, 2))).argmin(dim=2)
+    fp32[fp32 == 9] = 2
+    assert float((got == fp32).float().mean()) > 0.999
+
+
 @pytest.mark.parametrize("k", [1, 3, 16, 17, 32, 36, 512, 600, 1024, 2000])
 def test_nearest_from_products_is_the_elementwise_argmin(k):
     """pqhsa_nearest_from_products against the three torch ops it stands for, bit for bit: equal
