@@ -120,12 +120,12 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, size_t orow, int b,
     __shared__ float acc_s[kFoldLanes][kD];
     __shared__ float den_s[kFoldLanes];
     const int tid = threadIdx.x;
-    __builtin_amdgcn_s_waitcnt(0);  // this thread's stores of the partial have completed before the flag is set
+    drain_memory_ops();  // this thread's stores of the partial have completed before the flag is set
     __syncthreads();
     if (tid < kWave) {  // (at most 64 splits: one flag per lane)
         uint32_t *flags = a.arrive + orow * kMaxSplits;
         if (tid == 0) __hip_atomic_store(flags + split, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(0);  // ... and the flag is visible before the row's flags are read
+        drain_memory_ops();  // ... and the flag is visible before the row's flags are read
         const uint32_t set = tid < a.splits ? __hip_atomic_load(flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
         const bool all_set = __ballot(set == 0u) == 0ull;
         if (tid == 0) last_s = all_set && atomicAdd(a.arrive + a.rows * kMaxSplits + orow, 1u) == 0u;

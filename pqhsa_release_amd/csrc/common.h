@@ -293,6 +293,17 @@ __device__ inline float wave_prefix_f32(float v) {
     return v;
 }
 
+// ---- ordering of device-scope accesses without a cache-wide fence --------------------------
+// Waits until every memory operation this wave has issued has completed: a device-scope store
+// (written through to the level all XCDs share) is then visible to device-scope loads of any
+// other workgroup.  The signal fences keep the compiler from moving memory accesses across the
+// wait (the wait itself is not a memory operation to it).
+__device__ inline void drain_memory_ops() {
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
 // k = min(max(ceil(n * fraction), 0), n), or min(topk, n) when no fraction is given
 __host__ __device__ inline int resolve_k(int n, double fraction, int topk) {
     int k;

@@ -31,8 +31,10 @@ __global__ __launch_bounds__(kEncThreads, HINT ? 2 : 3) void encode_bulk_kernel(
     const int slot = a.slot0[b] + j;
     const size_t esz = DT == PQHSA_F32 ? 4 : 2;
 
-    if (!(HINT && a.assign_out))
+    if (!(HINT && a.assign_out)) {  // (uniform over the workgroup, like the early return above)
         for (int i = tid; i < kM * kCodes * kSub; i += kEncThreads) cb_s[i] = a.codebooks[(size_t)bh * kM * kCodes * kSub + i];
+        __syncthreads();  // every wave reads all of cb_s below; the candidate form has no other barrier before that
+    }
 
     float x[kD];
     float nrm = 1.0f;

@@ -1813,9 +1813,18 @@ __global__ __launch_bounds__(kSelThreads) void decode_small_kernel(SmallArgs a) 
 }
 
 // whether the short-context kernel serves a step of this shape
+// dynamic LDS of the short-context kernel: the centroid tile, two tables of L floats, the selected indices
+static size_t decode_small_lds(int L, int k_cap) {
+    return (size_t)kSmallTile * kSmallRow * sizeof(float) + 2 * (size_t)L * sizeof(float) + (size_t)k_cap * sizeof(int32_t);
+}
+
 bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap) {
-    // (one workgroup per query row; tables and selected indices in LDS: 135 KB tile + 8 L + 4 k_cap bytes)
-    return streams > 0 && (int64_t)streams * G <= 256 && n_max <= 16 * kSelThreads && L <= 1024 && k_cap <= 2048;
+    // One workgroup per query row.  Its LDS must fit a compute unit's 160 KB: the dynamic part above
+    // plus the kernel's static arrays (selection scratch, query row, PQ table, partial sums: rounded
+    // up to 14 KB); a shape that does not fit takes the general path.
+    constexpr size_t kStaticLds = 14 * 1024;
+    return streams > 0 && (int64_t)streams * G <= 256 && n_max <= 16 * kSelThreads && L <= 1024 && k_cap <= 2048 &&
+           decode_small_lds(L, k_cap) + kStaticLds <= 160 * 1024;
 }
 
 template <int KDT>
@@ -1845,8 +1854,7 @@ static int launch_decode_small_kdt(const SmallArgs &a, int streams, int64_t n_ma
 
 int launch_decode_small(SmallArgs a, int kv_dtype, int streams, int64_t n_max, hipStream_t stream) {
     a.sel_cap = a.k_cap;
-    const size_t lds = (size_t)kSmallTile * kSmallRow * sizeof(float) + 2 * (size_t)a.L * sizeof(float) +
-                       (size_t)a.sel_cap * sizeof(int32_t);
+    const size_t lds = decode_small_lds(a.L, a.sel_cap);
     int rc;
     if (kv_dtype == PQHSA_F32) rc = launch_decode_small_kdt<PQHSA_F32>(a, streams, n_max, lds, stream);
     else if (kv_dtype == PQHSA_BF16) rc = launch_decode_small_kdt<PQHSA_BF16>(a, streams, n_max, lds, stream);

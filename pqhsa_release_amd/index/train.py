@@ -201,9 +201,19 @@ def kmeans_l2_batched(vectors: torch.Tensor, num_clusters: int, *, max_iter: int
             # Few clusters (the 16 codewords of a subspace): row adds from a million keys would
             # queue up on 16 rows per problem.  The product with the 0/1 membership matrix adds
             # the same terms without that, and its column sums are the counts.
-            member = (assign.unsqueeze(-1) == torch.arange(num_clusters, device=dev)).float()      # [S, N, K]
-            sums = torch.bmm(member.transpose(1, 2), flat.view(s, n, dim)).reshape(s * num_clusters, dim)
-            counts = member.sum(dim=1).reshape(-1)
+            # (the membership matrix [S, rows, K] is formed a slab of rows at a time, under the memory
+            # budget of the assignment step; partial sums of slabs add up in fp32, another order than
+            # one row add per key)
+            ids = torch.arange(num_clusters, device=dev)
+            rows = max(4096, (1 << 27) // max(1, s * num_clusters))
+            sums = torch.zeros(s, num_clusters, dim, dtype=torch.float32, device=dev)
+            counts = torch.zeros(s, num_clusters, dtype=torch.float32, device=dev)
+            vf = flat.view(s, n, dim)
+            for i in range(0, n, rows):
+                member = (assign[:, i : i + rows].unsqueeze(-1) == ids).float()                    # [S, rows, K]
+                sums += torch.bmm(member.transpose(1, 2), vf[:, i : i + rows])
+                counts += member.sum(dim=1)
+            sums, counts = sums.reshape(s * num_clusters, dim), counts.reshape(-1)
         else:
             where = (assign + offsets).reshape(-1)
             sums = torch.zeros(s * num_clusters, dim, dtype=torch.float32, device=dev)

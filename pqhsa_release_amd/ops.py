@@ -587,7 +587,8 @@ class DecodeCall:
 
     def __init__(self, q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int,
                  full_max: int, fraction: float | None, topk: int, scale: float, workspace: DecodeWorkspace,
-                 eps: float = EPS, n_max: int | None = None, append_count: torch.Tensor | None = None) -> None:
+                 eps: float = EPS, n_max: int | None = None, append_count: torch.Tensor | None = None,
+                 general_path: bool = False, flags: int = 0) -> None:
         _need_cuda(q, out, seq_lens)
         if append_count is not None and (append_count.dtype != torch.int32 or append_count.numel() != index.batch
                                          or not append_count.is_cuda):
@@ -604,6 +605,7 @@ class DecodeCall:
         self._sel.fraction = float(fraction) if fraction else 0.0
         self._sel.topk = int(topk)
         self._sel.k_cap = workspace.k_cap
+        self._sel.flags = int(flags) | (_lib.SELECT_GENERAL_PATH if general_path else 0)
         self._sel.n_mean = index.n_mean
         self._keep = (q, out, kv, index, seq_lens, workspace, append_count)
         self.n_max = index.n_max if n_max is None else int(n_max)

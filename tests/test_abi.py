@@ -64,3 +64,61 @@ def test_launch_count_follows_the_short_context_rule():
     assert launches(4, 8192) == 5
     sel.flags, sel.k_cap = 0, 2049
     assert launches(4, 8192) == 5
+
+
+def test_short_context_rule_counts_the_whole_lds_footprint():
+    import ctypes
+
+    lib = _lib.load()
+    index, sel = _lib.Index(), _lib.Select()
+    index.batch, index.kv_heads = 1, 8
+
+    def launches(lists, k_cap):
+        index.num_lists, sel.k_cap = lists, k_cap
+        return lib.pqhsa_decode_step_launches(ctypes.byref(index), 4, 8192, ctypes.byref(sel), 0)
+
+    assert launches(512, 2048) == 1
+    assert launches(1024, 512) == 1
+    # 135 168 + 8 L + 4 k_cap bytes of dynamic LDS plus the static arrays pass 160 KB at this corner
+    assert launches(1024, 2048) == 5
+
+
+def header_struct_fields(name):
+    text = open(os.path.join(ROOT, "include", "pqhsa.h")).read()
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    return [re.search(r"(\w+)\s*$", decl.strip()).group(1) for decl in body.split(";") if decl.strip()]
+
+
+def test_ctypes_mirrors_follow_the_header_field_order():
+    for cname, mirror in (("pqhsa_kv_view", _lib.KvView), ("pqhsa_select", _lib.Select), ("pqhsa_index", _lib.Index)):
+        assert [f[0] for f in mirror._fields_] == header_struct_fields(cname), cname
+
+
+def test_integration_document_stub_matches_the_library_structs():
+    """The binding INTEGRATION.md shows is built from its text and laid over the library's mirrors:
+    same fields, same offsets, same sizes, and the argument list of pqhsa_decode_step."""
+    import ctypes
+
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = re.search(r"```python\n(import ctypes, torch.*?)```", text, flags=re.S).group(1)
+    structs = block[block.index("c_void_p, c_int32"):block.index("# pqhsa_index")]
+    ns = {"ctypes": ctypes}
+    exec(structs, ns)  # two ctypes.Structure definitions written in this repository's own document
+    for doc, mirror in ((ns["KvView"], _lib.KvView), (ns["Select"], _lib.Select)):
+        assert ctypes.sizeof(doc) == ctypes.sizeof(mirror)
+        assert [f[0] for f in doc._fields_] == [f[0] for f in mirror._fields_]
+        for fname, _ in mirror._fields_:
+            assert getattr(doc, fname).offset == getattr(mirror, fname).offset, fname
+            assert getattr(doc, fname).size == getattr(mirror, fname).size, fname
+    argtypes = re.search(r"pqhsa_decode_step\.argtypes = \[(.*?)\]", block, flags=re.S).group(1)
+    argtypes = re.sub(r"#[^\n]*", "", argtypes)
+    names = [a.strip() for a in argtypes.replace("\n", " ").split(",") if a.strip()]
+    ns.update(P=ctypes.POINTER, Index=_lib.Index)
+    got = [eval(a, ns) for a in names]
+    want = _lib.SIGNATURES["pqhsa_decode_step"][1]
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert ctypes.sizeof(g) == ctypes.sizeof(w)
+        assert (g is w) or (hasattr(g, "_type_") and hasattr(w, "_type_") and
+                            [f[0] for f in getattr(g._type_, "_fields_", [])] == [f[0] for f in getattr(w._type_, "_fields_", [])])

@@ -365,7 +365,7 @@ def test_decode_step_topk_bitexact_and_output_close(case, general_path):
     q_dtypes = [torch.float32] if case["dtype"] == torch.float32 else [torch.float32, case["dtype"]]
     for q_dtype in q_dtypes:
         q = p.q_tensor().to(q_dtype)
-        out = torch.empty_like(q)
+        out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
                         fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws, general_path=general_path)
         torch.cuda.synchronize()
@@ -429,7 +429,7 @@ def test_decode_step_all_selected_equals_dense_attention():
     idx = p.device_index(dev)
     kv = ops.kv_contiguous(*p.dense_kv())
     q = p.q_tensor()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ws = ops.DecodeWorkspace(idx, p.G, p.n_max)
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=1.0,
                     topk=0, scale=SCALE, workspace=ws)
@@ -491,7 +491,7 @@ def test_missing_or_bad_arguments_fail_loudly():
 def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
     """(The tests that use this are about the general path's estimate, candidate area and layouts.)"""
     q = p.q_tensor()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
                     topk=0, scale=SCALE, workspace=ws, general_path=general_path)
     torch.cuda.synchronize()
@@ -553,7 +553,7 @@ def test_decode_step_with_device_lengths_beyond_the_host_bounds_exits_normally()
     k_cap = ops.resolve_topk(p.n_max, 0.03, 0)
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
     q = p.q_tensor()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     # one row more on the device than the host sized the attention launch for
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local - 1, fraction=0.03,
                     topk=0, scale=SCALE, workspace=ws, general_path=True)
@@ -655,7 +655,7 @@ def test_hybrid_attend_paged_alone_matches_oracle():
             w = np.exp(logits[g].astype(np.float64) - float(logits[g].max()))
             mass[r] = torch.from_numpy(np.bincount(ix["list_ids"].astype(np.int64), weights=w, minlength=p.L)).float()
     q = p.q_tensor().float()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.hybrid_attend_paged(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
                             topk_idx=tidx.to(dev), topk_val=tval.to(dev), topk_cnt=tcnt.to(dev),
                             list_mass=mass.to(dev), row_max=rmax.to(dev), scale=SCALE)
@@ -724,7 +724,7 @@ def test_full_size_step_properties_at_the_benchmark_shapes(cfg):
     # the same step with fp32 queries and output (K/V stay bf16 in their pages): the stated bound as
     # it is, with no allowance for a 16-bit output's own rounding
     q32 = layer.q.float()
-    out32 = torch.empty_like(q32)
+    out32 = torch.full_like(q32, float("nan"))
     ops.decode_step(q32, out32, layer.kv, idx, G, layer.seq_lens, sink=sink, full_max=sink + bench.LOCAL,
                     fraction=bench.FRACTION, topk=0, scale=1.0 / np.sqrt(128.0), workspace=layer.ws)
     torch.cuda.synchronize()
@@ -781,27 +781,29 @@ def test_append_then_scan_at_the_long_context_shape():
     assert layer.ws.rescans() == 0
 
 
-def test_decode_step_graph_replays_match_eager_runs():
+@pytest.mark.parametrize("general_path", [False, True], ids=["one_launch", "general"])
+def test_decode_step_graph_replays_match_eager_runs(general_path):
     """The step recorded into a HIP graph and replayed several times, with eager work and
-    synchronisations between the replays, gives what the eager step gives for the same query."""
+    synchronisations between the replays: every replay gives the oracle's top-k sets and its
+    outputs within 2e-3 for the query of that round, and what the eager step gives."""
     dev = _cuda()
     p = Problem(lens=[2600, 1900], heads=2, groups=4, lists=32, dtype=torch.bfloat16, seed=43)
     idx = p.device_index(dev)
     kv = ops.kv_paged(*p.paged_kv("5d"))
     q = p.q_tensor().float()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
     call = ops.DecodeCall(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                          fraction=0.03, topk=0, scale=SCALE, workspace=ws)
+                          fraction=0.03, topk=0, scale=SCALE, workspace=ws, general_path=general_path)
     call.capture()
     gen = torch.Generator(device="cpu").manual_seed(5)
     base = q.clone()
     for round_ in range(4):
-        q.copy_(base + 0.3 * round_ * torch.randn(base.shape, generator=gen).to(dev))
+        q.copy_((base + 0.3 * round_ * torch.randn(base.shape, generator=gen).to(dev)).to(p.dtype).float())
         call.run()
         torch.cuda.synchronize()
         want_out, want_idx = out.clone(), ws.topk_idx.clone().sort(dim=1).values
-        out.zero_()
+        out.fill_(float("nan"))
         ws.topk_idx.fill_(-1)
         junk = (torch.randn(512, 512, device=dev) @ torch.randn(512, 512, device=dev)).sum()   # unrelated eager work
         torch.cuda.synchronize()
@@ -810,6 +812,16 @@ def test_decode_step_graph_replays_match_eager_runs():
         assert torch.equal(ws.topk_idx.sort(dim=1).values, want_idx), round_
         np.testing.assert_allclose(out.cpu().numpy(), want_out.cpu().numpy(), atol=1e-5, err_msg=str(round_))
         assert torch.isfinite(junk)
+        # ... and the replay against the fixed-order oracle on this round's query
+        qh = q.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        got_out = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        got_idx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        for (b, h), ix in p.index.items():
+            o_out, o_idx, _ = fixed.decode_step(qh[b, h], p.keys[b, h].numpy(), p.values[b, h].numpy(), ix, sink=p.sink,
+                                                local=p.local, fraction=0.03, scale=SCALE)
+            for g in range(p.G):
+                assert np.array_equal(np.sort(got_idx[b, h, g, : o_idx.shape[1]]), np.sort(o_idx[g])), (round_, b, h, g)
+            assert float(np.abs(got_out[b, h] - o_out).max()) <= 2e-3, (round_, b, h)
 
 
 @pytest.mark.parametrize("lens, heads", [
@@ -830,7 +842,7 @@ def test_ragged_batch_tile_hint_changes_no_result(lens, heads):
     want = {(b, h): p.oracle_step(b, h, 0.03)[1] for (b, h) in p.index}
     first = None
     for hint in (None, 0, 1, 300, p.n_max, 10 ** 9):
-        out = torch.empty_like(q)
+        out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
         ws.topk_idx.fill_(-1)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
                         topk=0, scale=SCALE, workspace=ws, general_path=True, n_mean=hint)
@@ -869,7 +881,7 @@ def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     frac = 0.04
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, frac, 0))
     q = p.q_tensor().float()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     one = torch.ones(p.B, dtype=torch.int32, device=dev)
     seq = torch.tensor(lens0, dtype=torch.int32, device=dev)
     call = ops.DecodeCall(q, out, kv, idx, p.G, seq, sink=p.sink, full_max=p.sink + p.local, fraction=frac, topk=0,
@@ -917,7 +929,7 @@ def test_device_counts_ahead_of_the_host_stay_inside_k_cap():
     assert ops.resolve_topk(n, 0.05, 0) > k_cap
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
     q = p.q_tensor()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     for general_path in (False, True):
         ws.topk_cnt.zero_()
         ops.decode_step(q, out, ops.kv_contiguous(*p.dense_kv()), idx, p.G, p.seq_lens(), sink=p.sink,
@@ -952,7 +964,7 @@ def test_decode_step_random_shapes_match_oracle(seed):
         kv = ops.kv_contiguous(*p.dense_kv()) if layout == "dense" else ops.kv_paged(*p.paged_kv(layout))
         ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, fraction, 0))
         q = p.q_tensor()
-        out = torch.empty_like(q)
+        out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
         general_path = rng.random() < 0.5     # else the single kernel for short contexts, where the shape fits it
         what = what + (general_path,)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
@@ -983,7 +995,7 @@ def test_decode_step_batch_of_more_than_256_query_rows():
     kv = ops.kv_paged(*p.paged_kv("5d"))
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.04, 0))
     q = p.q_tensor().float()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.04,
                     topk=0, scale=SCALE, workspace=ws)
     torch.cuda.synchronize()
@@ -1014,7 +1026,7 @@ def test_decode_step_wide_groups_and_many_lists(groups, lists, lens, general_pat
     kv = ops.kv_paged(*p.paged_kv("5d"))
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.05, 0))
     q = p.q_tensor().float()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.05,
                     topk=0, scale=SCALE, workspace=ws, general_path=general_path)
     torch.cuda.synchronize()
@@ -1112,7 +1124,7 @@ def test_event_log_counts_steps_and_samples_them():
     kv = ops.kv_paged(*p.paged_kv("5d"))
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.02, 0))
     q = p.q_tensor()
-    out = torch.empty_like(q)
+    out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
 
     def steps(count):
         for _ in range(count):

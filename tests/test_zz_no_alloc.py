@@ -24,7 +24,7 @@ def _both_ways(p, fraction):
     seq_lens = p.seq_lens()
     # the existing entry point, with a caller workspace
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
-    want_out = torch.empty_like(q)
+    want_out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.decode_step(q, want_out, kv, idx, p.G, seq_lens, sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
                     topk=0, scale=SCALE, workspace=ws)
     torch.cuda.synchronize()
