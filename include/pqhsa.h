@@ -109,7 +109,7 @@ typedef struct pqhsa_select {
     double fraction;
     int32_t topk;
     int32_t k_cap; /* row stride of topk_idx / topk_val; >= the largest k of the batch */
-    int32_t flags; /* 0, or PQHSA_SELECT_GENERAL_PATH */
+    int32_t flags; /* 0, or PQHSA_SELECT_GENERAL_PATH | PQHSA_SELECT_ONE_LAUNCH */
     int32_t n_mean; /* hint: mean number of indexed keys per sequence of the batch; 0 = unknown (n_max is
                        assumed).  Sizes the scan's tiles so that a ragged batch still fills the chip;
                        results do not depend on it. */
@@ -119,6 +119,13 @@ typedef struct pqhsa_select {
  * query rows in the batch, no append in the step) with one kernel, one workgroup per query row;
  * the results are the same.  This flag keeps such a step on the general five-kernel path. */
 #define PQHSA_SELECT_GENERAL_PATH 1
+/* On the general path, asks for the scan, the selection and the exact attention of a step as ONE
+ * launch whose workgroups hand work to each other through counters in the workspace (three
+ * launches per step instead of five; same results), for batches of sequences of about one length
+ * (n_mean within an eighth of n_max, or a single sequence) with a GQA group of 3 to 8 query rows;
+ * other shapes ignore the flag.  Off by default: on MI355X the three separate launches are
+ * faster (the one launch saves two launch gaps and loses more to device-scope memory traffic). */
+#define PQHSA_SELECT_ONE_LAUNCH 2
 
 const char *pqhsa_version(void);
 const char *pqhsa_last_error(void);
@@ -353,6 +360,14 @@ int pqhsa_decode_step_static(const void *q, int32_t q_dtype, void *out, const pq
 const uint32_t *pqhsa_decode_rescan_counter(void *workspace);
 
 /*
+ * Waits between workgroups of the fused scan + selection + attention launch that ran out since
+ * the workspace was first used (a device-memory counter inside the workspace).  Every such wait
+ * is bounded; one that runs out abandons its step (the output of that step is not valid) instead
+ * of hanging the GPU.  0 in normal operation.  No counterpart in the reference.
+ */
+const uint32_t *pqhsa_decode_fused_aborts(void *workspace);
+
+/*
  * Candidates the last step's scan kept per query row: u32 [B*H, padded_groups(G)] inside the
  * workspace (device memory, for monitoring the threshold estimate; rows of a padded group hold 0).
  */
@@ -361,9 +376,11 @@ const uint32_t *pqhsa_decode_candidate_counts(void *workspace);
 /*
  * Number of kernel launches pqhsa_decode_step makes for a step of this shape: 1 when the
  * short-context kernel serves it (no append, PQHSA_SELECT_GENERAL_PATH not set, at most 16 384
- * indexed keys per stream, at most 256 query rows, at most 1 024 lists, k_cap at most 2 048), else
- * PQHSA_PROFILE_KERNELS.  With one launch the event log books the whole step under its last slot
- * and the other slots hold only the cost of recording an event.  No counterpart in the
+ * indexed keys per stream, at most 256 query rows, at most 1 024 lists, k_cap at most 2 048), 3 when
+ * scan, selection and attention share one launch (see PQHSA_SELECT_ONE_LAUNCH; the event
+ * log books that launch under the scan's slot), else PQHSA_PROFILE_KERNELS.  With one launch the
+ * event log books the whole step under its last slot and the other slots hold only the cost of
+ * recording an event.  No counterpart in the
  * reference; for benchmarks and monitors that label per-kernel times.
  */
 int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t G, int32_t n_max, const pqhsa_select *select,

@@ -68,6 +68,7 @@ class Select(ctypes.Structure):
 
 
 SELECT_GENERAL_PATH = 1
+SELECT_ONE_LAUNCH = 2
 
 
 class PqhsaError(RuntimeError):
@@ -114,6 +115,7 @@ SIGNATURES = {
                                                 c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p]),
     "pqhsa_decode_rescan_counter": (c_void_p, [c_void_p]),
     "pqhsa_decode_candidate_counts": (c_void_p, [c_void_p]),
+    "pqhsa_decode_fused_aborts": (c_void_p, [c_void_p]),
     "pqhsa_attend_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "pqhsa_hybrid_attend_paged": (ctypes.c_int, [c_void_p, c_int32, c_void_p, _P(KvView), _P(Index), c_int32,
                                                  c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,

@@ -148,11 +148,13 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     return check_launch("attend");
 }
 
-int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
-                  int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
-                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
-                  float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
-                  bool even_rows, hipStream_t stream) {
+int attend_splits_room(int rows, int k_cap) { return splits_room(rows, k_cap); }
+
+// the arguments of the decode step's attention (launch shape aside)
+AttendArgs decode_attend_args(const void *q, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
+                              const int32_t *seq_lens, int sink, const int32_t *topk_idx, const int32_t *topk_cnt,
+                              int k_cap, const float *mass, const float *ref_val, float scale, float *partials,
+                              uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
@@ -164,6 +166,16 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
     a.ref0 = ref_val; a.ref_stride = GP;
     a.vbar = index->vbar; a.L = index->num_lists;
     a.n_commit_src = n_commit_src; a.n_commit_dst = n_commit_dst;
+    return a;
+}
+
+int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G,
+                  int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
+                  const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
+                  float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
+                  bool even_rows, hipStream_t stream) {
+    const AttendArgs a = decode_attend_args(q, out, kv, index, G, GP, seq_lens, sink, topk_idx, topk_cnt, k_cap, mass,
+                                            ref_val, scale, partials, arrive, n_commit_src, n_commit_dst);
     return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream, even_rows);
 }
 

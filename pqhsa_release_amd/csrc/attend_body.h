@@ -237,7 +237,7 @@ __device__ inline void attend_body(const AttendArgs &a, const int split, const i
     const int sink_end = min(a.sink, len);
     const int local_start = sink_end + n;
     const int F = sink_end + max(len - local_start, 0);
-    const int k = min(load_shared<FUSED>(a.topk_cnt + orow), (int)a.k_cap);  // never read past the row of the index array
+    const int k = max(min(load_shared<FUSED>(a.topk_cnt + orow), (int)a.k_cap), 0);  // never read past the row of the index array
     // (device-side lengths that ran ahead of the host's full_max are cut to what the launch was sized for)
     const int total = min(F + k, a.chunk_cap * a.splits);
     const int chunk = (total + a.splits - 1) / a.splits;
@@ -284,6 +284,8 @@ __device__ inline void attend_body(const AttendArgs &a, const int split, const i
             if (r < sink_end) pos = r;
             else if (r < F) pos = local_start + (r - sink_end);
             else pos = sink_end + (have ? ahead : load_shared<FUSED>(tk + (r - F)));
+            // (a selected index is a stored key of the sequence; whatever the array holds, the row stays inside it)
+            pos = max((int64_t)0, min(pos, (int64_t)len - 1));
             off_s[i] = row_offset(a.kv, b, h, pos);
         };
 #pragma unroll

@@ -36,6 +36,15 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
                   float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
                   bool even_rows, hipStream_t stream);
+bool decode_fused_fits(int batch, int heads, int G, int64_t n_cap, int64_t n_max, int64_t n_mean, int L);
+int decode_fused(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
+                 const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const float *qnorm, const float *lut,
+                 const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
+                 uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs, int64_t emit_cap, float *mass,
+                 uint32_t *rescans, int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, float *partials,
+                 uint32_t *arrive, uint32_t *sync_words, const AppendFinish *append, const int32_t *n_commit_src,
+                 int32_t *n_commit_dst, hipStream_t stream);
+size_t decode_fused_sync_words(int streams);
 size_t attend_partials_bytes(int rows, int k_cap);
 size_t attend_arrive_bytes(int rows);
 
@@ -43,7 +52,7 @@ static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Carve {
     float *qnorm, *lut, *ls;
-    uint32_t *emit_count, *rescans, *arrive;
+    uint32_t *emit_count, *rescans, *arrive, *sync;
     float *mass;
     size_t zero_words;
     uint32_t *thr_key;
@@ -77,6 +86,7 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.emit_count = reinterpret_cast<uint32_t *>(take(rows * 4));
     c.arrive = reinterpret_cast<uint32_t *>(take(attend_arrive_bytes((int)(BH * G))));  // attention: arrival flags and tickets per query row
     c.mass = reinterpret_cast<float *>(take(rows * L * 4));
+    c.sync = reinterpret_cast<uint32_t *>(take(decode_fused_sync_words((int)BH) * 4));  // the fused launch's progress counters and abort flag
     c.zero_words = (off - z0) / 4;
     c.qnorm = reinterpret_cast<float *>(take(rows * 4));
     c.lut = reinterpret_cast<float *>(take(rows * kM * kCodes * 4));
@@ -118,6 +128,12 @@ extern "C" const uint32_t *pqhsa_decode_rescan_counter(void *workspace) {
     return reinterpret_cast<const uint32_t *>(base);  // the first block of the carve-up
 }
 
+// Waits of the fused launch that ran out (each aborts its step), since the workspace was created.
+extern "C" const uint32_t *pqhsa_decode_fused_aborts(void *workspace) {
+    char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
+    return reinterpret_cast<const uint32_t *>(base) + 1;
+}
+
 extern "C" const uint32_t *pqhsa_decode_candidate_counts(void *workspace) {
     char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
     return reinterpret_cast<const uint32_t *>(base + 256);  // the second block of the carve-up
@@ -128,7 +144,10 @@ extern "C" int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t 
     if (!index || !select) return 0;
     const bool small = !appending && !(select->flags & PQHSA_SELECT_GENERAL_PATH) &&
                        decode_small_fits(index->batch * index->kv_heads, G, n_max, index->num_lists, select->k_cap);
-    return small ? 1 : PQHSA_PROFILE_KERNELS;
+    if (small) return 1;
+    const bool fused = (select->flags & PQHSA_SELECT_ONE_LAUNCH) &&
+                       decode_fused_fits(index->batch, index->kv_heads, G, index->n_cap, n_max, select->n_mean, index->num_lists);
+    return fused ? 3 : PQHSA_PROFILE_KERNELS;
 }
 
 static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
@@ -190,6 +209,12 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
                           append_count ? &ap : nullptr, c.n_after, c.nearest, stream);
     if (rc) return rc;
     profile_mark(kProfSample, stream);
+    if (pqhsa_decode_step_launches(index_in, G, n_max, select, append_count != nullptr) == 3)
+        return decode_fused(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, n_max, full_max + select->k_cap, c.qnorm, c.lut,
+                            c.ls, scale, select, c.emit_count, c.thr_key, c.k_row, c.ref_val, c.pairs, c.emit_cap, c.mass,
+                            c.rescans, topk_idx, topk_val, topk_cnt, c.partials, c.arrive, c.sync,
+                            append_count ? &ap : nullptr, append_count ? c.n_after : nullptr,
+                            append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
                             c.k_row, c.ref_val, c.pairs, c.aux, c.emit_cap, c.mass, c.rescans,
                             topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);

@@ -1330,15 +1330,21 @@ int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
 
 int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream);
 
-// sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
-int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
-                       const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
-                       uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
-                       uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
-                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
-                       hipStream_t stream) {
+// what the threshold estimate aims at for the longest row, plus its tolerance and a margin
+int64_t decode_expected_candidates(const pqhsa_index *index, int64_t n_max, const pqhsa_select *select) {
+    const double ns = (double)(index->s_cap < n_max ? index->s_cap : n_max);
+    const int kmax = resolve_k((int)n_max, select->fraction, select->topk);
+    const double ks = (double)(kmax > 1 ? kmax : 1) * ns / (double)(n_max > 1 ? n_max : 1);
+    const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
+    return (int64_t)((ceil(x * x) + 1.0) * 1.125 * ((double)n_max / (ns > 1.0 ? ns : 1.0)) * 1.12) + 64;
+}
+
+// threshold per row from the sampled keys (and, in a step that appends, the rest of the append);
+// thr_key is two rows long: the thresholds, then the largest sampled keys
+int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnorm, const float *lut,
+                      const float *list_scores, float scale, const pqhsa_select *select, uint32_t *thr_key,
+                      int32_t *k_row, float *ref_val, const AppendFinish *append, hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
-    // 1. threshold per row from the sampled keys (and, in a step that appends, the rest of the append)
     SampleArgs sa = {};
     sa.codes = index->s_codes; sa.list_ids = index->s_list_ids; sa.norms = index->s_norms; sa.s_cap = index->s_cap;
     sa.n_arr = index->n_idx; sa.ns_arr = index->s_n; sa.n_div = index->kv_heads;
@@ -1346,12 +1352,14 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
     sa.k_cap = select->k_cap;
     if (append) sa.append = *append;
-    uint32_t *hi_key = thr_key + (size_t)streams * GP;  // the threshold array is two rows long
-    sa.thr_key = thr_key; sa.hi_key = hi_key; sa.k_row = k_row; sa.ref_val = ref_val;
-    int rc = launch_sample_thresh(sa, streams, stream);
-    if (rc) return rc;
-    profile_mark(kProfEmit, stream);
-    // 2. the full scan
+    sa.thr_key = thr_key; sa.hi_key = thr_key + (size_t)streams * GP; sa.k_row = k_row; sa.ref_val = ref_val;
+    return launch_sample_thresh(sa, streams, stream);
+}
+
+// the arguments of the decode step's scan (launch shape aside)
+ScanArgs decode_scan_args(const pqhsa_index *index, int G, const float *qnorm, const float *lut, const float *list_scores,
+                          float scale, uint32_t *emit_count, uint32_t *thr_key, float *ref_val, void *pairs, uint16_t *aux,
+                          int64_t emit_cap, float *mass) {
     ScanArgs a = {};
     a.qnorm = qnorm; a.lut = lut; a.list_scores = list_scores; a.scale = scale; a.L = index->num_lists;
     a.n_div = index->kv_heads; a.G = G;
@@ -1360,6 +1368,25 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
     a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = emit_cap;
     a.mass = mass;
+    return a;
+}
+
+// sampled keys -> threshold estimate -> fused scan (candidates + per-list background) -> exact selection
+int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, const float *qnorm, const float *lut,
+                       const float *list_scores, float scale, const pqhsa_select *select, uint32_t *emit_count,
+                       uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
+                       uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
+                       int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
+                       hipStream_t stream) {
+    const int streams = index->batch * index->kv_heads;
+    // 1. threshold per row from the sampled keys
+    int rc = decode_thresholds(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val, append, stream);
+    if (rc) return rc;
+    uint32_t *hi_key = thr_key + (size_t)streams * GP;
+    profile_mark(kProfEmit, stream);
+    // 2. the full scan
+    const ScanArgs a = decode_scan_args(index, G, qnorm, lut, list_scores, scale, emit_count, thr_key, ref_val, pairs, aux,
+                                        emit_cap, mass);
     rc = launch_scan_emit(a, GP, streams, n_max, select->n_mean, stream);
     if (rc) return rc;
     profile_mark(kProfSelect, stream);
@@ -1372,14 +1399,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
     s.n_cap = index->n_cap; s.qnorm = qnorm; s.lut = lut; s.list_scores = list_scores; s.scale = scale;
     s.rescans = rescans;
-    {
-        // what the threshold estimate aims at for the longest row, plus its tolerance and a margin
-        const double ns = (double)(index->s_cap < n_max ? index->s_cap : n_max);
-        const int kmax = resolve_k((int)n_max, select->fraction, select->topk);
-        const double ks = (double)(kmax > 1 ? kmax : 1) * ns / (double)(n_max > 1 ? n_max : 1);
-        const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
-        s.expected_candidates = (int64_t)((ceil(x * x) + 1.0) * 1.125 * ((double)n_max / (ns > 1.0 ? ns : 1.0)) * 1.12) + 64;
-    }
+    s.expected_candidates = decode_expected_candidates(index, n_max, select);
     rc = launch_select_final(s, streams, stream);
     profile_mark(kProfAttend, stream);
     return rc;

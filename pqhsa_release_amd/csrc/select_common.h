@@ -542,11 +542,12 @@ __device__ inline void store_dev(uint2 *p, uint2 v) {
 struct PackedRecords {
     const uint2 *pairs;
     const int32_t *pos;  // the stream's position map
+    uint32_t pos_n, L;   // its length, and the number of lists (what a record holds is cut to them)
     __device__ inline uint32_t key(uint32_t p) const { return order_key(__uint_as_float(load_dev(pairs + p).x)); }
     __device__ inline CandRec rec(uint32_t p) const {
         const uint2 pr = load_dev(pairs + p);
-        const uint32_t stored = pr.y & kPackedPosMask;
-        return {order_key(__uint_as_float(pr.x)), (uint32_t)pos[stored], pr.y >> kPackedPosBits};
+        const uint32_t stored = min(pr.y & kPackedPosMask, pos_n - 1u);
+        return {order_key(__uint_as_float(pr.x)), (uint32_t)pos[stored], min(pr.y >> kPackedPosBits, L - 1u)};
     }
 };
 // every stored key of a stream as a candidate, scored again on every pass (a row whose estimate

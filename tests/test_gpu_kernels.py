@@ -345,10 +345,11 @@ def test_topk_radix_on_logit_matrix_with_ties(stride):
     dict(lens=[2200], heads=2, groups=7, lists=48, dtype=torch.bfloat16, fraction=0.02, kv="5d"),
     dict(lens=[1500], heads=1, groups=2, lists=16, dtype=torch.float16, fraction=0.1, kv="dense"),
 ])
-@pytest.mark.parametrize("general_path", [False, True])
+@pytest.mark.parametrize("general_path", [False, True, "fused"], ids=["short_context_kernel", "general", "general_one_launch"])
 def test_decode_step_topk_bitexact_and_output_close(case, general_path):
-    """Both forms of the step against the oracle: the single kernel that serves short contexts
-    (taken by default at these sizes) and the general five-kernel path."""
+    """All forms of the step against the oracle: the single kernel that serves short contexts
+    (taken by default at these sizes), the general path (scan, selection and attention, each its own
+    kernel where the shape allows) and the general path with those three in one launch."""
     dev = _cuda()
     p = Problem(lens=case["lens"], heads=case["heads"], groups=case["groups"], lists=case["lists"],
                 dtype=case["dtype"], seed=13)
@@ -367,7 +368,7 @@ def test_decode_step_topk_bitexact_and_output_close(case, general_path):
         q = p.q_tensor().to(q_dtype)
         out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                        fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                        fraction=case["fraction"], topk=0, scale=SCALE, workspace=ws, **_path(general_path))
         torch.cuda.synchronize()
         tol = 1e-4 if case["dtype"] == torch.float32 else 2e-3
         rel = 0.0 if q_dtype == torch.float32 else (2.0 ** -8 if q_dtype == torch.bfloat16 else 2.0 ** -11)
@@ -488,13 +489,26 @@ def test_missing_or_bad_arguments_fail_loudly():
         ops.lut_build(torch.zeros(1, 17, 128, device=dev), idx, 17)         # G too large
 
 
+def _path(general_path):
+    """Keyword arguments that pick the form of the step: False = the default (one kernel for short
+    contexts), True = the general path, "fused" = the general path with scan, selection and
+    attention in one launch (where the shape allows; else the flag changes nothing)."""
+    return dict(general_path=bool(general_path), one_launch=general_path == "fused")
+
+
 def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
-    """(The tests that use this are about the general path's estimate, candidate area and layouts.)"""
+    """(The tests that use this are about the general path's estimate, candidate area and layouts:
+    both of its forms are run, the three launches and the one-launch scan + selection + attention.)"""
+    runs = 1
+    if general_path is True and ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 3:
+        runs += _check_step(p, idx, kv, ws, fraction, tol, "fused")
     q = p.q_tensor()
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
+    ws.topk_idx.fill_(-1)
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
-                    topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                    topk=0, scale=SCALE, workspace=ws, **_path(general_path))
     torch.cuda.synchronize()
+    assert ws.fused_aborts() == 0
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
     o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
     for (b, h) in p.index:
@@ -503,6 +517,7 @@ def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
         for g in range(p.G):
             assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (b, h, g)
         assert np.abs(o[b, h] - want_out).max() <= tol, (b, h)
+    return runs
 
 
 def test_decode_step_rescans_rows_when_the_sampled_threshold_keeps_too_few():
@@ -520,8 +535,8 @@ def test_decode_step_rescans_rows_when_the_sampled_threshold_keeps_too_few():
     idx.s_codes[0, :ns], idx.s_list_ids[0, :ns], idx.s_norms[0, :ns] = codes[pick], lists[pick], norms[pick]
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.02, 0))
     before = ws.rescans()
-    _check_step(p, idx, ops.kv_contiguous(*p.dense_kv()), ws, 0.02)
-    assert ws.rescans() - before == p.G, "both rows should have taken the full re-scan"
+    runs = _check_step(p, idx, ops.kv_contiguous(*p.dense_kv()), ws, 0.02)
+    assert ws.rescans() - before == p.G * runs, "both rows should have taken the full re-scan"
     assert int(ws.candidate_counts()[0, : p.G].max()) < ops.resolve_topk(p.n_max, 0.02, 0)
 
 
@@ -535,8 +550,8 @@ def test_decode_step_selects_from_a_full_pass_when_candidates_outgrow_their_area
     k_cap = ops.resolve_topk(p.n_max, 0.02, 0)
     assert p.n(1) > 3 * k_cap + 2048
     ws = ops.DecodeWorkspace(raw, p.G, k_cap)
-    _check_step(p, raw, ops.kv_contiguous(*p.dense_kv()), ws, 0.02)
-    assert ws.rescans() == p.B * p.H * p.G
+    runs = _check_step(p, raw, ops.kv_contiguous(*p.dense_kv()), ws, 0.02)
+    assert ws.rescans() == p.B * p.H * p.G * runs
     assert int(ws.candidate_counts()[:, : p.G].min()) == p.n(1)   # the scan counted every key of the shorter row
 
 
@@ -565,11 +580,11 @@ def test_decode_step_with_device_lengths_beyond_the_host_bounds_exits_normally()
         for g in range(p.G):
             assert np.array_equal(np.sort(tidx[b, h, g, : want_idx.shape[1]]), np.sort(want_idx[g])), (b, h, g)
     # a scan sized for fewer keys than the device-side counts say
-    for general_path in (False, True):   # (the single-kernel form clamps the same way)
+    for general_path in (False, True, "fused"):   # (the single-kernel form clamps the same way)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local - 1, fraction=0.03,
-                        topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                        topk=0, scale=SCALE, workspace=ws, **_path(general_path))
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
-                        topk=0, scale=SCALE, workspace=ws, n_max=p.n_max - 1500, general_path=general_path)
+                        topk=0, scale=SCALE, workspace=ws, n_max=p.n_max - 1500, **_path(general_path))
         torch.cuda.synchronize()
         assert torch.isfinite(out.float()).all()
     cnt = ws.topk_cnt.cpu().numpy()
@@ -781,7 +796,7 @@ def test_append_then_scan_at_the_long_context_shape():
     assert layer.ws.rescans() == 0
 
 
-@pytest.mark.parametrize("general_path", [False, True], ids=["one_launch", "general"])
+@pytest.mark.parametrize("general_path", [False, True, "fused"], ids=["short_context_kernel", "general", "general_one_launch"])
 def test_decode_step_graph_replays_match_eager_runs(general_path):
     """The step recorded into a HIP graph and replayed several times, with eager work and
     synchronisations between the replays: every replay gives the oracle's top-k sets and its
@@ -794,7 +809,7 @@ def test_decode_step_graph_replays_match_eager_runs(general_path):
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
     call = ops.DecodeCall(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                          fraction=0.03, topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                          fraction=0.03, topk=0, scale=SCALE, workspace=ws, **_path(general_path))
     call.capture()
     gen = torch.Generator(device="cpu").manual_seed(5)
     base = q.clone()
@@ -930,18 +945,18 @@ def test_device_counts_ahead_of_the_host_stay_inside_k_cap():
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
     q = p.q_tensor()
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
-    for general_path in (False, True):
+    for general_path in (False, True, "fused"):
         ws.topk_cnt.zero_()
         ops.decode_step(q, out, ops.kv_contiguous(*p.dense_kv()), idx, p.G, p.seq_lens(), sink=p.sink,
                         full_max=p.sink + p.local, fraction=0.05, topk=0, scale=SCALE, workspace=ws, n_max=small,
-                        general_path=general_path)
+                        **_path(general_path))
         torch.cuda.synchronize()
         assert ws.topk_cnt.cpu().tolist() == [k_cap] * p.G
         got = ws.topk_idx.cpu().numpy()
         assert ((got >= 0) & (got < n)).all() and bool(torch.isfinite(out).all())
 
 
-@pytest.mark.parametrize("seed", [1, 2])
+@pytest.mark.parametrize("seed", [1, 2, 3])
 def test_decode_step_random_shapes_match_oracle(seed):
     """A seeded sweep over batch sizes, ragged lengths, group widths, list counts, dtypes, page
     layouts, selection fractions and sorted / insertion-order layouts: top-k sets bit-exact,
@@ -965,10 +980,11 @@ def test_decode_step_random_shapes_match_oracle(seed):
         ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, fraction, 0))
         q = p.q_tensor()
         out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
-        general_path = rng.random() < 0.5     # else the single kernel for short contexts, where the shape fits it
+        # the single kernel for short contexts where the shape fits it, or the general path in either form
+        general_path = rng.choice([False, False, True, "fused"])
         what = what + (general_path,)
         ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                        fraction=fraction, topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                        fraction=fraction, topk=0, scale=SCALE, workspace=ws, **_path(general_path))
         torch.cuda.synchronize()
         tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
         o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
@@ -1015,7 +1031,7 @@ def test_decode_step_batch_of_more_than_256_query_rows():
     assert ws.rescans() == 0
 
 
-@pytest.mark.parametrize("general_path", [False, True])
+@pytest.mark.parametrize("general_path", [False, True, "fused"], ids=["short_context_kernel", "general", "general_one_launch"])
 @pytest.mark.parametrize("groups,lists,lens", [(16, 64, [2600]), (12, 256, [5000, 1700]), (9, 512, [7000])])
 def test_decode_step_wide_groups_and_many_lists(groups, lists, lens, general_path):
     """Query groups of 9 to 16 rows (padded to 16 in the kernels) and list counts up to the
@@ -1028,7 +1044,7 @@ def test_decode_step_wide_groups_and_many_lists(groups, lists, lens, general_pat
     q = p.q_tensor().float()
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.05,
-                    topk=0, scale=SCALE, workspace=ws, general_path=general_path)
+                    topk=0, scale=SCALE, workspace=ws, **_path(general_path))
     torch.cuda.synchronize()
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
     o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
