@@ -109,7 +109,7 @@ typedef struct pqhsa_select {
     double fraction;
     int32_t topk;
     int32_t k_cap; /* row stride of topk_idx / topk_val; >= the largest k of the batch */
-    int32_t flags; /* 0, or PQHSA_SELECT_GENERAL_PATH | PQHSA_SELECT_ONE_LAUNCH */
+    int32_t flags; /* 0, or an OR of the PQHSA_SELECT_* flags below */
     int32_t n_mean; /* hint: mean number of indexed keys per sequence of the batch; 0 = unknown (n_max is
                        assumed).  Sizes the scan's tiles so that a ragged batch still fills the chip;
                        results do not depend on it. */
@@ -126,6 +126,14 @@ typedef struct pqhsa_select {
  * other shapes ignore the flag.  Off by default: on MI355X the three separate launches are
  * faster (the one launch saves two launch gaps and loses more to device-scope memory traffic). */
 #define PQHSA_SELECT_ONE_LAUNCH 2
+/* On the general path with a GQA group of 2 to 8 query rows (and at most 327 680 candidate slots
+ * per sequence), asks the exact attention to fetch a K/V row that several rows of the group
+ * selected ONCE per KV head: the selection records which rows selected each key and one of them
+ * fetches it for all.  Same results (to fp32 summation order).  Off by default: every query row
+ * fetches its own selected rows, as the stand-alone pqhsa_hybrid_attend_paged does; on MI355X
+ * that is faster at every measured shape, because rows of a group already meet in the L2 and the
+ * classification pass and the extra partial records cost more than the saved fetches. */
+#define PQHSA_SELECT_SHARE_ROWS 4
 
 const char *pqhsa_version(void);
 const char *pqhsa_last_error(void);

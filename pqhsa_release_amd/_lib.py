@@ -69,6 +69,7 @@ class Select(ctypes.Structure):
 
 SELECT_GENERAL_PATH = 1
 SELECT_ONE_LAUNCH = 2
+SELECT_SHARE_ROWS = 4
 
 
 class PqhsaError(RuntimeError):

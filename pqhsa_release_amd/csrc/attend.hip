@@ -20,6 +20,7 @@ PQHSA_TRACE_DECL(trace_attend)
 }
 #define PQHSA_ATTEND_MARK(wg, slot) PQHSA_TRACE_MARK(trace_attend, wg, slot)
 #include "attend_body.h"
+#include "attend_shared.h"
 
 namespace pqhsa {
 
@@ -41,6 +42,22 @@ __global__ __launch_bounds__(kAttThreads) void attend_partial_kernel(AttendArgs 
         split = blockIdx.x; g = blockIdx.y; bh = blockIdx.z;
     }
     attend_body<KDT, QDT, false>(a, split, g, bh, smem, blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z));
+}
+
+template <int KDT, int QDT, int SG>
+__global__ __launch_bounds__(kAttThreads, SG > 4 ? 2 : 3) void attend_shared_kernel(AttendArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    int split, g, bh;  // (the launch forms of attend_partial_kernel)
+    if (a.group_xcd) {
+        const int id = blockIdx.x, blk = id / (8 * a.G), in = id % (8 * a.G);
+        const int pair = blk * 8 + in % 8;
+        g = in / 8;
+        split = pair % a.splits;
+        bh = pair / a.splits;
+    } else {
+        split = blockIdx.x; g = blockIdx.y; bh = blockIdx.z;
+    }
+    attend_shared_body<KDT, QDT, SG>(a, split, g, bh, smem, blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z));
 }
 
 // Stand-alone form only: the caller's masses cover every indexed key of the row, so the
@@ -98,8 +115,12 @@ static int splits_room(int rows, int k_cap) { return pick_splits(rows, (k_cap > 
 // arrival flags (one word per split, 64 per query row) and one ticket counter per row
 size_t attend_arrive_bytes(int rows) { return (size_t)rows * (kMaxSplits + 1) * sizeof(uint32_t); }
 
-size_t attend_partials_bytes(int rows, int k_cap) {
-    return (size_t)rows * splits_room(rows, k_cap) * kPartWidth * sizeof(float);
+// (G > 0: room for the records of the form that shares K/V rows across a group of G query rows)
+size_t attend_partials_bytes(int rows, int k_cap, int G) {
+    const int GP = G > 0 ? padded_groups(G) : 0;
+    size_t width = kPartWidth;
+    if (G >= 2 && GP <= 8) width = (size_t)attend_shared_records(G <= 4 ? 4 : 8) * kRecWidth;
+    return (size_t)rows * splits_room(rows, k_cap) * width * sizeof(float);
 }
 
 int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max, bool mark, hipStream_t stream,
@@ -121,6 +142,36 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
     const size_t lds = attend_lds_bytes(chunk);
     a.group_xcd = even_rows && (BH * a.splits) % 8 == 0;
     dim3 grid = a.group_xcd ? dim3(a.splits * a.G * BH) : dim3(a.splits, a.G, BH);
+    if (a.share_map && a.G >= 2 && a.G <= 8) {  // every selected row fetched once per KV head
+        const int SG = a.G <= 4 ? 4 : 8;
+        const size_t lds_sh = SG == 4 ? attend_shared_lds_bytes<4>(chunk) : attend_shared_lds_bytes<8>(chunk);
+#define PQHSA_ATT_SH(KD, QD)                                                                                  \
+        {                                                                                                     \
+            const void *kern = SG == 4 ? reinterpret_cast<const void *>(attend_shared_kernel<KD, QD, 4>)      \
+                                       : reinterpret_cast<const void *>(attend_shared_kernel<KD, QD, 8>);     \
+            if (lds_sh > 32 * 1024) {                                                                         \
+                hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_sh); \
+                if (e != hipSuccess) {                                                                        \
+                    set_error("attend: cannot raise LDS limit: %s", hipGetErrorString(e));                    \
+                    return PQHSA_ELAUNCH;                                                                     \
+                }                                                                                             \
+            }                                                                                                 \
+            if (SG == 4) hipLaunchKernelGGL((attend_shared_kernel<KD, QD, 4>), grid, dim3(kAttThreads), lds_sh, stream, a); \
+            else hipLaunchKernelGGL((attend_shared_kernel<KD, QD, 8>), grid, dim3(kAttThreads), lds_sh, stream, a);        \
+        }
+        if (kv_dtype == PQHSA_BF16 && q_dtype == PQHSA_BF16) PQHSA_ATT_SH(PQHSA_BF16, PQHSA_BF16)
+        else if (kv_dtype == PQHSA_F32 && q_dtype == PQHSA_F32) PQHSA_ATT_SH(PQHSA_F32, PQHSA_F32)
+        else if (kv_dtype == PQHSA_F16 && q_dtype == PQHSA_F16) PQHSA_ATT_SH(PQHSA_F16, PQHSA_F16)
+        else if (kv_dtype == PQHSA_BF16 && q_dtype == PQHSA_F32) PQHSA_ATT_SH(PQHSA_BF16, PQHSA_F32)
+        else if (kv_dtype == PQHSA_F16 && q_dtype == PQHSA_F32) PQHSA_ATT_SH(PQHSA_F16, PQHSA_F32)
+        else {
+            set_error("attend: unsupported dtype pair (q %d, kv %d)", q_dtype, kv_dtype);
+            return PQHSA_EINVAL;
+        }
+#undef PQHSA_ATT_SH
+        if (mark) profile_mark(kProfKernels, stream);
+        return check_launch("attend_shared");
+    }
 #define PQHSA_ATT(KD, QD)                                                                              \
     {                                                                                                  \
         auto kern = attend_partial_kernel<KD, QD>;                                                     \
@@ -154,7 +205,8 @@ int attend_splits_room(int rows, int k_cap) { return splits_room(rows, k_cap); }
 AttendArgs decode_attend_args(const void *q, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                               const int32_t *seq_lens, int sink, const int32_t *topk_idx, const int32_t *topk_cnt,
                               int k_cap, const float *mass, const float *ref_val, float scale, float *partials,
-                              uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst) {
+                              uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
+                              const uint32_t *share_map, int64_t share_stride) {
     AttendArgs a = {};
     a.q = static_cast<const char *>(q); a.out = static_cast<char *>(out); a.kv = make_view(kv);
     a.H = index->kv_heads; a.G = G; a.seq_lens = seq_lens; a.n_idx = index->n_idx; a.sink = sink;
@@ -166,6 +218,7 @@ AttendArgs decode_attend_args(const void *q, void *out, const pqhsa_kv_view *kv,
     a.ref0 = ref_val; a.ref_stride = GP;
     a.vbar = index->vbar; a.L = index->num_lists;
     a.n_commit_src = n_commit_src; a.n_commit_dst = n_commit_dst;
+    a.share_map = share_map; a.share_stride = share_stride;
     return a;
 }
 
@@ -173,9 +226,10 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
                   float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
-                  bool even_rows, hipStream_t stream) {
+                  bool even_rows, const uint32_t *share_map, int64_t share_stride, hipStream_t stream) {
     const AttendArgs a = decode_attend_args(q, out, kv, index, G, GP, seq_lens, sink, topk_idx, topk_cnt, k_cap, mass,
-                                            ref_val, scale, partials, arrive, n_commit_src, n_commit_dst);
+                                            ref_val, scale, partials, arrive, n_commit_src, n_commit_dst, share_map,
+                                            share_stride);
     return launch_attend(a, q_dtype, kv->dtype, index->batch * index->kv_heads, rows_max, true, stream, even_rows);
 }
 
@@ -184,7 +238,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
 using namespace pqhsa;
 
 extern "C" size_t pqhsa_attend_workspace_bytes(int32_t B, int32_t H, int32_t G, int32_t num_lists) {
-    return attend_partials_bytes(B * H * G, 1 << 20) + (size_t)B * H * G * num_lists * sizeof(float) +
+    return attend_partials_bytes(B * H * G, 1 << 20, 0) + (size_t)B * H * G * num_lists * sizeof(float) +
            attend_arrive_bytes(B * H * G) + 1024;
 }
 
@@ -207,7 +261,7 @@ extern "C" int pqhsa_hybrid_attend_paged(const void *q, int32_t q_dtype, void *o
     if (BH == 0) return PQHSA_OK;
     char *w = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~(uintptr_t)255);
     float *partials = reinterpret_cast<float *>(w);
-    float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G, 1 << 20));
+    float *mass_adj = reinterpret_cast<float *>(w + attend_partials_bytes(BH * G, 1 << 20, 0));
     uint32_t *arrive = reinterpret_cast<uint32_t *>(
         (reinterpret_cast<uintptr_t>(mass_adj + (size_t)BH * G * L) + 255) & ~(uintptr_t)255);
     hipLaunchKernelGGL(subtract_selected_kernel, dim3(G, BH), dim3(kAttThreads), (size_t)L * sizeof(float), stream,

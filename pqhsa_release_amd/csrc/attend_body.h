@@ -45,6 +45,10 @@ struct AttendArgs {
     // after a fused append: the step's last kernel stores the new key counts into the index
     const int32_t *n_commit_src;  // [B] (NULL: nothing to store)
     int32_t *n_commit_dst;        // [B]
+    // the keys every query row selected, one bit per retrieval-local key index (NULL: every row fetches
+    // its own keys)
+    const uint32_t *share_map;    // [BH * G, share_stride] words
+    int64_t share_stride;
 };
 
 // One lane's 8 elements of a 128-element row as loaded (16 bytes for 2-byte types, 32 for fp32),

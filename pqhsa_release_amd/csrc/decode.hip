@@ -25,7 +25,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val,
                        void *pairs, uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
-                       const AppendFinish *append, hipStream_t stream);
+                       const AppendFinish *append, uint32_t *share_map, int64_t share_stride, hipStream_t stream);
 bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap);
 int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                  const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const pqhsa_select *select, float scale,
@@ -35,7 +35,7 @@ int decode_attend(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv
                   int GP, const int32_t *seq_lens, int sink, int rows_max, const int32_t *topk_idx,
                   const int32_t *topk_cnt, int k_cap, const float *mass, const float *ref_val, float scale,
                   float *partials, uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
-                  bool even_rows, hipStream_t stream);
+                  bool even_rows, const uint32_t *share_map, int64_t share_stride, hipStream_t stream);
 bool decode_fused_fits(int batch, int heads, int G, int64_t n_cap, int64_t n_max, int64_t n_mean, int L);
 int decode_fused(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                  const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const float *qnorm, const float *lut,
@@ -45,7 +45,7 @@ int decode_fused(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
                  uint32_t *arrive, uint32_t *sync_words, const AppendFinish *append, const int32_t *n_commit_src,
                  int32_t *n_commit_dst, hipStream_t stream);
 size_t decode_fused_sync_words(int streams);
-size_t attend_partials_bytes(int rows, int k_cap);
+size_t attend_partials_bytes(int rows, int k_cap, int G);
 size_t attend_arrive_bytes(int rows);
 
 static size_t al(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -67,6 +67,8 @@ struct Carve {
     float *partials;
     int32_t *n_after;  // [B] keys per sequence after this step's append
     unsigned long long *nearest;  // [BH, list blocks] nearest centroid to the appended key, per list block
+    uint32_t *share;              // [BH * G, share_stride] words: bitmap of the keys each query row selected
+    int64_t share_stride;
     size_t total;
 };
 
@@ -105,7 +107,11 @@ static Carve carve(char *base, int B, int H, int G, int64_t n_cap, int L, int k_
     c.topk_idx = reinterpret_cast<int32_t *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_val = reinterpret_cast<float *>(take(BH * G * (size_t)k_cap * 4));
     c.topk_cnt = reinterpret_cast<int32_t *>(take(BH * G * 4));
-    c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G), k_cap)));
+    c.partials = reinterpret_cast<float *>(take(attend_partials_bytes((int)(BH * G), k_cap, G)));
+    // one bit per stored key and query row: the keys the row selected (groups of 2 to 8 rows, as long as
+    // a row's bitmap fits the selection workgroup's LDS beside its tables)
+    c.share_stride = (G >= 2 && G <= 8 && n_cap <= 320 * 1024) ? (int64_t)((n_cap + 127) / 128 * 4) : 0;
+    c.share = reinterpret_cast<uint32_t *>(take(BH * G * (size_t)c.share_stride * 4));
     c.n_after = reinterpret_cast<int32_t *>(take((size_t)B * 4));
     c.nearest = reinterpret_cast<unsigned long long *>(take(BH * (size_t)lut_list_blocks(L) * 8));
     c.total = off;
@@ -215,16 +221,19 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
                             c.rescans, topk_idx, topk_val, topk_cnt, c.partials, c.arrive, c.sync,
                             append_count ? &ap : nullptr, append_count ? c.n_after : nullptr,
                             append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr, stream);
+    // (every selected K/V row is fetched once per KV head unless the caller asks for one fetch per query row)
+    uint32_t *share = (select->flags & PQHSA_SELECT_SHARE_ROWS) && c.share_stride != 0 ? c.share : nullptr;
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
                             c.k_row, c.ref_val, c.pairs, c.aux, c.emit_cap, c.mass, c.rescans,
-                            topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, stream);
+                            topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, share, c.share_stride, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials, c.arrive,
                          append_count ? c.n_after : nullptr,
                          append_count ? const_cast<int32_t *>(index_in->n_idx) : nullptr,
                          // rows of about one length (mean key count known and within an eighth of the longest)
-                         select->n_mean > 0 && (int64_t)select->n_mean * 8 >= (int64_t)n_max * 7, stream);
+                         select->n_mean > 0 && (int64_t)select->n_mean * 8 >= (int64_t)n_max * 7,
+                         share, c.share_stride, stream);
 }
 
 extern "C" int pqhsa_decode_step(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,

@@ -647,7 +647,8 @@ ScanArgs decode_scan_args(const pqhsa_index *index, int G, const float *qnorm, c
 AttendArgs decode_attend_args(const void *q, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                               const int32_t *seq_lens, int sink, const int32_t *topk_idx, const int32_t *topk_cnt,
                               int k_cap, const float *mass, const float *ref_val, float scale, float *partials,
-                              uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst);
+                              uint32_t *arrive, const int32_t *n_commit_src, int32_t *n_commit_dst,
+                              const uint32_t *share_map, int64_t share_stride);
 
 // threshold estimate, then scan + selection + attention in one launch (the caller has checked decode_fused_fits)
 int decode_fused(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
@@ -664,7 +665,7 @@ int decode_fused(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
     const ScanArgs sa = decode_scan_args(index, G, qnorm, lut, list_scores, scale, emit_count, thr_key, ref_val, pairs,
                                          nullptr, emit_cap, mass);
     const AttendArgs aa = decode_attend_args(q, out, kv, index, G, GP, seq_lens, sink, topk_idx, topk_cnt, select->k_cap,
-                                             mass, ref_val, scale, partials, arrive, n_commit_src, n_commit_dst);
+                                             mass, ref_val, scale, partials, arrive, n_commit_src, n_commit_dst, nullptr, 0);
     rc = launch_decode_fused(sa, aa, k_row, thr_key, thr_key + (size_t)streams * GP, ref_val, topk_idx, topk_val, topk_cnt,
                              select->k_cap, rescans, sync_words, decode_expected_candidates(index, n_max, select), GP,
                              streams, n_max, rows_max, q_dtype, kv->dtype, stream);

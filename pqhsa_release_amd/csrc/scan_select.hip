@@ -680,6 +680,9 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
         for (int l = tid; l < a.L; l += kSelThreads) mx[l] = 0.0f;
     for (int i = tid; i < kSelBins; i += kSelThreads) ss.hist[i] = 0u;
     if (tid == 0) ss.cont_count = 0u;
+    uint32_t *share_s = reinterpret_cast<uint32_t *>(ls_s + a.L);  // [share_stride] the row's winners, one bit per key
+    if (a.share_map)
+        for (int i = tid; i < (int)a.share_stride; i += kSelThreads) share_s[i] = 0u;
     __syncthreads();
     PQHSA_TRACE_MARK(trace_select, trace_wg, 1);
     SelectOut out;
@@ -688,6 +691,10 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
     out.k_cap = (uint32_t)a.k_cap;
     out.mx = mass_out ? mx : nullptr;
     out.ref1 = 0.0f;
+    if (a.share_map) {
+        out.share_bits = share_s;
+        out.share_len = (uint32_t)min((int64_t)a.share_stride * 32, a.n_cap);
+    }
     float ref1;
     bool done = false;
     if constexpr (RS > 0) {
@@ -718,6 +725,10 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
     }
     PQHSA_TRACE_MARK(trace_select, trace_wg, 5);
     __syncthreads();
+    if (a.share_map) {  // the row's bitmap of selected keys, whole (no clearing between steps)
+        uint32_t *dst = a.share_map + orow * a.share_stride;
+        for (int i = tid; i < (int)a.share_stride; i += kSelThreads) dst[i] = share_s[i];
+    }
     if (mass_out) {
         // The row's sums move to the k-th logit as their reference (it is at or above the scan's, so
         // the factor is at most 1); a row without usable sums from the scan starts from the losers alone.
@@ -854,7 +865,8 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
 int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     if (streams == 0) return PQHSA_OK;
     // list weights of the losers; the re-scan path parks a (128 + L)-float table there first
-    const size_t lds = (size_t)(kM * kCodes + 2 * a.L) * sizeof(float);
+    const size_t lds = (size_t)(kM * kCodes + 2 * a.L) * sizeof(float) + (a.share_map ? (size_t)a.share_stride * 4 : 0);
+    PQHSA_REQUIRE(lds <= 120 * 1024, "select_final: %zu bytes of LDS needed", lds);
     const dim3 grid(a.G, streams), block(kSelThreads);
     if (a.expected_candidates <= 0) hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
     else if (a.expected_candidates <= 8 * kSelThreads && (int64_t)a.G * streams > 256) {
@@ -1377,7 +1389,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
                        uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
-                       hipStream_t stream) {
+                       uint32_t *share_map, int64_t share_stride, hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
     // 1. threshold per row from the sampled keys
     int rc = decode_thresholds(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val, append, stream);
@@ -1399,6 +1411,7 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.codes = index->codes; s.list_ids = index->list_ids; s.norms = index->norms; s.pos = index->pos;
     s.n_cap = index->n_cap; s.qnorm = qnorm; s.lut = lut; s.list_scores = list_scores; s.scale = scale;
     s.rescans = rescans;
+    s.share_map = share_map; s.share_stride = share_stride;
     s.expected_candidates = decode_expected_candidates(index, n_max, select);
     rc = launch_select_final(s, streams, stream);
     profile_mark(kProfAttend, stream);

@@ -208,6 +208,10 @@ struct SelectArgs {
     float scale;
     uint32_t *rescans;     // [1] counter of rows that needed the full re-scan (diagnostics)
     int64_t expected_candidates;  // host's upper estimate of candidates per row (0: unknown)
+    // the keys each query row selected, as a bitmap over retrieval-local key indices (NULL: not kept):
+    // built in LDS by the row's workgroup and written out whole, so it needs no clearing
+    uint32_t *share_map;   // [rows (BH * G), share_stride] words
+    int64_t share_stride;  // words per row
 };
 
 // Exclusive prefix over the workgroup of a per-thread count (one barrier pair).
@@ -233,7 +237,10 @@ struct SelectOut {
     int32_t *lds_idx = nullptr;  // LDS copy of the selected indices, for a kernel that goes on to use them (room lds_cap)
     uint32_t lds_cap = 0u;
     bool dev = false;        // the outputs are read by other workgroups of the same launch: device-scope stores
+    uint32_t *share_bits = nullptr;  // LDS: one bit per retrieval-local key index, set for the row's winners (NULL: not kept)
+    uint32_t share_len = 0u;         // ... and the number of bits
     __device__ inline void winner(uint32_t at, uint32_t key, uint32_t where) const {
+        if (share_bits && at < k_cap && where < share_len) atomicOr(share_bits + (where >> 5), 1u << (where & 31u));
         if (at < k_cap) {
             if (dev) {
                 __hip_atomic_store(out_idx + at, (int32_t)where, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

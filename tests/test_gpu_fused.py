@@ -168,3 +168,81 @@ def test_fused_step_with_the_append_riding_on_it():
             assert torch.equal(torch.gather(lg, 2, tidx), tval), (t, b)
             assert torch.equal(tval.sort(dim=2, descending=True).values, torch.topk(lg, k, dim=2).values), (t, b)
         assert bool(torch.isfinite(out).all())
+
+
+# ---- K/V rows fetched once per KV head ------------------------------------------------------------
+def _steps(p, idx, kv, ws, q, fraction, **kw):
+    out = torch.full_like(q, float("nan"))
+    ws.topk_idx.fill_(-1)
+    ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=fraction,
+                    topk=0, scale=SCALE, workspace=ws, general_path=True, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("overlap", ["identical", "disjoint", "half"])
+@pytest.mark.parametrize("groups, dtype", [(4, torch.bfloat16), (2, torch.float32), (7, torch.float16)])
+def test_rows_of_a_group_that_select_identical_disjoint_and_half_overlapping_keys(overlap, groups, dtype):
+    """The attention that fetches a selected K/V row once per KV head, on groups whose query rows
+    select the same keys (every row is fetched for all rows by one owner), different keys (every
+    row fetches its own) or half of each other's: top-k sets are the oracle's, outputs within the
+    bound, and equal to the form in which every query row fetches its own rows."""
+    dev = _cuda()
+    p = Problem(lens=[9000, 9000], heads=2, groups=groups, lists=32, dtype=dtype, seed=501)
+    gen = torch.Generator().manual_seed(9)
+    for (b, h), q in p.queries.items():
+        keys = p.keys[b, h]
+        if overlap == "identical":      # the same query in every row of the group
+            q[:] = q[0]
+        elif overlap == "disjoint":     # needles far apart: unrelated keys
+            picks = torch.randperm(p.lens[b] - 200, generator=gen)[: p.G] + 100
+            q[:] = (keys[picks] + 0.05 * torch.randn(p.G, DIM, generator=gen)).to(dtype).float()
+        else:                           # pairs of rows around one needle each: about half of a pair's keys in common
+            picks = torch.randperm(p.lens[b] - 200, generator=gen)[: (p.G + 1) // 2] + 100
+            q[:] = (keys[picks].repeat_interleave(2, 0)[: p.G] + 0.25 * torch.randn(p.G, DIM, generator=gen)).to(dtype).float()
+    idx = p.device_index(dev)
+    kv = _kv(p, "5d" if dtype != torch.float32 else "dense")
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.04, 0))
+    q = p.q_tensor().float()
+    shared = _steps(p, idx, kv, ws, q, 0.04, share_rows=True)
+    tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+    own = _steps(p, idx, kv, ws, q, 0.04)
+    tol = 1e-4 if dtype == torch.float32 else 2e-3
+    o = shared.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    common = []
+    for (b, h) in p.index:
+        want_out, want_idx, _ = p.oracle_step(b, h, 0.04)
+        k = want_idx.shape[1]
+        for g in range(p.G):
+            assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (b, h, g)
+        assert float(np.abs(o[b, h] - want_out).max()) <= tol, (b, h)
+        union = len(set(np.concatenate([want_idx[g] for g in range(p.G)]).tolist()))
+        common.append(1.0 - union / (p.G * k))
+    assert float((shared - own).abs().max()) <= 2e-5
+    if overlap == "identical":
+        assert min(common) > 0.4 if p.G == 2 else min(common) > 0.7      # every key shared by all rows
+    elif overlap == "disjoint":
+        assert max(common) < 0.3
+
+
+def test_shared_fetch_over_many_rows_and_chunks():
+    """Many streams, the largest number of chunks per row the launch uses, rows that share most of their
+    keys: every output row must be folded exactly once (rows start as NaN), over repeated steps."""
+    dev = _cuda()
+    p = Problem(lens=[30000] * 3, heads=4, groups=4, lists=32, dtype=torch.bfloat16, seed=77)
+    for (b, h), q in p.queries.items():
+        q[2:] = q[:2]                    # two pairs of equal rows
+    idx = p.device_index(dev)
+    kv = _kv(p, "4d")
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.1, 0))   # about 3 000 rows per query: several chunks
+    q = p.q_tensor()
+    ref = _steps(p, idx, kv, ws, q, 0.1).float()
+    assert bool(torch.isfinite(ref).all())
+    for rep in range(40):
+        got = _steps(p, idx, kv, ws, q, 0.1, share_rows=True).float()
+        assert bool(torch.isfinite(got).all()), rep
+        assert float((got - ref).abs().max()) <= 2e-2, rep      # (bf16 outputs: one step of rounding)
+    o = got.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+    for (b, h) in list(p.index)[:3]:
+        want_out, _, _ = p.oracle_step(b, h, 0.1)
+        assert float(np.abs(o[b, h] - want_out).max()) <= 2e-3 + 2.0 ** -8 * float(np.abs(want_out).max()), (b, h)
