@@ -515,7 +515,8 @@ __global__ __launch_bounds__(kFusedThreads, GP >= 8 ? 3 : 4) void decode_fused_k
             else if (q == 1) __builtin_amdgcn_s_setprio(2);
             else if (q == 2) __builtin_amdgcn_s_setprio(1);
         }
-        scan_emit_body<GP, true>(f.scan, tile, bh, smem, blockIdx.x);
+        scan_emit_body<GP, true>(f.scan, tile, bh, reinterpret_cast<float *>(smem),
+                                          smem + kM * kCodes * GP * sizeof(float), blockIdx.x);
         PQHSA_TRACE_MARK(trace_fused, blockIdx.x, 2);
         signal_done(f.scan_done + (size_t)bh * kSyncStride);
         PQHSA_TRACE_MARK(trace_fused, blockIdx.x, 3);
@@ -564,6 +565,7 @@ int launch_decode_fused(const ScanArgs &scan_in, const AttendArgs &att_in, const
     // (one when the launch fills at most half the chip anyway)
     f.scan.stage_cap = emit_stage_cap(GP);
     f.scan.emit_aux = nullptr;
+    f.scan.packed_records = 1;  // (decode_fused_fits: positions and list ids fit the packed word)
     f.scan.tile_major = 0;
     const int64_t windows = (n_max + kWaveKeys - 1) / kWaveKeys;
     int64_t tiles = (env_int("PQHSA_FUSED_SCAN_WGS", 1024) + streams - 1) / streams;
@@ -596,7 +598,7 @@ int launch_decode_fused(const ScanArgs &scan_in, const AttendArgs &att_in, const
     f.sel_lag = max(1, env_int("PQHSA_FUSED_SEL_LAG", 1));
     f.att_lag = max(f.sel_lag + 1, env_int("PQHSA_FUSED_ATT_LAG", 2));
     const int steps = f.groups + f.att_lag;
-    const size_t lds_scan = scan_emit_lds_bytes(GP, f.scan.L, f.scan.stage_cap, false);
+    const size_t lds_scan = (size_t)kM * kCodes * GP * sizeof(float) + scan_emit_lds_bytes(GP, f.scan.L, f.scan.stage_cap, false);
     const size_t lds_sel = sizeof(SelectLds) + (size_t)(2 * f.scan.L + kM * kCodes) * sizeof(float);
     const size_t lds_att = attend_lds_bytes(chunk);
     size_t lds = lds_scan > lds_sel ? lds_scan : lds_sel;

@@ -53,6 +53,7 @@ struct ScanArgs {
     int tile_windows;         // the decode step's scan: 256-key windows per workgroup
     int tile_major;           // ... and the launch form: 0 grid (tiles, streams), 1 grid (streams, tiles), 2 packed
     int seqs;                 // ... and the number of sequences (streams / n_div), for the packed form
+    int packed_records;       // candidate records hold (logit bits, stored position | list id << 20): emit_aux and pos unused
 };
 
 template <int GP>
@@ -85,6 +86,22 @@ __device__ inline void lut_entry(const float *lut_s, uint32_t entry, float (&v)[
         }
     } else {
         v[0] = lut_s[entry];
+    }
+}
+
+// The same entry addressed by subspace m and the code's byte offset into the subspace (code x 8 for
+// the pair sub-tables, so that m and the pair index end up in the instruction's immediate offset).
+template <int GP>
+__device__ inline void lut_entry_at(const float *lut_s, int m, uint32_t code_x8, float (&v)[GP]) {
+    if constexpr (GP >= 2) {
+        const char *b = reinterpret_cast<const char *>(lut_s) + code_x8;
+#pragma unroll
+        for (int p = 0; p < GP / 2; ++p) {
+            const float2 t = *reinterpret_cast<const float2 *>(b + (size_t)(p * (kM * kCodes) + m * kCodes) * sizeof(float2));
+            v[2 * p] = t.x; v[2 * p + 1] = t.y;
+        }
+    } else {
+        v[0] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut_s) + (code_x8 >> 1) + (size_t)m * kCodes * sizeof(float));
     }
 }
 

@@ -28,8 +28,9 @@ PQHSA_TRACE_DECL(trace_scan)
 namespace pqhsa {
 
 template <int GP>
-__global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
+__global__ __launch_bounds__(kScanThreads, GP <= 4 ? 4 : GP == 8 ? 3 : 2) void scan_emit_kernel(ScanArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ __align__(16) float lut_s[kM * kCodes * GP];  // the PQ table, as pair sub-tables (lut_entry)
     // Which tile of which stream this workgroup takes.  An even batch is launched as a grid of
     // (tiles, streams).  A ragged batch is launched PACKED: one row of workgroups covers the tiles
     // that hold work, sequence after sequence (within a sequence tile-major, so that its streams
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_emit_kernel(ScanArgs a) {
         tile = blockIdx.x;
         bh = blockIdx.y;
     }
-    scan_emit_body<GP, false>(a, tile, bh, smem, blockIdx.x + (size_t)gridDim.x * blockIdx.y);
+    scan_emit_body<GP, false>(a, tile, bh, lut_s, smem, blockIdx.x + (size_t)gridDim.x * blockIdx.y);
 }
 
 // a packed launch walks the sequences' key counts in every workgroup: only for batches this small
@@ -94,14 +95,15 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
     a.tile_windows = (int)((windows_mean + tiles - 1) / tiles);
     tiles = (windows + a.tile_windows - 1) / a.tile_windows;
     const size_t lds = scan_emit_lds_bytes(GP, a.L, a.stage_cap, a.emit_aux != nullptr);
-    PQHSA_REQUIRE(lds <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);
+    PQHSA_REQUIRE(lds + (size_t)kM * kCodes * GP * sizeof(float) <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);
+    PQHSA_REQUIRE(!a.packed_records || (a.n_cap <= (int64_t)kPackedPosMask + 1 && a.L <= 4096),
+                  "scan_emit: packed candidate records hold 20 bits of position and 12 bits of list id");
     a.tile_major = packed ? 2 : ragged ? 1 : 0;
     a.seqs = seqs;
     dim3 grid = packed ? dim3((unsigned)(tiles * streams))
                        : ragged ? dim3(streams, (unsigned)tiles) : dim3((unsigned)tiles, streams);
-#define PQHSA_EMIT_CASE(gp)                                                                                 \
-    case gp: {                                                                                              \
-        auto kern = scan_emit_kernel<gp>;                                                                   \
+#define PQHSA_EMIT_KERNEL(kern)                                                                             \
+    {                                                                                                       \
         if (lds > 48 * 1024) {                                                                              \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                        \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);       \
@@ -111,7 +113,11 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
             }                                                                                               \
         }                                                                                                   \
         hipLaunchKernelGGL(kern, grid, dim3(kScanThreads), lds, stream, a);                                 \
-    } break;
+    }
+#define PQHSA_EMIT_CASE(gp)                                                                                 \
+    case gp:                                                                                                \
+        PQHSA_EMIT_KERNEL(scan_emit_kernel<gp>)                                                             \
+        break;
     switch (GP) {
         PQHSA_EMIT_CASE(1)
         PQHSA_EMIT_CASE(2)
@@ -122,6 +128,7 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
             set_error("scan_emit: unsupported padded group size %d", GP);
             return PQHSA_EINVAL;
     }
+#undef PQHSA_EMIT_KERNEL
 #undef PQHSA_EMIT_CASE
     return check_launch("scan_emit");
 }

@@ -12,23 +12,37 @@ namespace pqhsa {
 #define PQHSA_SCAN_MARK(wg, slot) do {} while (0)
 #endif
 
-// The work of one scan workgroup on tile `tile` of stream `bh`.  PACKED: candidate records hold the
-// key's stored position and list id in one word (pack_candidate) and leave with device-scope stores,
-// for readers in the same launch; the position map is not read.  `smem`: scan_emit_lds_bytes().
-template <int GP, bool PACKED>
-__device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const int bh, unsigned char *smem,
+// The eight table look-ups of one key need eight LDS byte offsets, code nibble x 8 bytes each.  Two
+// masked copies of the code word hold them as bytes (even nibbles in one, odd nibbles in the other),
+// so every offset is one byte extract.  (The empty asm keeps the compiler from folding the extract
+// back into a shift and a mask of the code word, one instruction more per look-up.)
+__device__ inline void nibble_offsets(uint32_t code, uint32_t &even, uint32_t &odd) {
+    even = (code << 3) & 0x78787878u;
+    odd = (code >> 1) & 0x78787878u;
+    asm volatile("" : "+v"(even), "+v"(odd));
+}
+
+// The work of one scan workgroup on tile `tile` of stream `bh`.  A candidate record holds the logit's
+// bit pattern and the key's retrieval-local index (read from the position map with the keys), with
+// the list id in a second array.  With a.packed_records it holds the key's STORED position and
+// its list id in one word instead (pack_candidate) and the position map is not read: the selection
+// looks up the candidates' indices.  DEV: records leave with device-scope stores, for readers in the
+// same launch.
+// `lut_s`: LDS for the PQ table, kM * kCodes * GP floats (a workgroup-static array, so that the
+// look-ups' table offsets are instruction immediates); `smem`: scan_emit_lds_bytes() of dynamic LDS.
+template <int GP, bool DEV>
+__device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const int bh, float *lut_s, unsigned char *smem,
                                       [[maybe_unused]] const size_t trace_wg) {
     constexpr int TH = kScanThreads;
     constexpr int kWaves = kScanWaves;
+    const bool packed = a.packed_records != 0;  // (uniform)
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int L = a.L;
     PQHSA_SCAN_MARK(trace_wg, 0);
 
-    // ---- LDS carve-up: PQ table (static), list scores, per-list sums, staging -------------------
-    float *lut_s = reinterpret_cast<float *>(smem);  // [128 entries][GP], as pair sub-tables (lut_entry)
-    smem += kM * kCodes * GP * sizeof(float);
+    // ---- LDS carve-up: list scores, per-list sums, staging ---------------------------------------
     float *ls_s = reinterpret_cast<float *>(smem);
     const size_t table_bytes = ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;
     unsigned char *after = smem + table_bytes;
@@ -37,6 +51,8 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
     uint32_t *wcnt_s = reinterpret_cast<uint32_t *>(after + mass_bytes);   // [waves][GP]
     uint32_t *base_s = wcnt_s + kWaves * 16;                           // [waves][GP]
     uint2 *stage_s = reinterpret_cast<uint2 *>(base_s + kWaves * 16);  // [waves][GP][stage_cap]
+    uint32_t *stage32 = reinterpret_cast<uint32_t *>(stage_s);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int cap_w = a.stage_cap;
     [[maybe_unused]] uint16_t *stage_aux = reinterpret_cast<uint16_t *>(stage_s + (size_t)kWaves * GP * cap_w);
 
@@ -57,8 +73,7 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
             k.cw = *reinterpret_cast<const uint4 *>(a.codes + base + i);
             k.lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + i);
             k.nw = *reinterpret_cast<const float4 *>(a.norms + base + i);
-            if constexpr (!PACKED)
-                if (a.pos) k.pw = *reinterpret_cast<const int4 *>(a.pos + base + i);
+            if (a.pos && !packed) k.pw = *reinterpret_cast<const int4 *>(a.pos + base + i);
         }
         return k;
     };
@@ -154,8 +169,6 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
         const uint2 lw = cur.lw;
         const float4 nw = cur.nw;
         const int4 pw = cur.pw;
-        // what a candidate record says of the key: its retrieval-local index, or (PACKED) its stored position
-        const uint32_t ridx[kKeysPerThread] = {(uint32_t)pw.x, (uint32_t)pw.y, (uint32_t)pw.z, (uint32_t)pw.w};
         if (next < nwin) cur = fetch(next);  // the wave's next window travels while this one is scored
         {
             const uint32_t c[4] = {cw.x, cw.y, cw.z, cw.w};
@@ -169,6 +182,9 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
             constexpr int KB = GP <= 2 ? 4 : (GP == 4 ? 2 : 1);
 #pragma unroll
             for (int j0 = 0; j0 < 4; j0 += KB) {
+                uint32_t even[KB], odd[KB];
+#pragma unroll
+                for (int j = 0; j < KB; ++j) nibble_offsets(c[j0 + j], even[j], odd[j]);
                 // the sum starts from the first entry: table entries are fma chains from +0 and never
                 // -0, so 0 + entry (the oracle's first step) is the entry itself
 #pragma unroll
@@ -176,7 +192,8 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
 #pragma unroll
                     for (int j = j0; j < j0 + KB; ++j) {
                         float v[GP];
-                        lut_entry<GP>(lut_s, m * kCodes + ((c[j] >> (4 * m)) & 15u), v);
+                        const uint32_t off8 = (((m & 1) ? odd[j - j0] : even[j - j0]) >> (8 * (m >> 1))) & 0xffu;
+                        lut_entry_at<GP>(lut_s, m, off8, v);
 #pragma unroll
                         for (int g = 0; g < GP; ++g) s[j][g] = m == 0 ? v[g] : s[j][g] + v[g];
                     }
@@ -201,95 +218,68 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
                 for (int g = 0; g < GP; ++g) s[j][g] = -INFINITY;
             }
         }
-        // The comparisons stay lane masks in scalar registers: whether the wave has any candidate is
-        // their union, and the per-lane bit sets are only built for the few windows that have one.
-        bool cand[4][GP];
+        // what a candidate record says of the key beside its logit
+        uint32_t word[kKeysPerThread];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = (uint32_t)(j == 0 ? pw.x : j == 1 ? pw.y : j == 2 ? pw.z : pw.w);  // (the stored position when no map was read)
+            word[j] = packed ? pack_candidate(w, lid[j]) : w;
+        }
+        // Row by row.  The comparisons stay lane masks in scalar registers, and everything about the
+        // candidates' slots is scalar arithmetic on those masks (their bit counts) but the rank of a
+        // lane inside its mask.  Slots go to key 0 of every lane first, then key 1, ...; within one, by lane.
         float e[4][GP];
-        unsigned long long any = 0ull;
 #pragma unroll
         for (int g = 0; g < GP; ++g) {
+            bool cand[4];
+            unsigned long long cm[4];
+            uint32_t tot = 0u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                cand[j][g] = s[j][g] >= thr_f[g];
-                any |= __ballot(cand[j][g]);
-                e[j][g] = cand[j][g] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
+                cand[j] = s[j][g] >= thr_f[g];
+                cm[j] = __ballot(cand[j]);
+                tot += (uint32_t)__popcll(cm[j]);
+                e[j][g] = cand[j] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
             }
-        }
-        if (any != 0ull) {  // wave-uniform
-            uint32_t emit_mask[GP];  // bit j set: key j of this lane is a candidate of row g
-#pragma unroll
-            for (int g = 0; g < GP; ++g) {
-                emit_mask[g] = 0u;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (cand[j][g]) emit_mask[g] |= 1u << j;
-            }
-            // slot of every candidate inside its wave, per row: prefix sums of the lanes' counts,
-            // two rows to a 32-bit word
-            uint32_t excl[GP], tot[GP];
-#pragma unroll
-            for (int g2 = 0; g2 < GP; g2 += 2) {
-                uint32_t packed = __popc(emit_mask[g2]);
-                if constexpr (GP > 1) packed |= (uint32_t)__popc(emit_mask[g2 + 1 < GP ? g2 + 1 : g2]) << 16;
-                const uint32_t incl = wave_prefix_u32(packed);
-                const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
-                const uint32_t ex = incl - packed;
-                excl[g2] = ex & 0xffffu;
-                tot[g2] = total & 0xffffu;
-                if (g2 + 1 < GP) {
-                    excl[g2 + 1 < GP ? g2 + 1 : g2] = ex >> 16;
-                    tot[g2 + 1 < GP ? g2 + 1 : g2] = total >> 16;
-                }
-            }
+            if (tot == 0u) continue;  // wave-uniform
             // A window whose candidates do not fit the row's staging area (a list close to the
-            // query: most of its keys are candidates) writes them straight to memory.  Lane g
-            // reserves the space of row g, so all rows share one round trip to memory.
-            uint32_t direct = 0u, want_res = 0u;
-#pragma unroll
-            for (int g = 0; g < GP; ++g) {
-                if (tot[g] != 0u && wcnt[g] + tot[g] > (uint32_t)cap_w) {
-                    direct |= 1u << g;
-                    if (lane == g) want_res = tot[g];
-                }
+            // query: most of its keys are candidates) reserves room in memory and writes them there.
+            const bool to_memory = wcnt[g] + tot > (uint32_t)cap_w;
+            uint32_t first = wcnt[g];
+            if (to_memory) {
+                uint32_t at = 0u;
+                if (lane == 0) at = atomicAdd(&a.emit_count[(size_t)bh * GP + g], tot);
+                first = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
+            } else {
+                wcnt[g] += tot;
             }
-            uint32_t at = 0u;
-            if (direct != 0u && want_res != 0u) at = atomicAdd(&a.emit_count[(size_t)bh * GP + lane], want_res);
+            const size_t o = ((size_t)bh * GP + g) * a.emit_cap;
+            const uint32_t srow = ((uint32_t)wave_u * GP + g) * (uint32_t)cap_w;  // (scalar)
 #pragma unroll
-            for (int g = 0; g < GP; ++g) {
-                if (tot[g] == 0u) continue;  // wave-uniform
-                if ((direct >> g) & 1u) {
-                    const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)at, g);
-                    uint32_t slot = first + excl[g];
-                    const size_t o = ((size_t)bh * GP + g) * a.emit_cap;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (!((emit_mask[g] >> j) & 1u)) continue;
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t cnt_j = (uint32_t)__popcll(cm[j]);
+                if (cnt_j == 0u) continue;  // wave-uniform
+                if (cand[j]) {
+                    // rank of the lane among the candidates of key j; the scalar part of the slot joins in the address
+                    const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(cm[j] >> 32),
+                                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)cm[j], 0u));
+                    const uint32_t slot = first + rank;
+                    const uint2 rec = make_uint2(__float_as_uint(s[j][g]), word[j]);
+                    if (to_memory) {
                         if (slot < (uint32_t)a.emit_cap) {  // a row past its room is settled by the selection's full pass
-                            if constexpr (PACKED) {
-                                store_dev(a.emit_pairs + o + slot, make_uint2(__float_as_uint(s[j][g]), pack_candidate(ridx[j], lid[j])));
-                            } else {
-                                a.emit_pairs[o + slot] = make_uint2(__float_as_uint(s[j][g]), ridx[j]);
-                                if (a.emit_aux) a.emit_aux[o + slot] = (uint16_t)lid[j];
-                            }
+                            if constexpr (DEV) store_dev(a.emit_pairs + o + slot, rec);
+                            else a.emit_pairs[o + slot] = rec;
+                            if (a.emit_aux) a.emit_aux[o + slot] = (uint16_t)lid[j];
                         }
-                        ++slot;
-                    }
-                } else {
-                    const size_t srow = ((size_t)wave * GP + g) * cap_w;
-                    uint32_t slot = wcnt[g] + excl[g];
-                    wcnt[g] += tot[g];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (!((emit_mask[g] >> j) & 1u)) continue;
-                        if constexpr (PACKED) {
-                            stage_s[srow + slot] = make_uint2(__float_as_uint(s[j][g]), pack_candidate(ridx[j], lid[j]));
-                        } else {
-                            stage_s[srow + slot] = make_uint2(__float_as_uint(s[j][g]), ridx[j]);
-                            if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
-                        }
-                        ++slot;
+                    } else {
+                        // (two 4-byte stores: one LDS instruction that takes the halves from any two registers)
+                        uint32_t *st = stage32 + 2u * (srow + first) + 2u * rank;
+                        st[0] = rec.x;
+                        st[1] = rec.y;
+                        if (a.emit_aux) stage_aux[srow + slot] = (uint16_t)lid[j];
                     }
                 }
+                first += cnt_j;
             }
         }
         // ---- background: weights summed per list ----------------------------------------------
@@ -309,19 +299,18 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
                 v[g] = simple ? (e[0][g] + e[1][g]) + (e[2][g] + e[3][g]) : 0.0f;
                 pre[g] = wave_prefix_f32(v[g]);
             }
-            if (is_start || is_end) {
+            if (is_start || is_end) {  // (a zero is added like anything else: no test per sum)
 #pragma unroll
                 for (int g = 0; g < GP; ++g) {
                     const float add = is_start ? (is_end ? v[g] : v[g] - pre[g]) : pre[g];
-                    if (add != 0.0f) atomicAdd(&mass_s[lid[0] * GP + g], add);
+                    atomicAdd(&mass_s[lid[0] * GP + g], add);
                 }
             }
             if (!simple) {  // a lane whose four keys straddle lists adds them one by one
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
 #pragma unroll
-                    for (int g = 0; g < GP; ++g)
-                        if (e[j][g] != 0.0f) atomicAdd(&mass_s[lid[j] * GP + g], e[j][g]);
+                    for (int g = 0; g < GP; ++g) atomicAdd(&mass_s[lid[j] * GP + g], e[j][g]);
                 }
             }
         }
@@ -366,12 +355,10 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
         const size_t srow = ((size_t)wave * GP + g) * cap_w;
         for (uint32_t i = lane; i < c; i += kWave) {
             if (first + i >= (uint32_t)a.emit_cap) break;
-            if constexpr (PACKED) {
-                store_dev(a.emit_pairs + o + first + i, stage_s[srow + i]);
-            } else {
-                a.emit_pairs[o + first + i] = stage_s[srow + i];
-                if (a.emit_aux) a.emit_aux[o + first + i] = stage_aux[srow + i];
-            }
+            const uint2 rec = stage_s[srow + i];
+            if constexpr (DEV) store_dev(a.emit_pairs + o + first + i, rec);
+            else a.emit_pairs[o + first + i] = rec;
+            if (a.emit_aux) a.emit_aux[o + first + i] = stage_aux[srow + i];
         }
     }
     PQHSA_SCAN_MARK(trace_wg, 3);
@@ -385,10 +372,10 @@ inline int emit_stage_cap(int GP) {
     return cap < 32 ? 32 : cap;
 }
 
-// dynamic LDS of scan_emit_body: PQ table, list scores, per-list sums, counters, staging
+// dynamic LDS of scan_emit_body: list scores, per-list sums, counters, staging (the PQ table is apart)
 inline size_t scan_emit_lds_bytes(int GP, int L, int stage_cap, bool aux) {
     const size_t tbl = ((size_t)L * GP * sizeof(float) + 15) & ~(size_t)15;
-    size_t lds = (size_t)kM * kCodes * GP * sizeof(float) + 2 * tbl + 2 * kScanWaves * 16 * sizeof(uint32_t) +
+    size_t lds = 2 * tbl + 2 * kScanWaves * 16 * sizeof(uint32_t) +
                  (size_t)kScanWaves * GP * stage_cap * sizeof(uint2);
     if (aux) lds += (size_t)kScanWaves * GP * stage_cap * sizeof(uint16_t);
     return lds;

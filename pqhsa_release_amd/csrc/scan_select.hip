@@ -641,27 +641,34 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
     const int k = a.k_row[row];
     uint2 *pairs = a.pairs + row * a.emit_cap;
     uint16_t *aux = a.aux ? a.aux + row * a.emit_cap : nullptr;
+    const MemRecords recs = {pairs, aux, a.raw_keys, a.packed, a.pos ? a.pos + (size_t)bh * a.n_cap : nullptr,
+                             (uint32_t)a.n_cap, (uint32_t)a.L};
     constexpr int RA = RS > 0 ? RS : 1;
     uint32_t skey[RA], swhere[RA], slist[RA];
-    if constexpr (RS > 0) {
+    uint32_t cnt;
+    uint2 pr[RA];
+    if constexpr (RS > 0) {  // (slots past the row's room read its last slot; they are masked by the count below)
 #pragma unroll
-        for (int r = 0; r < RS; ++r) {
-            const int64_t p = (int64_t)r * kSelThreads + tid;
-            const bool ok = p < a.emit_cap;
-            const uint2 pr = ok ? pairs[p] : make_uint2(0u, 0u);
-            skey[r] = record_key(pr.x, a.raw_keys);
-            swhere[r] = pr.y;
-            slist[r] = (aux && ok) ? aux[p] : 0u;
-        }
+        for (int r = 0; r < RS; ++r) pr[r] = pairs[min((int64_t)r * kSelThreads + tid, a.emit_cap - 1)];
     }
-    uint32_t cnt = a.emit_count[row];
-    const uint32_t lo_hint = a.thr_key ? a.thr_key[row] : 0u;
-    const uint32_t hi_hint = a.hi_key ? a.hi_key[row] : 0u;
+    cnt = a.emit_count[row];
     // losers' weights join the scan's per-list sums of the row (same reference), unless those have to start over
     float *mass_out = a.mass ? a.mass + (size_t)bh * a.L * a.GP + g : nullptr;
-    const float ref0 = mass_out ? a.ref_val[row] : -INFINITY;
-    // (the scan's sum of this thread's first list is requested now and merged at the end: no round trip then)
-    const float scan_mass = (mass_out && tid < a.L) ? mass_out[(size_t)tid * a.GP] : 0.0f;
+    uint32_t lo_hint, hi_hint;
+    float ref0, scan_mass;
+    if constexpr (RS > 0) {  // (these forms are launched with hints and sums: plain loads, all in flight together)
+        lo_hint = a.thr_key[row];
+        hi_hint = a.hi_key[row];
+        ref0 = a.ref_val[row];
+        scan_mass = mass_out[(size_t)min(tid, a.L - 1) * a.GP];
+        __builtin_amdgcn_sched_barrier(0);
+    } else {
+        lo_hint = a.thr_key ? a.thr_key[row] : 0u;
+        hi_hint = a.hi_key ? a.hi_key[row] : 0u;
+        ref0 = mass_out ? a.ref_val[row] : -INFINITY;
+        // (the scan's sum of this thread's first list is requested now and merged at the end: no round trip then)
+        scan_mass = (mass_out && tid < a.L) ? mass_out[(size_t)tid * a.GP] : 0.0f;
+    }
     // The estimate kept too few keys, or more than the candidate area holds: every stored key of
     // the row becomes a candidate, scored again on each pass of the selection, and the row's
     // background sums start over, relative to the k-th logit.
@@ -683,6 +690,21 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
     uint32_t *share_s = reinterpret_cast<uint32_t *>(ls_s + a.L);  // [share_stride] the row's winners, one bit per key
     if (a.share_map)
         for (int i = tid; i < (int)a.share_stride; i += kSelThreads) share_s[i] = 0u;
+    if constexpr (RS > 0) {
+        // Packed records (the launcher sends other records to the RS = 0 form).  The look-ups of the
+        // retrieval-local indices are the last loads requested, so that nothing else queues behind
+        // them; they travel while the keys are sorted out.  (Slots past the count look up slot 0.)
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            skey[r] = record_key(pr[r].x, a.raw_keys);
+            swhere[r] = (uint32_t)r * kSelThreads + tid < cnt ? min(pr[r].y & kPackedPosMask, recs.pos_n - 1u) : 0u;
+            slist[r] = min(pr[r].y >> kPackedPosBits, recs.L - 1u);
+        }
+        if (recs.pos) {  // (uniform)
+#pragma unroll
+            for (int r = 0; r < RS; ++r) swhere[r] = (uint32_t)recs.pos[swhere[r]];
+        }
+    }
     __syncthreads();
     PQHSA_TRACE_MARK(trace_select, trace_wg, 1);
     SelectOut out;
@@ -701,7 +723,7 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
         if (!rescan && cnt <= (uint32_t)RS * kSelThreads) {
 #pragma unroll
             for (int r = 0; r < RS; ++r) {
-                if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, swhere[r] = 0u, slist[r] = 0u;
+                if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, slist[r] = 0u;  // (their index is that of slot 0: unused)
             }
             select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1, lo_hint, hi_hint);
             done = true;
@@ -716,12 +738,12 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
         bool in_regs = false;
         if constexpr (RS == 0) {  // no estimate: pick the register variant from the count
             in_regs = cnt <= 16u * kSelThreads;
-            if (cnt <= 4u * kSelThreads) select_regs<4>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else if (cnt <= 8u * kSelThreads) select_regs<8>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
-            else if (in_regs) select_regs<16>(a.raw_keys, cnt, k, pairs, aux, out, red, wsum, &ss, &ref1);
+            if (cnt <= 4u * kSelThreads) select_regs<4>(recs, cnt, k, out, red, wsum, &ss, &ref1);
+            else if (cnt <= 8u * kSelThreads) select_regs<8>(recs, cnt, k, out, red, wsum, &ss, &ref1);
+            else if (in_regs) select_regs<16>(recs, cnt, k, out, red, wsum, &ss, &ref1);
         }
         // more candidates than the register variants hold (rare): stream them from memory
-        if (!in_regs) select_stream(MemRecords{pairs, aux, a.raw_keys}, cnt, k, out, red, wsum, &ss, &ref1);
+        if (!in_regs) select_stream(recs, cnt, k, out, red, wsum, &ss, &ref1);
     }
     PQHSA_TRACE_MARK(trace_select, trace_wg, 5);
     __syncthreads();
@@ -868,7 +890,9 @@ int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
     const size_t lds = (size_t)(kM * kCodes + 2 * a.L) * sizeof(float) + (a.share_map ? (size_t)a.share_stride * 4 : 0);
     PQHSA_REQUIRE(lds <= 120 * 1024, "select_final: %zu bytes of LDS needed", lds);
     const dim3 grid(a.G, streams), block(kSelThreads);
-    if (a.expected_candidates <= 0) hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
+    // (the forms that request the candidates before they know the count read packed records only)
+    if (a.expected_candidates <= 0 || !a.packed || !a.thr_key || !a.hi_key || !a.mass)
+        hipLaunchKernelGGL(select_final_kernel<0>, grid, block, lds, stream, a);
     else if (a.expected_candidates <= 8 * kSelThreads && (int64_t)a.G * streams > 256) {
         if (a.expected_candidates <= 4 * kSelThreads) hipLaunchKernelGGL((select_final_kernel<4, true>), grid, block, lds, stream, a);
         else hipLaunchKernelGGL((select_final_kernel<8, true>), grid, block, lds, stream, a);
@@ -1368,6 +1392,10 @@ int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnor
     return launch_sample_thresh(sa, streams, stream);
 }
 
+bool decode_packs_records(const pqhsa_index *index) {
+    return index->n_cap <= (int64_t)kPackedPosMask + 1 && index->num_lists <= 4096;
+}
+
 // the arguments of the decode step's scan (launch shape aside)
 ScanArgs decode_scan_args(const pqhsa_index *index, int G, const float *qnorm, const float *lut, const float *list_scores,
                           float scale, uint32_t *emit_count, uint32_t *thr_key, float *ref_val, void *pairs, uint16_t *aux,
@@ -1380,6 +1408,10 @@ ScanArgs decode_scan_args(const pqhsa_index *index, int G, const float *qnorm, c
     a.thr_key = thr_key; a.ref_val = ref_val; a.emit_count = emit_count;
     a.emit_pairs = static_cast<uint2 *>(pairs); a.emit_aux = aux; a.emit_cap = emit_cap;
     a.mass = mass;
+    // candidate records name the key by stored position (and list) in one word when both fit: the
+    // scan then leaves the position map alone and the selection looks up the candidates' indices
+    a.packed_records = decode_packs_records(index);
+    if (a.packed_records) a.emit_aux = nullptr;
     return a;
 }
 
@@ -1404,7 +1436,8 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     profile_mark(kProfSelect, stream);
     // 3. exact selection among the candidates
     SelectArgs s = {};
-    s.pairs = static_cast<uint2 *>(pairs); s.raw_keys = 1; s.aux = aux; s.emit_cap = emit_cap; s.emit_count = emit_count;
+    s.pairs = static_cast<uint2 *>(pairs); s.raw_keys = 1; s.aux = a.packed_records ? nullptr : aux; s.packed = a.packed_records;
+    s.emit_cap = emit_cap; s.emit_count = emit_count;
     s.k_row = k_row; s.thr_key = thr_key; s.hi_key = hi_key; s.n_arr = index->n_idx; s.rows_per_n = index->kv_heads * GP; s.GP = GP; s.G = G;
     s.topk_idx = topk_idx; s.topk_val = topk_val; s.topk_cnt = topk_cnt; s.k_cap = select->k_cap;
     s.mass = mass; s.ref_val = ref_val; s.L = index->num_lists;

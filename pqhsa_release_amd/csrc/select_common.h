@@ -178,6 +178,7 @@ struct SelectArgs {
     uint2 *pairs;          // [rows, emit_cap] (key, retrieval-local index)
     int raw_keys;          // the pairs hold logit bit patterns, not order-preserving keys (the decode step's scan writes those)
     uint16_t *aux;         // [rows, emit_cap] list ids (NULL: none)
+    int packed;            // the second word of a pair is pack_candidate(stored position, list id): `pos` translates it, no aux
     int64_t emit_cap;
     uint32_t *emit_count;  // [rows]
     const int32_t *k_row;  // [rows]
@@ -440,18 +441,87 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
 // order-preserving key of a candidate record: the record holds it, or the logit's bit pattern
 __device__ inline uint32_t record_key(uint32_t x, int raw) { return raw ? order_key(__uint_as_float(x)) : x; }
 
+// One candidate as the streaming selection sees it.
+struct CandRec {
+    uint32_t key, where, list;
+};
+
+// A packed candidate record: the logit's bit pattern and one word that holds the key's STORED
+// position (low 20 bits) and its list id (high 12 bits).  The retrieval-local index, which the tie
+// rule and the output are defined on, is looked up in the stream's position map.
+constexpr int kPackedPosBits = 20;
+constexpr uint32_t kPackedPosMask = (1u << kPackedPosBits) - 1u;
+__device__ inline uint32_t pack_candidate(uint32_t stored, uint32_t list) { return stored | (list << kPackedPosBits); }
+__device__ inline uint2 load_dev(const uint2 *p) {
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+    return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
+}
+__device__ inline void store_dev(uint2 *p, uint2 v) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), (unsigned long long)v.x | ((unsigned long long)v.y << 32),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// candidates in memory: (key or logit bits, second word) pairs; the second word is the key's
+// retrieval-local index, with list ids in `aux`, or (packed) a pack_candidate word
+struct MemRecords {
+    const uint2 *pairs;
+    const uint16_t *aux;
+    int raw;
+    int packed;
+    const int32_t *pos;  // packed: the stream's position map (NULL: a stored position is the index)
+    uint32_t pos_n, L;   // packed: its length and the number of lists (what a record holds is cut to them)
+    __device__ inline uint32_t key(uint32_t p) const { return record_key(pairs[p].x, raw); }
+    // retrieval-local index and list id of record p, whose pair is pr
+    __device__ inline void split(uint2 pr, uint32_t p, uint32_t &where, uint32_t &list) const {
+        if (packed) {
+            const uint32_t stored = min(pr.y & kPackedPosMask, pos_n - 1u);
+            where = pos ? (uint32_t)pos[stored] : stored;
+            list = min(pr.y >> kPackedPosBits, L - 1u);
+        } else {
+            where = pr.y;
+            list = aux ? (uint32_t)aux[p] : 0u;
+        }
+    }
+    __device__ inline CandRec rec(uint32_t p) const {
+        const uint2 pr = pairs[p];
+        CandRec r;
+        r.key = record_key(pr.x, raw);
+        split(pr, p, r.where, r.list);
+        return r;
+    }
+};
+
 template <int R>
-__device__ inline void select_regs(int raw, uint32_t cnt, int k, const uint2 *pairs, const uint16_t *aux,
-                                   SelectOut out, uint32_t (*red)[kSelWaves],
+__device__ inline void select_regs(const MemRecords &src, uint32_t cnt, int k, SelectOut out, uint32_t (*red)[kSelWaves],
                                    uint32_t *wsum, SelScratch *ss, float *ref1_out) {
     uint32_t key[R], where[R], list[R];
+    uint2 pr[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {  // all loads in flight before the first use
         const uint32_t p = (uint32_t)r * kSelThreads + threadIdx.x;
-        const uint2 pr = p < cnt ? pairs[p] : make_uint2(0u, 0u);
-        key[r] = p < cnt ? record_key(pr.x, raw) : 0u;
-        where[r] = pr.y;
-        list[r] = (aux && p < cnt) ? aux[p] : 0u;
+        pr[r] = p < cnt ? src.pairs[p] : make_uint2(0u, 0u);
+    }
+    if (src.packed) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t p = (uint32_t)r * kSelThreads + threadIdx.x;
+            key[r] = p < cnt ? record_key(pr[r].x, src.raw) : 0u;
+            where[r] = min(pr[r].y & kPackedPosMask, src.pos_n - 1u);
+            list[r] = min(pr[r].y >> kPackedPosBits, src.L - 1u);
+        }
+        if (src.pos) {  // (one batch of look-ups)
+#pragma unroll
+            for (int r = 0; r < R; ++r) where[r] = (uint32_t)src.pos[where[r]];
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t p = (uint32_t)r * kSelThreads + threadIdx.x;
+            key[r] = p < cnt ? record_key(pr[r].x, src.raw) : 0u;
+            where[r] = pr[r].y;
+            list[r] = (src.aux && p < cnt) ? src.aux[p] : 0u;
+        }
     }
     select_loaded<R>(key, where, list, cnt, k, out, red, wsum, ss, ref1_out);
 }
@@ -514,47 +584,16 @@ __device__ inline uint32_t kth_largest_mem(ValAt val_at, uint32_t cnt, uint32_t 
     return lo;
 }
 
-// One candidate as the streaming selection sees it.
-struct CandRec {
-    uint32_t key, where, list;
-};
-// candidates in memory: (key or logit bits, retrieval-local index) pairs and list ids
-struct MemRecords {
-    const uint2 *pairs;
-    const uint16_t *aux;
-    int raw;
-    __device__ inline uint32_t key(uint32_t p) const { return record_key(pairs[p].x, raw); }
-    __device__ inline CandRec rec(uint32_t p) const {
-        const uint2 pr = pairs[p];
-        return {record_key(pr.x, raw), pr.y, aux ? (uint32_t)aux[p] : 0u};
-    }
-};
-
-// A candidate record of the fused decode kernel: the logit's bit pattern and one word that holds
-// the key's STORED position (low 20 bits) and its list id (high 12 bits).  The retrieval-local
-// index, which the tie rule and the output are defined on, is looked up in the position map.
-constexpr int kPackedPosBits = 20;
-constexpr uint32_t kPackedPosMask = (1u << kPackedPosBits) - 1u;
-__device__ inline uint32_t pack_candidate(uint32_t stored, uint32_t list) { return stored | (list << kPackedPosBits); }
-__device__ inline uint2 load_dev(const uint2 *p) {
-    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-    return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
-}
-__device__ inline void store_dev(uint2 *p, uint2 v) {
-    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), (unsigned long long)v.x | ((unsigned long long)v.y << 32),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 // ... read with device-scope loads (they were written by other workgroups of the same launch)
 struct PackedRecords {
     const uint2 *pairs;
-    const int32_t *pos;  // the stream's position map
-    uint32_t pos_n, L;   // its length, and the number of lists (what a record holds is cut to them)
+    const int32_t *pos;  // NULL: the records hold retrieval-local indices; else stored positions, translated by this map
+    uint32_t pos_n, L;   // keys per stream and the number of lists (what a record holds is cut to them)
     __device__ inline uint32_t key(uint32_t p) const { return order_key(__uint_as_float(load_dev(pairs + p).x)); }
     __device__ inline CandRec rec(uint32_t p) const {
         const uint2 pr = load_dev(pairs + p);
-        const uint32_t stored = min(pr.y & kPackedPosMask, pos_n - 1u);
-        return {order_key(__uint_as_float(pr.x)), (uint32_t)pos[stored], min(pr.y >> kPackedPosBits, L - 1u)};
+        const uint32_t at = min(pr.y & kPackedPosMask, pos_n - 1u);
+        return {order_key(__uint_as_float(pr.x)), pos ? (uint32_t)pos[at] : at, min(pr.y >> kPackedPosBits, L - 1u)};
     }
 };
 // every stored key of a stream as a candidate, scored again on every pass (a row whose estimate
