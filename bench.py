@@ -51,11 +51,31 @@ KERNELS = ["lut_build", "sample_thresh", "scan_emit", "select_final", "attend"]
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_step_cfg{cfg}_hbm_traffic.json")
 
 
+def kernel_sources_digest():
+    """SHA-256 over the library's kernel sources (file names and contents, in name order): the stamp a
+    counter measurement carries, so that a figure measured on other kernels is not passed on as today's."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "pqhsa_release_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(cfg_id, kernel):
+    """(HBM bytes per launch from the committed counter runs, the commit they were taken at); the bytes
+    are None when there is no measurement of this kernel or the kernel sources have changed since."""
     try:
         with open(TRAFFIC_FILE.format(cfg=cfg_id)) as f:
             rec = json.load(f)
-        return int(rec["bytes_per_launch"][kernel]), rec.get("commit")
+        nbytes = int(rec["bytes_per_launch"][kernel])
+        if rec.get("sources_sha256") != kernel_sources_digest():
+            return None, rec.get("commit")
+        return nbytes, rec.get("commit")
     except (OSError, KeyError, ValueError):
         return None, None
 
@@ -512,6 +532,14 @@ class Timed:
         self.event_every = max(1, event_every)
         self.ms_per_step, dom_ms = self.logged_run(self.steps, self.dominant_i, self.event_every)
         self.dominant_us = dom_ms[self.dominant_i] * 1000.0
+        # the candidate scan measured the same way, in a pass of its own (the second half of the metric)
+        self.scan_us = None
+        scan_i = KERNELS.index("scan_emit")
+        if self.launches != 1 and scan_i != self.dominant_i:
+            _, scan_ms = self.logged_run(self.steps, scan_i, self.event_every)
+            self.scan_us = scan_ms[scan_i] * 1000.0
+        elif self.launches != 1:
+            self.scan_us = self.dominant_us
         layer = self.layers[0]
         ab = self.bytes = layer.algorithmic_bytes()
         self.algo = {"lut_build": ab["tables"], "sample_thresh": ab["sample"], "scan_emit": ab["scan"],
@@ -559,6 +587,26 @@ class Timed:
             "traffic_measured_at_commit": commit,
             "algorithmic_bytes": nbytes,
             "launch_us": round(self.dominant_us, 3),
+            "launches_timed": (self.steps + self.event_every - 1) // self.event_every,
+        }
+
+    def roofline_scan(self):
+        """The candidate scan against the HBM roofline (None for a step served by the one-kernel path)."""
+        if self.scan_us is None or self.scan_us <= 0:
+            return None
+        nbytes = self.algo["scan_emit"]
+        traffic, commit = measured_traffic(self.cfg_id, "scan_emit")
+        return {
+            "kernel": "scan_emit",
+            "bound": "hbm",
+            "achieved": round(nbytes / 1e3 / self.scan_us, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(nbytes / 1e3 / self.scan_us / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "traffic_measured_at_commit": commit,
+            "algorithmic_bytes": nbytes,
+            "launch_us": round(self.scan_us, 3),
             "launches_timed": (self.steps + self.event_every - 1) // self.event_every,
         }
 
@@ -700,6 +748,7 @@ def main():
                    "num_lists": LISTS, "top_fraction": FRACTION, "sink": SINK, "local_window": LOCAL,
                    "kv_dtype": str(layer.dtype).replace("torch.", ""), "resident_layers": len(run.layers)},
         "roofline": run.roofline(),
+        "roofline_scan": run.roofline_scan(),
         "tokens_per_s": round(layer.B / (MODEL_LAYERS * ms_per_step / 1000.0), 1),
         "step_bytes_MB": round(ab["total"] / 1e6, 2),
         "step_roofline_frac": run.step_frac(),
@@ -730,6 +779,10 @@ def main():
     copy_gbps = copy_bandwidth(device)
     result["hbm_copy_GBps"] = round(copy_gbps, 1)
     result["roofline"]["frac_of_copy"] = round(result["roofline"]["achieved"] / copy_gbps, 4)
+    if result["roofline_scan"]:
+        result["roofline_scan"]["frac_of_copy"] = round(result["roofline_scan"]["achieved"] / copy_gbps, 4)
+    # the whole step against the same ceiling: its algorithmic bytes over the timed step
+    result["step_frac_of_copy"] = round(ab["total"] / 1e3 / (ms_per_step * 1000.0) / copy_gbps, 4)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(layer, args.cpu_seconds)
     others = args.other_configs if args.other_configs is not None else args.config == 2

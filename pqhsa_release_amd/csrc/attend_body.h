@@ -99,11 +99,14 @@ struct RawSlice {
 // that too and reads the row's flags: the workgroup whose flag became visible last sees them all
 // set.  Two that finish together may both see that, so those few draw a ticket from a counter and
 // the first folds: all partials under the row's maximum, with the background term, into the
-// output row.  (One counter incremented by every split instead of the flags serialises at the
-// memory side, about 0.27 us per increment: 8.6 us for a row of 32 splits.)  No cache-wide
-// write-back or invalidation is needed (a device-scope fence per workgroup made the kernel
-// several times slower).  Flags and counters are cleared by an earlier kernel of the step.
+// output row.  One counter incremented by every split instead of the flags serialises at the
+// memory side, about 0.27 us per increment (8.6 us for a row of 32 splits), but is a single round
+// trip where the flags take three: rows of at most kCountedSplits chunks are counted in instead.
+// No cache-wide write-back or invalidation is needed (a device-scope fence per workgroup made the
+// kernel several times slower).  Flags and counters are cleared by an earlier kernel of the step
+// (a counted row leaves its counter at zero by itself).
 constexpr int kFoldLanes = kAttThreads / kD;  // splits folded side by side
+constexpr int kCountedSplits = 8;
 
 // LDS of one attention workgroup apart from its list of row addresses
 struct __align__(16) AttendLds {
@@ -138,9 +141,18 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, AttendLds &lds, siz
     float(&acc_s)[kFoldLanes][kD] = lds.acc_s;
     float(&den_s)[kFoldLanes] = lds.den_s;
     const int tid = threadIdx.x;
-    drain_memory_ops();  // this thread's stores of the partial have completed before the flag is set
-    __syncthreads();
-    if (tid < kWave) {  // (at most 64 splits: one flag per lane)
+    drain_memory_ops();  // this thread's stores of the partial have completed ...
+    __syncthreads();     // ... and so have those of the whole workgroup
+    if (a.splits <= kCountedSplits) {
+        // few workgroups per row: each counts itself in (one round trip to memory); the one that draws
+        // the last number folds and puts the counter back to zero
+        if (tid == 0) {
+            uint32_t *count = a.arrive + a.rows * kMaxSplits + orow;
+            const uint32_t before = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_s = before + 1u == (uint32_t)a.splits;
+            if (last_s) __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    } else if (tid < kWave) {  // (at most 64 splits: one flag per lane)
         uint32_t *flags = a.arrive + orow * kMaxSplits;
         if (tid == 0) __hip_atomic_store(flags + split, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         drain_memory_ops();  // ... and the flag is visible before the row's flags are read
@@ -155,6 +167,21 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, AttendLds &lds, siz
     if (a.n_commit_dst && g == 0 && h == 0 && tid == 0) a.n_commit_dst[b] = a.n_commit_src[b];
     const float *part = a.partials + orow * a.splits * kPartWidth;
     const float r0 = (n > 0 && a.mass0) ? load_shared<FUSED>(a.ref0 + (size_t)bh * a.ref_stride + g) : -INFINITY;
+    // a row of few chunks: what this thread folds is requested now, together with the maxima below
+    constexpr int kPre = kCountedSplits / kFoldLanes;
+    const bool pre = a.splits <= kCountedSplits;
+    float pre_m[kPre], pre_l[kPre], pre_v[kPre], pre_b[kPre];
+    if (pre) {
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) {
+            const int s = sl + i * kFoldLanes;
+            const float *p = part + (s < a.splits ? s : 0) * kPartWidth;
+            pre_m[i] = s < a.splits ? peek(p) : -INFINITY;
+            pre_l[i] = peek(p + 1);
+            pre_v[i] = peek(p + 4 + d);
+            pre_b[i] = peek(p + 4 + kD + d);
+        }
+    }
     // the first wave takes one split per lane (at most 64 splits): maximum and mass sum
     if (tid < kWave) {
         float m = -INFINITY, ms0 = 0.0f;
@@ -179,14 +206,25 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, AttendLds &lds, siz
     }
     const float f0 = (ms0 != 0.0f && r0 > -INFINITY) ? __expf(r0 - m) : 0.0f;
     float acc = 0.0f, den = 0.0f;
+    if (pre) {  // (same order of additions as the loop below)
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) {
+            if (sl + i * kFoldLanes >= a.splits) break;
+            const float w = pre_m[i] == -INFINITY ? 0.0f : __expf(pre_m[i] - m);
+            den = __builtin_fmaf(pre_l[i], w, den);
+            acc = __builtin_fmaf(pre_v[i], w, acc);
+            acc = __builtin_fmaf(pre_b[i], f0, acc);
+        }
+    } else {
 #pragma unroll 4
-    for (int s = sl; s < a.splits; s += kFoldLanes) {  // independent loads: several splits in flight at once
-        const float *p = part + s * kPartWidth;
-        const float pm = peek(p);
-        const float w = pm == -INFINITY ? 0.0f : __expf(pm - m);
-        den = __builtin_fmaf(peek(p + 1), w, den);
-        acc = __builtin_fmaf(peek(p + 4 + d), w, acc);
-        acc = __builtin_fmaf(peek(p + 4 + kD + d), f0, acc);
+        for (int s = sl; s < a.splits; s += kFoldLanes) {  // independent loads: several splits in flight at once
+            const float *p = part + s * kPartWidth;
+            const float pm = peek(p);
+            const float w = pm == -INFINITY ? 0.0f : __expf(pm - m);
+            den = __builtin_fmaf(peek(p + 1), w, den);
+            acc = __builtin_fmaf(peek(p + 4 + d), w, acc);
+            acc = __builtin_fmaf(peek(p + 4 + kD + d), f0, acc);
+        }
     }
     acc_s[sl][d] = acc;
     if (d == 0) den_s[sl] = den;

@@ -1166,3 +1166,68 @@ def test_event_log_counts_steps_and_samples_them():
     steps(2)                                       # the log is off again: nothing recorded, nothing to collect
     assert lib.pqhsa_profile_every(0) != 0 and b"stride" in lib.pqhsa_last_error()
 
+
+
+def test_fold_of_sixty_four_partials_per_row_over_hundreds_of_launches():
+    """The hand-over between the workgroups of a query row in the exact attention: every workgroup
+    writes its partial result and a flag, and the one that finds all flags set folds the partials.
+    Here each of 512 query rows (16 ragged sequences, 8 KV heads, groups of 4) attends over up to
+    24 388 rows, which the launch cuts into the largest number of chunks it uses, 64 per query row
+    (32 768 workgroups per launch; short sequences leave some of their chunks empty).  The stand-alone
+    entry point is launched 300 times on one selection: every output must equal the first bit for
+    bit (the fold adds the partials in chunk order whichever workgroup does it, so a partial read
+    before it was complete, or a row folded twice or not at all, shows), and the first must equal a
+    dense fp32 attention over the same rows."""
+    import bench
+
+    dev = _cuda()
+    layer = bench.Layer(3, 977, torch.device(dev))
+    B, H, G = layer.B, layer.H, layer.G
+    rows = B * H * G
+    k_cap = 24320
+    full_max = bench.SINK + bench.LOCAL
+    assert rows == 512 and (full_max + k_cap + 383) // 384 == 64
+    gen = torch.Generator(device=dev).manual_seed(5)
+    tidx = torch.zeros(rows, k_cap, dtype=torch.int32, device=dev)
+    tcnt = torch.zeros(rows, dtype=torch.int32, device=dev)
+    for b in range(B):
+        n_b = layer.n[b]
+        cnt = min(n_b, k_cap)
+        for hg in range(H * G):
+            r = b * H * G + hg
+            tidx[r, :cnt] = torch.randperm(n_b, generator=gen, device=dev)[:cnt].to(torch.int32)
+            tcnt[r] = cnt
+    # no background: per-list masses of zero, and selected logits so low that nothing is taken off them
+    tval = torch.full((rows, k_cap), -1e30, device=dev)
+    mass = torch.zeros(rows, bench.LISTS, device=dev)
+    rmax = torch.zeros(rows, device=dev)
+    q = layer.q.float()
+    scale = 1.0 / np.sqrt(128.0)
+
+    def launch():
+        out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
+        ops.hybrid_attend_paged(q, out, layer.kv, layer.index, G, layer.seq_lens, sink=bench.SINK, full_max=full_max,
+                                topk_idx=tidx, topk_val=tval, topk_cnt=tcnt, list_mass=mass, row_max=rmax, scale=scale)
+        torch.cuda.synchronize()
+        return out
+
+    first = launch()
+    assert bool(torch.isfinite(first).all())
+    # dense attention over the same rows, for the shortest and the longest sequence and two more
+    order = sorted(range(B), key=lambda b: layer.lens[b])
+    for b in (order[0], order[-1], order[B // 2], order[1]):
+        ln = layer.lens[b]
+        for h, g in ((0, 0), (H - 1, G - 1), (3, 1)):
+            r = (b * H + h) * G + g
+            cnt = int(tcnt[r])
+            pos = torch.cat([torch.arange(bench.SINK, device=dev), torch.arange(ln - bench.LOCAL, ln, device=dev),
+                             bench.SINK + tidx[r, :cnt].long()])
+            assert len(set(pos.tolist())) == pos.numel()
+            keys, values = ops.paged_gather_at(layer.kv, b, pos.unsqueeze(0).expand(H, -1).contiguous())
+            w = torch.softmax((keys[h].float() @ q[b, h * G + g]) * scale, dim=0)
+            want = w @ values[h].float()
+            err = float((first[b, h * G + g] - want).abs().max())
+            assert err <= 2e-3, (b, h, g, err)
+    for rep in range(300):
+        again = launch()
+        assert torch.equal(again, first), (rep, float((again - first).abs().max()))
