@@ -228,31 +228,13 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
         // Row by row.  The comparisons stay lane masks in scalar registers, and everything about the
         // candidates' slots is scalar arithmetic on those masks (their bit counts) but the rank of a
         // lane inside its mask.  Slots go to key 0 of every lane first, then key 1, ...; within one, by lane.
+        // A row whose candidates of this window do not fit its staging area (a list close to the
+        // query: most of its keys are candidates) writes them straight to memory; those rows are
+        // settled after the others, so that all of them share one round trip for their reservations.
         float e[4][GP];
-#pragma unroll
-        for (int g = 0; g < GP; ++g) {
-            bool cand[4];
-            unsigned long long cm[4];
-            uint32_t tot = 0u;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                cand[j] = s[j][g] >= thr_f[g];
-                cm[j] = __ballot(cand[j]);
-                tot += (uint32_t)__popcll(cm[j]);
-                e[j][g] = cand[j] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
-            }
-            if (tot == 0u) continue;  // wave-uniform
-            // A window whose candidates do not fit the row's staging area (a list close to the
-            // query: most of its keys are candidates) reserves room in memory and writes them there.
-            const bool to_memory = wcnt[g] + tot > (uint32_t)cap_w;
-            uint32_t first = wcnt[g];
-            if (to_memory) {
-                uint32_t at = 0u;
-                if (lane == 0) at = atomicAdd(&a.emit_count[(size_t)bh * GP + g], tot);
-                first = (uint32_t)__builtin_amdgcn_readfirstlane((int)at);
-            } else {
-                wcnt[g] += tot;
-            }
+        uint32_t direct = 0u, want_res = 0u;
+        auto emit_row = [&](const int g, const bool (&cand)[4], const unsigned long long (&cm)[4], uint32_t first,
+                            const bool to_memory) {
             const size_t o = ((size_t)bh * GP + g) * a.emit_cap;
             const uint32_t srow = ((uint32_t)wave_u * GP + g) * (uint32_t)cap_w;  // (scalar)
 #pragma unroll
@@ -280,6 +262,43 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
                     }
                 }
                 first += cnt_j;
+            }
+        };
+#pragma unroll
+        for (int g = 0; g < GP; ++g) {
+            bool cand[4];
+            unsigned long long cm[4];
+            uint32_t tot = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                cand[j] = s[j][g] >= thr_f[g];
+                cm[j] = __ballot(cand[j]);
+                tot += (uint32_t)__popcll(cm[j]);
+                e[j][g] = cand[j] ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][g], kLog2e, nref2[g]));
+            }
+            if (tot == 0u) continue;  // wave-uniform
+            if (wcnt[g] + tot > (uint32_t)cap_w) {  // (wave-uniform) straight to memory, below
+                direct |= 1u << g;
+                if (lane == g) want_res = tot;
+                continue;
+            }
+            emit_row(g, cand, cm, wcnt[g], false);
+            wcnt[g] += tot;
+        }
+        if (direct != 0u) {  // (wave-uniform, rare) lane g reserves the room of row g: one round trip for all rows
+            uint32_t at = 0u;
+            if (want_res != 0u) at = atomicAdd(&a.emit_count[(size_t)bh * GP + lane], want_res);
+#pragma unroll
+            for (int g = 0; g < GP; ++g) {
+                if (!((direct >> g) & 1u)) continue;  // wave-uniform
+                bool cand[4];
+                unsigned long long cm[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {  // (the comparison again: its masks were not kept)
+                    cand[j] = s[j][g] >= thr_f[g];
+                    cm[j] = __ballot(cand[j]);
+                }
+                emit_row(g, cand, cm, (uint32_t)__builtin_amdgcn_readlane((int)at, g), true);
             }
         }
         // ---- background: weights summed per list ----------------------------------------------
