@@ -10,11 +10,12 @@
 // The kernel is bound by vector instruction issue with four waves per SIMD.  (Tried and slower:
 // windows handed out through counters in memory — the atomics' answers return in order, with the
 // index loads queued behind them; 1024-thread workgroups, one per compute unit — the slowest of
-// 16 waves holds the whole unit; larger staging areas — fewer workgroups fit a unit.)
+// 16 waves holds the whole unit; staging areas so large that fewer workgroups fit a unit.)
 //
-// Candidate slots come from a wave prefix sum: sparse windows go to wave-private LDS staging (one
-// reservation in memory per workgroup and row, at the end), a window too dense for the staging
-// area reserves once per row and writes straight to memory.  Stored keys are ordered by list, so
+// Candidate slots come from the bit counts of the compare masks (scalar) and the rank of a lane
+// within its mask: sparse windows go to wave-private LDS staging (one reservation in memory per
+// workgroup and row, at the end), the rows of a window too dense for their staging areas share one
+// reservation round trip and write straight to memory.  Stored keys are ordered by list, so
 // the per-list sums are wave-level segment sums with one LDS update per (wave, list).
 #include "common.h"
 #include "scan_common.h"
@@ -94,7 +95,11 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
     if (tiles < 1) tiles = 1;
     a.tile_windows = (int)((windows_mean + tiles - 1) / tiles);
     tiles = (windows + a.tile_windows - 1) / a.tile_windows;
-    const size_t lds = scan_emit_lds_bytes(GP, a.L, a.stage_cap, a.emit_aux != nullptr);
+    size_t lds = scan_emit_lds_bytes(GP, a.L, a.stage_cap, a.emit_aux != nullptr);
+    if (lds + (size_t)kM * kCodes * GP * sizeof(float) > 150 * 1024) {  // many lists: a smaller staging area
+        a.stage_cap = a.stage_cap / 2 < 32 ? 32 : a.stage_cap / 2;
+        lds = scan_emit_lds_bytes(GP, a.L, a.stage_cap, a.emit_aux != nullptr);
+    }
     PQHSA_REQUIRE(lds + (size_t)kM * kCodes * GP * sizeof(float) <= 150 * 1024, "scan_emit: %zu bytes of LDS needed", lds);
     PQHSA_REQUIRE(!a.packed_records || (a.n_cap <= (int64_t)kPackedPosMask + 1 && a.L <= 4096),
                   "scan_emit: packed candidate records hold 20 bits of position and 12 bits of list id");
