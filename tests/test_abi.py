@@ -159,8 +159,9 @@ def test_ctypes_mirrors_follow_the_header_field_order():
 
 
 def test_integration_document_stub_matches_the_library_structs():
-    """The binding INTEGRATION.md shows is built from its text and laid over the library's mirrors:
-    same fields, same offsets, same sizes, and the argument list of pqhsa_decode_step."""
+    """The ctypes binding that the integration notes at the repository root show is built from their
+    text and laid over the library's mirrors: same fields, same offsets, same sizes, and the argument
+    list of pqhsa_decode_step."""
     import ctypes
 
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()

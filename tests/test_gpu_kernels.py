@@ -827,7 +827,7 @@ def test_decode_step_graph_replays_match_eager_runs(general_path):
         assert torch.equal(ws.topk_idx.sort(dim=1).values, want_idx), round_
         np.testing.assert_allclose(out.cpu().numpy(), want_out.cpu().numpy(), atol=1e-5, err_msg=str(round_))
         assert torch.isfinite(junk)
-        # ... and the replay against the fixed-order oracle on this round's query
+        # ... and the replay against the fixed-order oracle on this pass's query
         qh = q.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
         got_out = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
         got_idx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
