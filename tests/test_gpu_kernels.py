@@ -1231,3 +1231,21 @@ def test_fold_of_sixty_four_partials_per_row_over_hundreds_of_launches():
     for rep in range(300):
         again = launch()
         assert torch.equal(again, first), (rep, float((again - first).abs().max()))
+
+
+def test_candidate_records_of_an_index_with_more_than_a_million_slots_per_sequence():
+    """A candidate record names its key by stored position in 20 bits of one word; an index whose
+    sequences have room for more than 2^20 keys keeps the records of (logit, retrieval-local index)
+    with the list ids in a second array, read with the position map in the scan and selected without
+    a look-up.  Same step, same oracle; the dense windows of the needle queries exercise the rows
+    that write straight to memory in that form too."""
+    dev = _cuda()
+    p = Problem(lens=[20000, 9000], heads=2, groups=4, lists=32, seed=47)
+    idx = p.device_index(dev, spare=(1 << 20))
+    assert idx.n_cap > (1 << 20)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 5   # (no one-launch form either)
+    before = ws.rescans()
+    assert _check_step(p, idx, kv, ws, 0.03) == 1
+    assert ws.rescans() == before
