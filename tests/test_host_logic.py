@@ -479,3 +479,25 @@ def test_ema_rows_moves_the_rows_that_got_vectors_and_no_others():
             want = 0.75 * before[j] + 0.25 * (mine.sum(0) / mine.shape[0])
             torch.testing.assert_close(table[j], want, rtol=0, atol=1e-6)
     assert torch.equal(table[7], before[7])
+
+
+def test_bench_passes_counter_traffic_on_only_for_the_kernels_it_was_measured_on(tmp_path, monkeypatch):
+    """bench.py's roofline objects carry the HBM bytes per launch from the committed counter runs only
+    while the kernel sources are the ones the counters were taken on (a digest in the file)."""
+    import json
+
+    import bench
+
+    digest = bench.kernel_sources_digest()
+    assert len(digest) == 64 and digest == bench.kernel_sources_digest()
+    rec = {"commit": "abc1234", "sources_sha256": digest, "bytes_per_launch": {"attend": 123, "scan_emit": 45}}
+    path = tmp_path / "decode_step_cfg{cfg}_hbm_traffic.json"
+    (tmp_path / "decode_step_cfg7_hbm_traffic.json").write_text(json.dumps(rec))
+    monkeypatch.setattr(bench, "TRAFFIC_FILE", str(path))
+    assert bench.measured_traffic(7, "attend") == (123, "abc1234")
+    assert bench.measured_traffic(7, "scan_emit") == (45, "abc1234")
+    assert bench.measured_traffic(7, "lut_build") == (None, None)          # no figure for this kernel
+    assert bench.measured_traffic(8, "attend") == (None, None)             # no file for this configuration
+    rec["sources_sha256"] = "0" * 64                                        # measured on other kernels
+    (tmp_path / "decode_step_cfg7_hbm_traffic.json").write_text(json.dumps(rec))
+    assert bench.measured_traffic(7, "attend") == (None, "abc1234")
