@@ -691,18 +691,14 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
     if (a.share_map)
         for (int i = tid; i < (int)a.share_stride; i += kSelThreads) share_s[i] = 0u;
     if constexpr (RS > 0) {
-        // Packed records (the launcher sends other records to the RS = 0 form).  The look-ups of the
-        // retrieval-local indices are the last loads requested, so that nothing else queues behind
-        // them; they travel while the keys are sorted out.  (Slots past the count look up slot 0.)
+        // Packed records (the launcher sends other records to the RS = 0 form): the stored position for
+        // now; the look-ups of the retrieval-local indices are requested inside the selection, once
+        // the keys' histogram updates are under way.  (Slots past the count look up slot 0.)
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
             skey[r] = record_key(pr[r].x, a.raw_keys);
             swhere[r] = (uint32_t)r * kSelThreads + tid < cnt ? min(pr[r].y & kPackedPosMask, recs.pos_n - 1u) : 0u;
             slist[r] = min(pr[r].y >> kPackedPosBits, recs.L - 1u);
-        }
-        if (recs.pos) {  // (uniform)
-#pragma unroll
-            for (int r = 0; r < RS; ++r) swhere[r] = (uint32_t)recs.pos[swhere[r]];
         }
     }
     __syncthreads();
@@ -725,7 +721,14 @@ __global__ __launch_bounds__(kSelThreads, PACK ? 8 : 4) void select_final_kernel
             for (int r = 0; r < RS; ++r) {
                 if ((uint32_t)r * kSelThreads + tid >= cnt) skey[r] = 0u, slist[r] = 0u;  // (their index is that of slot 0: unused)
             }
-            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1, lo_hint, hi_hint);
+            const int32_t *pos_row = recs.pos;
+            auto look_up = [&]() {
+                if (pos_row) {  // (uniform)
+#pragma unroll
+                    for (int r = 0; r < RS; ++r) swhere[r] = (uint32_t)pos_row[swhere[r]];
+                }
+            };
+            select_loaded<RS>(skey, swhere, slist, cnt, k, out, red, wsum, &ss, &ref1, lo_hint, hi_hint, false, look_up);
             done = true;
         }
     }

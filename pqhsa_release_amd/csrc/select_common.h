@@ -260,11 +260,16 @@ struct SelectOut {
 
 // Candidates in registers (cnt <= R * 1024): candidate p = r * 1024 + tid sits in slot r of thread
 // tid; slots at or past cnt hold key 0.
-template <int R>
+// `late` is called once by every thread after the keys' histogram updates are issued and before
+// `where` is first read: a place to request what `where` still lacks (it may write `where`).
+struct NothingLate {
+    __device__ inline void operator()() const {}
+};
+template <int R, typename Late = NothingLate>
 __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], const uint32_t (&list)[R], uint32_t cnt,
                                      int k, SelectOut out, uint32_t (*red)[kSelWaves],
                                      uint32_t *wsum, SelScratch *ss, float *ref1_out, uint32_t lo_hint = 0u,
-                                     uint32_t hi_hint = 0u, bool lo_exact = false) {
+                                     uint32_t hi_hint = 0u, bool lo_exact = false, Late late = Late()) {
     const int tid = threadIdx.x;
     int step = 0;
     bool exact = false;
@@ -302,6 +307,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
                         : key[r] <= lo_key ? 0u : min((key[r] - lo_key) >> shift, (uint32_t)kSelBins - 1u);
             if (bucket[r] != 0xffffffffu) atomicAdd(&ss->hist[bucket[r]], 1u);
         }
+        late();
         if (tid == 0) ss->bin = 0xffffffffu;
         __syncthreads();
         PQHSA_SELECT_MARK(2);
@@ -351,6 +357,7 @@ __device__ inline void select_loaded(uint32_t (&key)[R], uint32_t (&where)[R], c
             searched = true;
         }
     } else {  // nothing is selected: the reference of the losers' weights is the largest key
+        late();
         uint32_t kmax = 0u;
 #pragma unroll
         for (int r = 0; r < R; ++r) kmax = max(kmax, key[r]);
