@@ -544,6 +544,9 @@ class Timed:
         ab = self.bytes = layer.algorithmic_bytes()
         self.algo = {"lut_build": ab["tables"], "sample_thresh": ab["sample"], "scan_emit": ab["scan"],
                      "select_final": 0, "attend": ab["exact"] + ab["full"] + ab["bg"]}
+        if self.launches == 4:  # tables and threshold estimate share the first launch (booked under its slot)
+            self.algo["lut_build"] += self.algo["sample_thresh"]
+            self.algo["sample_thresh"] = 0
         if self.launches == 1:
             self.survey_us = {name: (us if name == self.dominant else 0.0) for name, us in self.survey_us.items()}
             self.algo = {name: (ab["total"] if name == self.dominant else 0) for name in KERNELS}
@@ -611,12 +614,18 @@ class Timed:
         }
 
     def label(self, name):
+        if self.launches == 4 and name == "lut_build":
+            return "tables_thresh (tables + threshold estimate)"
         return "decode_small (whole step)" if self.launches == 1 and name == self.dominant else name
+
+    def hidden(self, name):
+        """Slots of the event log that hold no launch of their own in this step's form."""
+        return (self.launches == 1 and name != self.dominant) or (self.launches == 4 and name == "sample_thresh")
 
     def kernels(self):
         out = {}
         for name in KERNELS:
-            if self.launches == 1 and name != self.dominant:
+            if self.hidden(name):
                 continue
             us = self.survey_us[name]
             out[self.label(name)] = {"us": round(us, 3), "algo_MB": round(self.algo[name] / 1e6, 3),
@@ -634,8 +643,7 @@ class Timed:
                 "step_bytes_MB": round(self.bytes["total"] / 1e6, 2), "step_roofline_frac": self.step_frac(),
                 "launches_per_step": self.launches,
                 "dominant": {"kernel": r["kernel"], "launch_us": r["launch_us"], "GBps": r["achieved"], "frac": r["frac"]},
-                "kernels_us": {self.label(k): round(v, 2) for k, v in self.survey_us.items()
-                               if self.launches != 1 or k == self.dominant},
+                "kernels_us": {self.label(k): round(v, 2) for k, v in self.survey_us.items() if not self.hidden(k)},
                 "rescanned_rows": sum(l.ws.rescans() for l in self.layers)}
 
     def gather_ceiling(self, reps=30):

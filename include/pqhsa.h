@@ -134,6 +134,12 @@ typedef struct pqhsa_select {
  * that is faster at every measured shape, because rows of a group already meet in the L2 and the
  * classification pass and the extra partial records cost more than the saved fetches. */
 #define PQHSA_SELECT_SHARE_ROWS 4
+/* A step of the general path that appends nothing, with at most 256 query rows (batches padded to
+ * a multiple of 8 streams), at most 512 lists and at most 8 192 sampled keys per stream, builds
+ * each query row's lookup tables and its threshold estimate in ONE launch (four launches per step
+ * instead of five; same tables, thresholds and results to the bit).  This flag keeps the two as
+ * separate launches, as steps of every other shape have them. */
+#define PQHSA_SELECT_SEPARATE_TABLES 8
 
 const char *pqhsa_version(void);
 const char *pqhsa_last_error(void);
@@ -386,7 +392,9 @@ const uint32_t *pqhsa_decode_candidate_counts(void *workspace);
  * short-context kernel serves it (no append, PQHSA_SELECT_GENERAL_PATH not set, at most 16 384
  * indexed keys per stream, at most 256 query rows, at most 1 024 lists, k_cap at most 2 048), 3 when
  * scan, selection and attention share one launch (see PQHSA_SELECT_ONE_LAUNCH; the event
- * log books that launch under the scan's slot), else PQHSA_PROFILE_KERNELS.  With one launch the
+ * log books that launch under the scan's slot), PQHSA_PROFILE_KERNELS - 1 when the tables and
+ * the threshold estimate share a launch (see PQHSA_SELECT_SEPARATE_TABLES; booked under the
+ * tables' slot), else PQHSA_PROFILE_KERNELS.  With one launch the
  * event log books the whole step under its last slot and the other slots hold only the cost of
  * recording an event.  No counterpart in the
  * reference; for benchmarks and monitors that label per-kernel times.

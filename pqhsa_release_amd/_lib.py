@@ -70,6 +70,7 @@ class Select(ctypes.Structure):
 SELECT_GENERAL_PATH = 1
 SELECT_ONE_LAUNCH = 2
 SELECT_SHARE_ROWS = 4
+SELECT_SEPARATE_TABLES = 8
 
 
 class PqhsaError(RuntimeError):

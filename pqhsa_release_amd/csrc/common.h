@@ -210,14 +210,6 @@ __device__ inline float wave_max(float v) {
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
     return v;
 }
-__device__ inline uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        uint32_t o = (uint32_t)__shfl_xor((int)v, off, kWave);
-        v = v > o ? v : o;
-    }
-    return v;
-}
 __device__ inline int wave_sum_i32(int v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
@@ -239,6 +231,17 @@ constexpr int kDppBcast15 = 0x142;     // lane 15 of each row to the next row
 constexpr int kDppBcast31 = 0x143;     // lane 31 to rows 2 and 3
 constexpr int kDppWaveShl1 = 0x130;    // lane i reads lane i+1 of the wave (0 for the last lane)
 constexpr int kDppWaveShr1 = 0x138;    // lane i reads lane i-1 of the wave (0 for lane 0)
+
+// largest value of the wave, returned in every lane
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)dpp_move<kDppXor1>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppXor2>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppHalfMirror>((int)v));
+    v = max(v, (uint32_t)dpp_move<kDppMirror>((int)v));
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(r0, r1), max(r2, r3));
+}
 
 // sum over the 16 lanes of a row group (one DPP row), returned in each of them
 __device__ inline float group_sum16(float v) {

@@ -25,7 +25,13 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        uint32_t *emit_count, uint32_t *thr_key, int32_t *k_row, float *ref_val,
                        void *pairs, uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
-                       const AppendFinish *append, uint32_t *share_map, int64_t share_stride, hipStream_t stream);
+                       const AppendFinish *append, uint32_t *share_map, int64_t share_stride, bool thresholds_known,
+                       hipStream_t stream);
+bool decode_tables_thresh_fits(const pqhsa_index *index, int G);
+int decode_tables_thresholds(const void *q, int q_dtype, const pqhsa_index *index, int G, int GP, float eps, float *qnorm,
+                             float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, float scale,
+                             const pqhsa_select *select, uint32_t *thr_key, int32_t *k_row, float *ref_val,
+                             hipStream_t stream);
 bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap);
 int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                  const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const pqhsa_select *select, float scale,
@@ -153,7 +159,10 @@ extern "C" int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t 
     if (small) return 1;
     const bool fused = (select->flags & PQHSA_SELECT_ONE_LAUNCH) &&
                        decode_fused_fits(index->batch, index->kv_heads, G, index->n_cap, n_max, select->n_mean, index->num_lists);
-    return fused ? 3 : PQHSA_PROFILE_KERNELS;
+    if (fused) return 3;
+    // tables and thresholds in one launch when nothing is appended and every query row gets a compute unit
+    const bool merged = !appending && !(select->flags & PQHSA_SELECT_SEPARATE_TABLES) && decode_tables_thresh_fits(index, G);
+    return merged ? PQHSA_PROFILE_KERNELS - 1 : PQHSA_PROFILE_KERNELS;
 }
 
 static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqhsa_kv_view *kv,
@@ -211,10 +220,18 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     const pqhsa_index *index_in = index;
     index = &after;
     profile_mark(kProfLut, stream);
-    rc = launch_lut_build(q, q_dtype, index_in, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words,
-                          append_count ? &ap : nullptr, c.n_after, c.nearest, stream);
-    if (rc) return rc;
-    profile_mark(kProfSample, stream);
+    const bool merged = pqhsa_decode_step_launches(index_in, G, n_max, select, append_count != nullptr) == PQHSA_PROFILE_KERNELS - 1;
+    if (merged) {  // (the event log books the launch under the table slot)
+        rc = decode_tables_thresholds(q, q_dtype, index_in, G, GP, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words, scale,
+                                      select, c.thr_key, c.k_row, c.ref_val, stream);
+        if (rc) return rc;
+        profile_mark(kProfSample, stream);
+    } else {
+        rc = launch_lut_build(q, q_dtype, index_in, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words,
+                              append_count ? &ap : nullptr, c.n_after, c.nearest, stream);
+        if (rc) return rc;
+        profile_mark(kProfSample, stream);
+    }
     if (pqhsa_decode_step_launches(index_in, G, n_max, select, append_count != nullptr) == 3)
         return decode_fused(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, n_max, full_max + select->k_cap, c.qnorm, c.lut,
                             c.ls, scale, select, c.emit_count, c.thr_key, c.k_row, c.ref_val, c.pairs, c.emit_cap, c.mass,
@@ -225,7 +242,7 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     uint32_t *share = (select->flags & PQHSA_SELECT_SHARE_ROWS) && c.share_stride != 0 ? c.share : nullptr;
     rc = decode_scan_select(index, G, GP, n_max, c.qnorm, c.lut, c.ls, scale, select, c.emit_count, c.thr_key,
                             c.k_row, c.ref_val, c.pairs, c.aux, c.emit_cap, c.mass, c.rescans,
-                            topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, share, c.share_stride, stream);
+                            topk_idx, topk_val, topk_cnt, append_count ? &ap : nullptr, share, c.share_stride, merged, stream);
     if (rc) return rc;
     return decode_attend(q, q_dtype, out, kv, index, G, GP, seq_lens, sink, full_max + select->k_cap, topk_idx,
                          topk_cnt, select->k_cap, c.mass, c.ref_val, scale, c.partials, c.arrive,

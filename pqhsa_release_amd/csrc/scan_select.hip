@@ -497,26 +497,61 @@ struct SampleArgs {
 constexpr double kMarginSigmas = 5.0;
 constexpr int kSampleRegsMax = 32;  // sampled keys per thread: at most 32768 per row
 
-// R sampled keys per thread (s_cap <= R * 1024, chosen by the host).  The sampled keys are
-// requested before anything else, together with the row's tables and counts, so the kernel has
-// one round trip to memory before it computes.
-template <int R>
-__global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ __align__(16) uint32_t red[2][kSelWaves];
-    __shared__ uint32_t wsum[2 * kSelWaves];
-    __shared__ __align__(16) uint32_t hist[kSelBins];
-    __shared__ uint32_t found[2];
+// LDS of one threshold workgroup, beside its tables
+struct ThreshLds {
+    __align__(16) uint32_t red[2][kSelWaves];
+    uint32_t wsum[2 * kSelWaves];
+    __align__(16) uint32_t hist[kSelBins];
+    uint32_t found[2];
+};
+
+// The work of the workgroup of query row g of stream bh.  R sampled keys per thread (s_cap <=
+// R * 1024, chosen by the host).  The sampled keys are requested before anything else, together
+// with the row's tables and counts, so the kernel has one round trip to memory before it computes.
+// `tables(lut_s, ls_s, request, early)` leaves the row's PQ table and list scores in LDS (it may hold
+// barriers: every thread calls it) and returns the row's query norm; on the way it calls request()
+// once, where the loads of the first sampled keys should join its own, and then early() once, where
+// arithmetic on the stream's key counts costs it nothing.
+template <int R, int kBatch, class Tables>
+__device__ inline void sample_thresh_body(const SampleArgs &a, const int g, const int bh, ThreshLds &tl,
+                                          unsigned char *smem, [[maybe_unused]] const size_t trace_wg, Tables tables) {
+    uint32_t(&red)[2][kSelWaves] = tl.red;
+    uint32_t(&wsum)[2 * kSelWaves] = tl.wsum;
+    uint32_t(&hist)[kSelBins] = tl.hist;
+    uint32_t(&found)[2] = tl.found;
     const int tid = threadIdx.x;
-    const int g = blockIdx.x;
-    const int bh = blockIdx.y;
-    if (g == a.GP) {  // the extra workgroup of a step that appends: it shares this launch, nothing else
-        append_finish(a.append, bh);
-        return;
-    }
     const size_t row = (size_t)bh * a.GP + g;
-    [[maybe_unused]] const size_t trace_wg = blockIdx.x + (size_t)gridDim.x * blockIdx.y;
     PQHSA_TRACE_MARK(trace_sample, trace_wg, 0);
+    const size_t base = (size_t)bh * a.s_cap;  // (loads of one batch of kBatch are all in flight before their first use)
+    uint32_t code[kBatch], lid[kBatch];
+    float kn[kBatch];
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            // (the arrays are allocated up to s_cap; a slot past the row's sample is loaded without
+            // a branch, from the last slot, and left out below)
+            const int64_t p = min((int64_t)(r0 + r) * kSelThreads + tid, a.s_cap - 1);
+            code[r] = a.codes[base + p];
+            lid[r] = a.list_ids[base + p];
+            kn[r] = a.norms[base + p];
+        }
+    };
+    const int n = a.n_arr[bh / a.n_div];
+    const int ns = a.ns_arr[bh / a.n_div];
+    float *lut_s = reinterpret_cast<float *>(smem);   // [128]
+    float *ls_s = lut_s + kM * kCodes;                // [L]
+    // how many sampled keys the threshold keeps (`tables` calls this where it has time to spare)
+    int k = 0;
+    double want_d = 0.0;
+    auto resolve = [&]() __attribute__((always_inline)) {
+        // (the device-side count may have moved past what the host sized k_cap for: stay inside it)
+        k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
+        // expected sampled keys among the top max(k, 1), plus the margin
+        const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
+        const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
+        want_d = ceil(x * x) + 1.0;
+    };
+    const float qn = tables(lut_s, ls_s, [&]() __attribute__((always_inline)) { fetch(0); }, resolve);
     if (g >= a.G) {
         if (tid == 0) {
             a.thr_key[row] = 0xffffffffu;
@@ -526,34 +561,6 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         }
         return;
     }
-    constexpr int kBatch = R < 8 ? R : 8;  // loads of one batch are all in flight before their first use
-    const size_t base = (size_t)bh * a.s_cap;
-    uint32_t code[kBatch], lid[kBatch];
-    float kn[kBatch];
-    auto fetch = [&](int r0) {
-#pragma unroll
-        for (int r = 0; r < kBatch; ++r) {
-            const int64_t p = (int64_t)(r0 + r) * kSelThreads + tid;
-            const bool ok = p < a.s_cap;  // the arrays are allocated (and zero) up to s_cap
-            code[r] = ok ? a.codes[base + p] : 0u;
-            lid[r] = ok ? a.list_ids[base + p] : 0u;
-            kn[r] = ok ? a.norms[base + p] : 0.0f;
-        }
-    };
-    fetch(0);
-    const int n = a.n_arr[bh / a.n_div];
-    const int ns = a.ns_arr[bh / a.n_div];
-    float *lut_s = reinterpret_cast<float *>(smem);   // [128]
-    float *ls_s = lut_s + kM * kCodes;                // [L]
-    for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
-    for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
-    const float qn = a.qnorm[row];
-    // (the device-side count may have moved past what the host sized k_cap for: stay inside it)
-    const int k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
-    // expected sampled keys among the top max(k, 1), plus the margin
-    const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
-    const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
-    const double want_d = ceil(x * x) + 1.0;
     if (ns <= 0 || want_d >= (double)ns) {
         // sample too small to say anything: every key is a candidate and no background sum is formed
         if (tid == 0) {
@@ -614,6 +621,208 @@ __global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a
         a.k_row[row] = k;
         a.ref_val[row] = t == 0u ? -INFINITY : key_to_float(t);
     }
+}
+
+// the row's tables as an earlier launch left them in memory
+struct TablesFromMemory {
+    const SampleArgs &a;
+    int g, bh;
+    template <class Request, class Early>
+    __device__ float operator()(float *lut_s, float *ls_s, Request request, Early early) const {
+        const int tid = threadIdx.x;
+        request();
+        for (int i = tid; i < kM * kCodes; i += kSelThreads) lut_s[i] = a.lut[((size_t)bh * kM * kCodes + i) * a.GP + g];
+        for (int i = tid; i < a.L; i += kSelThreads) ls_s[i] = a.list_scores[((size_t)bh * a.L + i) * a.GP + g];
+        const float qn = a.qnorm[(size_t)bh * a.GP + g];
+        early();
+        return qn;
+    }
+};
+
+template <int R>
+__global__ __launch_bounds__(kSelThreads) void sample_thresh_kernel(SampleArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ ThreshLds t;
+    const int g = blockIdx.x;
+    const int bh = blockIdx.y;
+    if (g == a.GP) {  // the extra workgroup of a step that appends: it shares this launch, nothing else
+        append_finish(a.append, bh);
+        return;
+    }
+    sample_thresh_body<R, (R < 8 ? R : 8)>(a, g, bh, t, smem, blockIdx.x + (size_t)gridDim.x * blockIdx.y,
+                                           TablesFromMemory{a, g, bh});
+}
+
+// ---- tables and threshold estimate in one launch -------------------------------------------------
+// The workgroup of a query row builds the row's own tables (what lut_build_kernel computes for it,
+// by the same fixed-order chains, so to the same bits), leaves them in memory for the scan and the
+// selection, and goes on to the row's threshold estimate with the copy it holds in LDS: one launch
+// and one round trip to memory where the two kernels take two of each.  The row's L centroids
+// (at most 512) pass through LDS in two halves, elements 0..63 of every centroid and then elements
+// 64..127; a lane per list runs the list's chain over the first half, keeps the sum and goes on
+// over the second (eight waves for 512 lists).  The rows of one stream read the same centroids, so
+// their workgroups are dealt to one XCD (workgroups 8 apart), whose L2 fetches them once.
+constexpr int kTtLists = 512;               // lists a workgroup can stage
+constexpr int kTtHalf = kD / 2;             // elements per staged half
+constexpr int kTtStride = kTtHalf + 4;      // floats per staged half centroid (16-byte aligned rows that miss each other's banks)
+constexpr int kXcdCount = 8;
+
+struct TablesArgs {
+    const char *q;             // [B, H * G, 128]
+    const float *coarse;       // [BH, L, 128]
+    const float *codebooks;    // [BH, 8, 16, 16]
+    float eps;
+    float *qnorm, *lut, *list_scores;   // outputs, laid out as lut_build_kernel writes them
+    uint32_t *zero_base;       // scratch that the step's later kernels accumulate into
+    size_t zero_words;
+    int streams;
+};
+
+template <int DT, int R>
+__global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p, SampleArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ ThreshLds t;
+    __shared__ __align__(16) float qrow[kD];
+    __shared__ float qn_s;
+    const int tid = threadIdx.x;
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int g = slot % a.GP;
+    const int bh = (slot / a.GP) * kXcdCount + xcd;
+    const bool idle = bh >= p.streams;  // (the grid is whole rounds of the 8 XCDs)
+    const bool live = !idle && g < a.G;
+    // the query row first of all: its norm is computed while everything else travels
+    // (every wave loads elements lane and lane + 64, of a row that exists when its own does not:
+    // no branch to wait in; the first wave uses them)
+    const int lane = tid % kWave;
+    const size_t q_row = live ? (size_t)bh * a.G + g : 0;  // row (b * H + h) * G + g of q
+    const char *q_ptr = p.q + q_row * kD * (DT == PQHSA_F32 ? 4 : 2);
+    float qa = load1<DT>(q_ptr, lane), qb = load1<DT>(q_ptr, lane + kWave);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!live) qa = qb = 0.0f;
+    auto clear_scratch = [&]() __attribute__((always_inline)) {
+        const size_t nthreads = (size_t)gridDim.x * kSelThreads;
+        for (size_t i = (size_t)blockIdx.x * kSelThreads + tid; i < p.zero_words; i += nthreads) p.zero_base[i] = 0u;
+    };
+    if (idle) {
+        clear_scratch();
+        return;
+    }
+    const int L = a.L, GP = a.GP;
+    float *cs = reinterpret_cast<float *>(smem) + ((kM * kCodes + L + 3) & ~3);  // [kTtLists][kTtStride], past the tables
+
+    auto tables = [&](float *lut_s, float *ls_s, auto request, auto early) __attribute__((always_inline)) -> float {
+        // both halves of the centroids are requested at once, 8 loads of 16 bytes per thread and half:
+        // load u of a half is float4 (tid + 1024 u) of it, which is part i % 16 of list i / 16
+        // (no branch: what lies past the last list is loaded from the last list's end and never used;
+        // named values rather than arrays, which the compiler would keep in scratch memory here)
+        const float4 *c4 = reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD);
+        constexpr int kParts = kTtHalf / 4;  // float4 per half centroid
+        static_assert(kTtLists * kParts == 8 * kSelThreads, "the halves below are written out for 8 loads per thread");
+        const int last4 = L * (kD / 4) - 1;
+        auto centroid4 = [&](int half, int u) __attribute__((always_inline)) {
+            const int i = tid + u * kSelThreads;
+            return c4[min((i / kParts) * (kD / 4) + half * kParts + i % kParts, last4)];
+        };
+        const float4 a0 = centroid4(0, 0), a1 = centroid4(0, 1), a2 = centroid4(0, 2), a3 = centroid4(0, 3);
+        const float4 a4 = centroid4(0, 4), a5 = centroid4(0, 5), a6 = centroid4(0, 6), a7 = centroid4(0, 7);
+        const float4 b0 = centroid4(1, 0), b1 = centroid4(1, 1), b2 = centroid4(1, 2), b3 = centroid4(1, 3);
+        const float4 b4 = centroid4(1, 4), b5 = centroid4(1, 5), b6 = centroid4(1, 6), b7 = centroid4(1, 7);
+        __builtin_amdgcn_sched_barrier(0);
+        request();  // (the sampled keys behind the centroids: they are not needed before the tables stand)
+
+        // the row's norm by the first wave alone, while the others wait for their centroids: one
+        // chain over d in order, as in lut_build_kernel, every lane running it on the elements read
+        // from their lanes one by one
+        if (tid < kWave) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int d = 0; d < kWave; ++d) {
+                const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qa), d));
+                ss = __builtin_fmaf(x, x, ss);
+            }
+#pragma unroll
+            for (int d = 0; d < kWave; ++d) {
+                const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qb), d));
+                ss = __builtin_fmaf(x, x, ss);
+            }
+            const float nrm = sqrtf(ss);
+            const float qn0 = nrm < p.eps ? p.eps : nrm;
+            qrow[lane] = qa / qn0;
+            qrow[lane + kWave] = qb / qn0;
+            if (lane == 0) {
+                qn_s = qn0;
+                p.qnorm[(size_t)bh * GP + g] = live ? qn0 : 0.0f;
+            }
+        }
+        PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 5);
+        early();  // (the caller's arithmetic on the stream's key counts, while the centroids travel)
+        clear_scratch();
+        // PQ table: entry (m, c) by thread m * 16 + c of the workgroup's last two waves, after the
+        // list chains (the codebook entry is requested once the first half has left its registers:
+        // requested with the centroids, it would only stand in their way)
+        const bool lut_thread = tid >= kSelThreads - kM * kCodes;
+        const int e = lut_thread ? tid - (kSelThreads - kM * kCodes) : 0;
+        float4 w[kSub / 4];
+        const float4 *w4 = reinterpret_cast<const float4 *>(p.codebooks + ((size_t)bh * kM * kCodes + e) * kSub);
+        auto pq_table = [&]() __attribute__((always_inline)) {
+            const float *qm = qrow + (e / kCodes) * kSub;
+            float acc = 0.0f;
+            if (live) {
+#pragma unroll
+                for (int j = 0; j < kSub / 4; ++j) {
+                    acc = __builtin_fmaf(qm[4 * j], w[j].x, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 1], w[j].y, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 2], w[j].z, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 3], w[j].w, acc);
+                }
+            }
+            lut_s[e] = acc;
+            p.lut[((size_t)bh * kM * kCodes + e) * GP + g] = acc;
+        };
+        // list scores: list l by lane l % 64 of wave l / 64
+        const int l = tid;
+        float score = 0.0f;
+        auto stage = [&](int u, const float4 &v) __attribute__((always_inline)) {
+            const int i = tid + u * kSelThreads;
+            *reinterpret_cast<float4 *>(cs + (size_t)(i / kParts) * kTtStride + (i % kParts) * 4) = v;
+        };
+        auto run_half = [&](int half, const float4 &v0, const float4 &v1, const float4 &v2, const float4 &v3,
+                            const float4 &v4, const float4 &v5, const float4 &v6, const float4 &v7) __attribute__((always_inline)) {
+            stage(0, v0); stage(1, v1); stage(2, v2); stage(3, v3);
+            stage(4, v4); stage(5, v5); stage(6, v6); stage(7, v7);
+            if (half == 0) {
+#pragma unroll
+                for (int j = 0; j < kSub / 4; ++j) w[j] = w4[j];  // (every thread: no branch between the loads in flight)
+            }
+            __syncthreads();
+            if (half == 0) PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 6);
+            if (l < L && live) {  // the chain runs over d in order, four elements per LDS read
+                const float *c = cs + (size_t)l * kTtStride;
+                const float *qq4 = qrow + half * kTtHalf;
+#pragma unroll 4
+                for (int d4 = 0; d4 < kParts; ++d4) {
+                    const float4 cc = *reinterpret_cast<const float4 *>(c + 4 * d4);
+                    const float4 qq = *reinterpret_cast<const float4 *>(qq4 + 4 * d4);
+                    score = __builtin_fmaf(qq.x, cc.x, score);
+                    score = __builtin_fmaf(qq.y, cc.y, score);
+                    score = __builtin_fmaf(qq.z, cc.z, score);
+                    score = __builtin_fmaf(qq.w, cc.w, score);
+                }
+            }
+            __syncthreads();
+        };
+        run_half(0, a0, a1, a2, a3, a4, a5, a6, a7);  // (its first barrier also publishes the normalised row)
+        run_half(1, b0, b1, b2, b3, b4, b5, b6, b7);
+        const float qn = qn_s;
+        if (l < L) {
+            ls_s[l] = score;
+            p.list_scores[((size_t)bh * L + l) * GP + g] = score;
+        }
+        PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 7);
+        if (lut_thread) pq_table();  // (the caller has a barrier before the tables' first use)
+        return qn;
+    };
+    sample_thresh_body<R, 4>(a, g, bh, t, smem, blockIdx.x, tables);  // (short batches: the centroids fill the registers)
 }
 
 
@@ -885,6 +1094,32 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
     else if (a.s_cap <= 16 * kSelThreads) hipLaunchKernelGGL(sample_thresh_kernel<16>, grid, block, lds, stream, a);
     else hipLaunchKernelGGL(sample_thresh_kernel<kSampleRegsMax>, grid, block, lds, stream, a);
     return check_launch("sample_thresh");
+}
+
+// Whether the tables and the threshold estimate of a step share one launch: no append, every
+// row's workgroup on a compute unit of its own (it fills one), and sample and lists within what
+// the kernel is compiled for.
+bool tables_thresh_fits(int streams, int GP, int L, int64_t s_cap) {
+    const int rounds = (streams + kXcdCount - 1) / kXcdCount;
+    return rounds * kXcdCount * GP <= 256 && L <= kTtLists && s_cap <= 8 * kSelThreads;
+}
+
+int launch_tables_thresh(TablesArgs p, int q_dtype, SampleArgs a, hipStream_t stream) {
+    PQHSA_REQUIRE(tables_thresh_fits(p.streams, a.GP, a.L, a.s_cap), "tables_thresh: shape outside the kernel's range");
+    PQHSA_REQUIRE(p.q && p.coarse && p.codebooks && p.qnorm && p.lut && p.list_scores, "tables_thresh: NULL argument");
+    const int rounds = (p.streams + kXcdCount - 1) / kXcdCount;
+    dim3 grid(rounds * kXcdCount * a.GP), block(kSelThreads);
+    const size_t lds = (size_t)((kM * kCodes + a.L + 3) & ~3) * 4 + (size_t)kTtLists * kTtStride * 4;
+    const bool small = a.s_cap <= 4 * kSelThreads;
+#define PQHSA_TT(DT_, R_)                                                                           \
+    do {                                                                                            \
+        const int rc = raise_lds_limit((const void *)tables_thresh_kernel<DT_, R_>, lds, "tables_thresh"); \
+        if (rc) return rc;                                                                          \
+        hipLaunchKernelGGL((tables_thresh_kernel<DT_, R_>), grid, block, lds, stream, p, a);        \
+    } while (0)
+    PQHSA_DISPATCH_DTYPE(q_dtype, if (small) PQHSA_TT(DT, 4); else PQHSA_TT(DT, 8));
+#undef PQHSA_TT
+    return check_launch("tables_thresh");
 }
 
 int launch_select_final(SelectArgs a, int streams, hipStream_t stream) {
@@ -1378,11 +1613,9 @@ int64_t decode_expected_candidates(const pqhsa_index *index, int64_t n_max, cons
     return (int64_t)((ceil(x * x) + 1.0) * 1.125 * ((double)n_max / (ns > 1.0 ? ns : 1.0)) * 1.12) + 64;
 }
 
-// threshold per row from the sampled keys (and, in a step that appends, the rest of the append);
-// thr_key is two rows long: the thresholds, then the largest sampled keys
-int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnorm, const float *lut,
-                      const float *list_scores, float scale, const pqhsa_select *select, uint32_t *thr_key,
-                      int32_t *k_row, float *ref_val, const AppendFinish *append, hipStream_t stream) {
+static SampleArgs decode_sample_args(const pqhsa_index *index, int G, int GP, const float *qnorm, const float *lut,
+                                     const float *list_scores, float scale, const pqhsa_select *select,
+                                     uint32_t *thr_key, int32_t *k_row, float *ref_val) {
     const int streams = index->batch * index->kv_heads;
     SampleArgs sa = {};
     sa.codes = index->s_codes; sa.list_ids = index->s_list_ids; sa.norms = index->s_norms; sa.s_cap = index->s_cap;
@@ -1390,9 +1623,36 @@ int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnor
     sa.qnorm = qnorm; sa.lut = lut; sa.list_scores = list_scores; sa.scale = scale;
     sa.L = index->num_lists; sa.GP = GP; sa.G = G; sa.fraction = select->fraction; sa.topk = select->topk;
     sa.k_cap = select->k_cap;
-    if (append) sa.append = *append;
     sa.thr_key = thr_key; sa.hi_key = thr_key + (size_t)streams * GP; sa.k_row = k_row; sa.ref_val = ref_val;
-    return launch_sample_thresh(sa, streams, stream);
+    return sa;
+}
+
+// threshold per row from the sampled keys (and, in a step that appends, the rest of the append);
+// thr_key is two rows long: the thresholds, then the largest sampled keys
+int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnorm, const float *lut,
+                      const float *list_scores, float scale, const pqhsa_select *select, uint32_t *thr_key,
+                      int32_t *k_row, float *ref_val, const AppendFinish *append, hipStream_t stream) {
+    SampleArgs sa = decode_sample_args(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val);
+    if (append) sa.append = *append;
+    return launch_sample_thresh(sa, index->batch * index->kv_heads, stream);
+}
+
+bool decode_tables_thresh_fits(const pqhsa_index *index, int G) {
+    return tables_thresh_fits(index->batch * index->kv_heads, padded_groups(G), index->num_lists, index->s_cap);
+}
+
+// the tables of every query row and its threshold in one launch (a step without an append whose
+// shape decode_tables_thresh_fits accepts); clears zero_words words at zero_base as lut_build does
+int decode_tables_thresholds(const void *q, int q_dtype, const pqhsa_index *index, int G, int GP, float eps, float *qnorm,
+                             float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, float scale,
+                             const pqhsa_select *select, uint32_t *thr_key, int32_t *k_row, float *ref_val,
+                             hipStream_t stream) {
+    const SampleArgs sa = decode_sample_args(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val);
+    TablesArgs p = {};
+    p.q = static_cast<const char *>(q); p.coarse = index->coarse; p.codebooks = index->codebooks; p.eps = eps;
+    p.qnorm = qnorm; p.lut = lut; p.list_scores = list_scores; p.zero_base = zero_base; p.zero_words = zero_words;
+    p.streams = index->batch * index->kv_heads;
+    return launch_tables_thresh(p, q_dtype, sa, stream);
 }
 
 bool decode_packs_records(const pqhsa_index *index) {
@@ -1424,10 +1684,12 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        uint32_t *thr_key, int32_t *k_row, float *ref_val, void *pairs,
                        uint16_t *aux, int64_t emit_cap, float *mass, uint32_t *rescans,
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt, const AppendFinish *append,
-                       uint32_t *share_map, int64_t share_stride, hipStream_t stream) {
+                       uint32_t *share_map, int64_t share_stride, bool thresholds_known, hipStream_t stream) {
     const int streams = index->batch * index->kv_heads;
-    // 1. threshold per row from the sampled keys
-    int rc = decode_thresholds(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val, append, stream);
+    // 1. threshold per row from the sampled keys (unless the launch that built the tables has left them)
+    int rc = thresholds_known ? PQHSA_OK
+                              : decode_thresholds(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row,
+                                                  ref_val, append, stream);
     if (rc) return rc;
     uint32_t *hi_key = thr_key + (size_t)streams * GP;
     profile_mark(kProfEmit, stream);

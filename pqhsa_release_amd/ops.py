@@ -535,7 +535,8 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
                 seq_lens: torch.Tensor, *, sink: int, full_max: int, fraction: float | None, topk: int,
                 scale: float, workspace: DecodeWorkspace, eps: float = EPS, n_max: int | None = None,
                 append_count: torch.Tensor | None = None, general_path: bool = False,
-                n_mean: int | None = None, one_launch: bool = False, share_rows: bool = False) -> torch.Tensor:
+                n_mean: int | None = None, one_launch: bool = False, share_rows: bool = False,
+                separate_tables: bool = False) -> torch.Tensor:
     """One PQ-HSA decode-attention step for the whole batch; the result is written to ``out``.
     ``n_mean`` (default: the index's host-side mean key count) is the hint that sizes the scan's tiles
     for ragged batches; results do not depend on it.
@@ -545,6 +546,8 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     about one length, GQA groups of 3 to 8; same results, measured slower than the three launches).
     ``share_rows`` asks for one fetch per KV head of a K/V row that several query rows of a GQA group
     selected (``PQHSA_SELECT_SHARE_ROWS``: groups of 2 to 8; same results, measured slower).
+    ``separate_tables`` keeps the table building and the threshold estimate of a step as two launches
+    where they would share one (``PQHSA_SELECT_SEPARATE_TABLES``; same results).
     With ``append_count`` (device int32 [B]) the step first appends one key to every sequence whose
     entry is positive (``pqhsa_append_decode_step``): ``n_max`` must count the appended key and the
     caller calls ``index.note_appended`` afterwards."""
@@ -561,7 +564,8 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
     sel.topk = int(topk)
     sel.k_cap = workspace.k_cap
     sel.flags = ((_lib.SELECT_GENERAL_PATH if general_path else 0) | (_lib.SELECT_ONE_LAUNCH if one_launch else 0)
-                 | (_lib.SELECT_SHARE_ROWS if share_rows else 0))
+                 | (_lib.SELECT_SHARE_ROWS if share_rows else 0)
+                 | (_lib.SELECT_SEPARATE_TABLES if separate_tables else 0))
     sel.n_mean = index.n_mean if n_mean is None else max(0, min(int(n_mean), 2**31 - 1))
     n_max = index.n_max if n_max is None else int(n_max)
     args = (q.data_ptr(), dtype_code(q.dtype), out.data_ptr(), kv.ref(), index.ref(), groups, seq_lens.data_ptr(),
@@ -578,14 +582,16 @@ def decode_step(q: torch.Tensor, out: torch.Tensor, kv: KvSource, index: DeviceI
 
 
 def decode_step_launches(index: DeviceIndex, groups: int, workspace: DecodeWorkspace, *, n_max: int | None = None,
-                         appending: bool = False, general_path: bool = False, one_launch: bool = False) -> int:
+                         appending: bool = False, general_path: bool = False, one_launch: bool = False,
+                         separate_tables: bool = False) -> int:
     """Kernel launches ``decode_step`` makes for a step of this shape: 1 when the short-context
-    kernel serves it, 3 when scan, selection and attention share a launch, else 5
-    (``pqhsa_decode_step_launches``).  No GPU work."""
+    kernel serves it, 3 when scan, selection and attention share a launch, 4 when the tables and the
+    threshold estimate do, else 5 (``pqhsa_decode_step_launches``).  No GPU work."""
     sel = Select()
     sel.k_cap = workspace.k_cap
     sel.n_mean = index.n_mean
-    sel.flags = (_lib.SELECT_GENERAL_PATH if general_path else 0) | (_lib.SELECT_ONE_LAUNCH if one_launch else 0)
+    sel.flags = ((_lib.SELECT_GENERAL_PATH if general_path else 0) | (_lib.SELECT_ONE_LAUNCH if one_launch else 0)
+                 | (_lib.SELECT_SEPARATE_TABLES if separate_tables else 0))
     n_max = index.n_max if n_max is None else int(n_max)
     return int(_lib.load().pqhsa_decode_step_launches(index.ref(), groups, n_max, ctypes.byref(sel), int(appending)))
 
@@ -601,7 +607,8 @@ class DecodeCall:
     def __init__(self, q, out, kv: KvSource, index: DeviceIndex, groups: int, seq_lens, *, sink: int,
                  full_max: int, fraction: float | None, topk: int, scale: float, workspace: DecodeWorkspace,
                  eps: float = EPS, n_max: int | None = None, append_count: torch.Tensor | None = None,
-                 general_path: bool = False, one_launch: bool = False, share_rows: bool = False, flags: int = 0) -> None:
+                 general_path: bool = False, one_launch: bool = False, share_rows: bool = False,
+                 separate_tables: bool = False, flags: int = 0) -> None:
         _need_cuda(q, out, seq_lens)
         if append_count is not None and (append_count.dtype != torch.int32 or append_count.numel() != index.batch
                                          or not append_count.is_cuda):
@@ -619,7 +626,8 @@ class DecodeCall:
         self._sel.topk = int(topk)
         self._sel.k_cap = workspace.k_cap
         self._sel.flags = (int(flags) | (_lib.SELECT_GENERAL_PATH if general_path else 0)
-                           | (_lib.SELECT_ONE_LAUNCH if one_launch else 0) | (_lib.SELECT_SHARE_ROWS if share_rows else 0))
+                           | (_lib.SELECT_ONE_LAUNCH if one_launch else 0) | (_lib.SELECT_SHARE_ROWS if share_rows else 0)
+                           | (_lib.SELECT_SEPARATE_TABLES if separate_tables else 0))
         self._sel.n_mean = index.n_mean
         self._keep = (q, out, kv, index, seq_lens, workspace, append_count)
         self.n_max = index.n_max if n_max is None else int(n_max)

@@ -13,7 +13,8 @@ The marks (slot numbers as printed):
   lut     0 start, 1 query rows loaded, 2 rows normalised, 3 centroid tile staged (tables written
           for the table block), 4 end
   sample  0 start, 1 tables and first sampled keys loaded, 2 sampled keys scored, 3 smallest and
-          largest key known, 4 threshold found (end)
+          largest key known, 4 threshold found (end); where the launch also builds the tables (no
+          lut launch then): 5 query row normalised, 6 first 256 centroids staged, 7 list scores done
   scan    0 start, 1 tables staged, 2 last window scored, 3 candidates and per-list sums flushed (end)
   select  0 start, 1 candidates requested and LDS cleared, 2 histogram of the keys built, 3 k-th key
           found and ties ranked, 4 output slots assigned, 5 winners and losers' weights written, 6 end
@@ -70,6 +71,7 @@ def main():
             print(f"== {name}: no marks (the kernel did not run at this configuration)")
             continue
         used = [s for s in range(SLOTS) if (a[:, s] != 0).any()]
+        used.sort(key=lambda s: np.median(a[:, s][a[:, s] != 0]))  # (in the order the workgroups pass them)
         rel = (a - a[:, 0].min()) / 100.0
         print(f"== {name} (cfg {args.config}): {len(a)} workgroups; first start to last end {rel[:, used].max():.2f} us")
         print("| mark | workgroups | earliest | 10 % | median | 90 % | latest |")

@@ -55,78 +55,50 @@ def test_launch_count_follows_the_short_context_rule():
 
     index.n_cap = 1 << 18
     assert launches(4, 16384) == 1
-    assert launches(4, 16385) == 5            # more keys than a workgroup holds in registers
+    assert launches(4, 16385) == 4            # more keys than a workgroup holds in registers
     assert launches(4, 8192, appending=1) == 5
     assert launches(16, 8192) == 1 and launches(16, 8192) == launches(16, 1)
     index.batch = 3                           # 3 * 8 * 16 query rows > 256
     assert launches(16, 8192) == 5
     index.batch = 1
     sel.flags = _lib.SELECT_GENERAL_PATH
-    assert launches(4, 8192) == 5
+    assert launches(4, 8192) == 4
     sel.flags, sel.k_cap = 0, 2049
+    assert launches(4, 8192) == 4
+    # tables and threshold estimate in one launch: unless the caller keeps them apart, for steps
+    # without an append whose query rows (streams padded to a multiple of 8) each get a compute
+    # unit, with at most 512 lists and 8 192 sampled keys per stream
+    sel.flags = _lib.SELECT_SEPARATE_TABLES
     assert launches(4, 8192) == 5
+    sel.flags = 0
+    index.batch = 9                           # 72 streams x 4 rows > 256
+    assert launches(4, 20000) == 5
+    index.batch = 7                           # 56 streams x 4 rows
+    assert launches(4, 20000) == 4 and launches(4, 20000, appending=1) == 5
+    index.batch, index.kv_heads = 7, 9        # 63 streams, padded to 64: 256 rows
+    assert launches(4, 20000) == 4 and launches(5, 20000) == 5
+    index.batch, index.kv_heads = 1, 8
+    index.num_lists = 513
+    assert launches(4, 20000) == 5
+    index.num_lists, index.s_cap = 512, 8200
+    assert launches(4, 20000) == 5
+    index.s_cap = 8192
+    assert launches(4, 20000) == 4
     # scan + selection + attention in one launch: only when asked for, and only for shapes it serves
     sel.flags = _lib.SELECT_ONE_LAUNCH
     assert launches(4, 20000) == 3 and launches(7, 20000) == 3
-    assert launches(4, 8192) == 1 and launches(2, 20000) == 5 and launches(16, 20000) == 5
-    index.batch, sel.n_mean = 4, 0            # several sequences of unknown lengths
-    assert launches(4, 20000) == 5
-    sel.n_mean = 19000                        # ... of about one length
-    assert launches(4, 20000) == 3
-    sel.n_mean = 9000
-    assert launches(4, 20000) == 5
-    index.n_cap = (1 << 20) + 8               # stored positions no longer fit a candidate record's 20 bits
-    index.batch, sel.n_mean = 1, 0
-    assert launches(4, 20000) == 5
-
-
-def test_struct_layouts_match_the_header():
-    import ctypes
-
-    # sizes implied by include/pqhsa.h on LP64: pointers and int64 8-byte aligned
-    assert ctypes.sizeof(_lib.KvView) == 8 + 8 + 4 + 4 + 8 * 4 + 4 + 4 + 8
-    assert ctypes.sizeof(_lib.Index) == 15 * 8 + 2 * 8 + 4 * 3 + 4
-    assert ctypes.sizeof(_lib.Select) == 24
-
-
-def test_launch_count_follows_the_short_context_rule():
-    import ctypes
-
-    lib = _lib.load()
-    index, sel = _lib.Index(), _lib.Select()
-    index.batch, index.kv_heads, index.num_lists = 1, 8, 512
-    sel.k_cap = 328
-
-    def launches(groups, n_max, appending=0):
-        return lib.pqhsa_decode_step_launches(ctypes.byref(index), groups, n_max, ctypes.byref(sel), appending)
-
-    index.n_cap = 1 << 18
-    assert launches(4, 16384) == 1
-    assert launches(4, 16385) == 5            # more keys than a workgroup holds in registers
-    assert launches(4, 8192, appending=1) == 5
-    assert launches(16, 8192) == 1 and launches(16, 8192) == launches(16, 1)
-    index.batch = 3                           # 3 * 8 * 16 query rows > 256
-    assert launches(16, 8192) == 5
-    index.batch = 1
-    sel.flags = _lib.SELECT_GENERAL_PATH
-    assert launches(4, 8192) == 5
-    sel.flags, sel.k_cap = 0, 2049
-    assert launches(4, 8192) == 5
-    # scan + selection + attention in one launch: only when asked for, and only for shapes it serves
-    sel.flags = _lib.SELECT_ONE_LAUNCH
-    assert launches(4, 20000) == 3 and launches(7, 20000) == 3
-    assert launches(4, 8192) == 3 and launches(2, 20000) == 5 and launches(16, 20000) == 5
+    assert launches(4, 8192) == 3 and launches(2, 20000) == 4 and launches(16, 20000) == 4
     sel.k_cap = 328
     assert launches(4, 8192) == 1             # (the short-context kernel comes first)
     index.batch, sel.n_mean = 4, 0            # several sequences of unknown lengths
-    assert launches(4, 20000) == 5
+    assert launches(4, 20000) == 4
     sel.n_mean = 19000                        # ... of about one length
     assert launches(4, 20000) == 3
     sel.n_mean = 9000
-    assert launches(4, 20000) == 5
+    assert launches(4, 20000) == 4
     index.n_cap = (1 << 20) + 8               # stored positions no longer fit a candidate record's 20 bits
     index.batch, sel.n_mean = 1, 0
-    assert launches(4, 20000) == 5
+    assert launches(4, 20000) == 4
 
 
 def test_short_context_rule_counts_the_whole_lds_footprint():

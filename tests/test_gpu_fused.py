@@ -42,7 +42,7 @@ def test_fused_step_matches_oracle_and_separate_launches(case):
     k_cap = ops.resolve_topk(p.n_max, case["fraction"], 0)
     ws = ops.DecodeWorkspace(idx, p.G, k_cap)
     assert ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 3
-    assert ops.decode_step_launches(idx, p.G, ws, general_path=True) == 5
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True, separate_tables=True) == 5
     q = p.q_tensor().float()
     tol = 1e-4 if case["dtype"] == torch.float32 else 2e-3
     results = {}

@@ -492,16 +492,21 @@ def test_missing_or_bad_arguments_fail_loudly():
 def _path(general_path):
     """Keyword arguments that pick the form of the step: False = the default (one kernel for short
     contexts), True = the general path, "fused" = the general path with scan, selection and
-    attention in one launch (where the shape allows; else the flag changes nothing)."""
-    return dict(general_path=bool(general_path), one_launch=general_path == "fused")
+    attention in one launch (where the shape allows; else the flag changes nothing), "apart" = the
+    general path with the tables and the threshold estimate as two launches."""
+    return dict(general_path=bool(general_path), one_launch=general_path == "fused",
+                separate_tables=general_path == "apart")
 
 
 def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
     """(The tests that use this are about the general path's estimate, candidate area and layouts:
-    both of its forms are run, the three launches and the one-launch scan + selection + attention.)"""
+    every form of it that the shape allows is run: tables and thresholds in one launch or two, and
+    the one-launch scan + selection + attention.)"""
     runs = 1
     if general_path is True and ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 3:
         runs += _check_step(p, idx, kv, ws, fraction, tol, "fused")
+    if general_path is True and ops.decode_step_launches(idx, p.G, ws, general_path=True) == 4:
+        runs += _check_step(p, idx, kv, ws, fraction, tol, "apart")
     q = p.q_tensor()
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
     ws.topk_idx.fill_(-1)
@@ -1127,6 +1132,61 @@ def test_topk_radix_many_candidates_selected_from_memory():
         assert np.array_equal(val[r, : k[r]], x[r, got], equal_nan=True), r
 
 
+TABLES_CASES = [
+    # query rows of a padded group, list counts that end inside a tile / a phase, streams that do not fill a round of 8
+    dict(lens=[20000], heads=2, groups=3, lists=64, dtype=torch.bfloat16),
+    dict(lens=[17000, 9000, 30000], heads=3, groups=1, lists=200, dtype=torch.float16),
+    dict(lens=[18000], heads=1, groups=7, lists=300, dtype=torch.float32),
+    dict(lens=[17000, 17500], heads=4, groups=4, lists=512, dtype=torch.bfloat16),
+    dict(lens=[20000], heads=1, groups=16, lists=16, dtype=torch.bfloat16),
+    dict(lens=[2000, 700, 60, 1500], heads=2, groups=2, lists=40, dtype=torch.float32),   # (one sequence without indexed keys)
+]
+
+
+@pytest.mark.parametrize("case", TABLES_CASES, ids=[str(i) for i in range(len(TABLES_CASES))])
+def test_tables_and_thresholds_in_one_launch_match_the_two_launches(case):
+    """A step without an append builds each query row's tables inside the row's threshold
+    workgroup (four launches); the same step with the two kept apart (five) must leave the same
+    tables and thresholds to the bit -- seen through the number of candidates every row's scan
+    keeps -- and both must agree with the oracle."""
+    dev = _cuda()
+    p = Problem(lens=case["lens"], heads=case["heads"], groups=case["groups"], lists=case["lists"],
+                dtype=case["dtype"], seed=131)
+    idx = p.device_index(dev)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True) == 4
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True, separate_tables=True) == 5
+    q = p.q_tensor()
+    # (the output has the query's type: half an ulp of it on top of the arithmetic's own tolerance)
+    half_ulp = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[case["dtype"]]
+    tol = 1e-4 if case["dtype"] == torch.float32 else 2e-3
+    seen = {}
+    for apart in (True, False, False):
+        out = torch.full_like(q, float("nan"))
+        ws.topk_idx.fill_(-1)
+        ws.topk_cnt.fill_(-1)
+        ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.03,
+                        topk=0, scale=SCALE, workspace=ws, general_path=True, separate_tables=apart)
+        torch.cuda.synchronize()
+        counts = ws.candidate_counts().cpu().numpy().copy()
+        tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
+        o = out.float().cpu().numpy().reshape(p.B, p.H, p.G, DIM)
+        if apart:
+            seen = dict(counts=counts, out=o)
+        else:
+            assert np.array_equal(counts, seen["counts"])
+            assert bool((np.abs(o - seen["out"]) <= 1e-5 + 2.0 * half_ulp * np.abs(o)).all())
+        for (b, h) in p.index:
+            if p.n(b) == 0:
+                continue
+            want_out, want_idx, _ = p.oracle_step(b, h, 0.03)
+            k = want_idx.shape[1]
+            for g in range(p.G):
+                assert np.array_equal(np.sort(tidx[b, h, g, :k]), np.sort(want_idx[g])), (apart, b, h, g)
+            assert bool((np.abs(o[b, h] - want_out) <= tol + half_ulp * np.abs(want_out)).all()), (apart, b, h)
+
+
 def test_event_log_counts_steps_and_samples_them():
     """The per-kernel event log of the decode step: every step logged, one kernel only, and one
     step in three; the number of logged steps and which kernels carry a time."""
@@ -1142,10 +1202,11 @@ def test_event_log_counts_steps_and_samples_them():
     q = p.q_tensor()
     out = torch.full_like(q, float("nan"))  # a row no workgroup folds would stay NaN
 
-    def steps(count):
+    def steps(count, separate_tables=True):
         for _ in range(count):
             ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local,
-                            fraction=0.02, topk=0, scale=SCALE, workspace=ws, general_path=True)
+                            fraction=0.02, topk=0, scale=SCALE, workspace=ws, general_path=True,
+                            separate_tables=separate_tables)
 
     def collect():
         kms = (ctypes.c_float * 5)()
@@ -1157,6 +1218,12 @@ def test_event_log_counts_steps_and_samples_them():
     steps(5)
     seen, kms = collect()
     assert seen == 5 and all(0.0 < v < 50.0 for v in kms), (seen, kms)
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True) == 4
+    _lib.check(lib.pqhsa_profile_enable(16), "enable")
+    steps(4, separate_tables=False)                # tables and thresholds in one launch: booked under the first slot
+    seen, merged = collect()
+    assert seen == 4 and all(0.0 < v < 50.0 for i, v in enumerate(merged) if i != 1), (seen, merged)
+    assert 0.0 <= merged[1] < kms[1], (merged, kms)   # (an empty slot: the cost of recording an event)
     _lib.check(lib.pqhsa_profile_enable(16), "enable")
     _lib.check(lib.pqhsa_profile_only(4), "only")
     _lib.check(lib.pqhsa_profile_every(3), "every")
@@ -1245,7 +1312,7 @@ def test_candidate_records_of_an_index_with_more_than_a_million_slots_per_sequen
     assert idx.n_cap > (1 << 20)
     kv = ops.kv_contiguous(*p.dense_kv())
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
-    assert ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 5   # (no one-launch form either)
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True, one_launch=True) == 5   # (no one-launch form either, and too large a sample for tables and thresholds in one launch)
     before = ws.rescans()
     assert _check_step(p, idx, kv, ws, 0.03) == 1
     assert ws.rescans() == before
