@@ -27,11 +27,11 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                        int32_t *topk_idx, float *topk_val, int32_t *topk_cnt,
                        const AppendFinish *append, uint32_t *share_map, int64_t share_stride, bool thresholds_known,
                        hipStream_t stream);
-bool decode_tables_thresh_fits(const pqhsa_index *index, int G);
+bool decode_tables_thresh_fits(const pqhsa_index *index, int G, bool appending);
 int decode_tables_thresholds(const void *q, int q_dtype, const pqhsa_index *index, int G, int GP, float eps, float *qnorm,
                              float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, float scale,
                              const pqhsa_select *select, uint32_t *thr_key, int32_t *k_row, float *ref_val,
-                             hipStream_t stream);
+                             const AppendFinish *append, int32_t *n_after, hipStream_t stream);
 bool decode_small_fits(int streams, int G, int64_t n_max, int L, int k_cap);
 int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv, const pqhsa_index *index, int G, int GP,
                  const int32_t *seq_lens, int sink, int64_t n_max, int rows_max, const pqhsa_select *select, float scale,
@@ -160,8 +160,8 @@ extern "C" int32_t pqhsa_decode_step_launches(const pqhsa_index *index, int32_t 
     const bool fused = (select->flags & PQHSA_SELECT_ONE_LAUNCH) &&
                        decode_fused_fits(index->batch, index->kv_heads, G, index->n_cap, n_max, select->n_mean, index->num_lists);
     if (fused) return 3;
-    // tables and thresholds in one launch when nothing is appended and every query row gets a compute unit
-    const bool merged = !appending && !(select->flags & PQHSA_SELECT_SEPARATE_TABLES) && decode_tables_thresh_fits(index, G);
+    // tables and thresholds in one launch when every query row gets a compute unit
+    const bool merged = !(select->flags & PQHSA_SELECT_SEPARATE_TABLES) && decode_tables_thresh_fits(index, G, appending != 0);
     return merged ? PQHSA_PROFILE_KERNELS - 1 : PQHSA_PROFILE_KERNELS;
 }
 
@@ -223,7 +223,7 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     const bool merged = pqhsa_decode_step_launches(index_in, G, n_max, select, append_count != nullptr) == PQHSA_PROFILE_KERNELS - 1;
     if (merged) {  // (the event log books the launch under the table slot)
         rc = decode_tables_thresholds(q, q_dtype, index_in, G, GP, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words, scale,
-                                      select, c.thr_key, c.k_row, c.ref_val, stream);
+                                      select, c.thr_key, c.k_row, c.ref_val, append_count ? &ap : nullptr, c.n_after, stream);
         if (rc) return rc;
         profile_mark(kProfSample, stream);
     } else {

@@ -170,7 +170,9 @@ struct AppendFinish {
     int kv_dtype;
 };
 
-__device__ inline void append_finish(const AppendFinish &f, int bh) {
+// `found`: the caller already holds the nearest centroid's key (squared distance bits above the
+// list id, as the list blocks of the table kernel leave them in f.nearest) and passes it as `best`.
+__device__ inline void append_finish(const AppendFinish &f, int bh, bool found = false, unsigned long long best = ~0ull) {
     __shared__ float xs[kD];
     __shared__ float nrm_s;
     __shared__ int list_s;
@@ -191,9 +193,12 @@ __device__ inline void append_finish(const AppendFinish &f, int bh) {
 #pragma unroll
         for (int e = 0; e < kSub / 4; ++e) cw[e] = w4[e];
     }
-    unsigned long long part = ~0ull;
-    if (tid < f.blocks) part = f.nearest[(size_t)bh * f.blocks + tid];
-    part = wave_min_u64(part, kWave);  // at most 64 list blocks
+    unsigned long long part = best;
+    if (!found) {
+        part = ~0ull;
+        if (tid < f.blocks) part = f.nearest[(size_t)bh * f.blocks + tid];
+        part = wave_min_u64(part, kWave);  // at most 64 list blocks
+    }
     __syncthreads();
     if (tid == 0) {
         float ss = 0.0f;

@@ -490,6 +490,7 @@ struct SampleArgs {
     int32_t *k_row;
     float *ref_val;
     AppendFinish append;       // count != NULL: one more workgroup per stream completes the step's append
+    int counts_before_append;  // n_arr holds the counts from before this step's append (append.count says who appends)
 };
 
 // Standard deviations of the sampling noise by which the expected number of keys above the
@@ -536,7 +537,8 @@ __device__ inline void sample_thresh_body(const SampleArgs &a, const int g, cons
             kn[r] = a.norms[base + p];
         }
     };
-    const int n = a.n_arr[bh / a.n_div];
+    int n = a.n_arr[bh / a.n_div];
+    if (a.counts_before_append && append_wanted(a.append.enc, a.append.count, bh / a.n_div)) ++n;
     const int ns = a.ns_arr[bh / a.n_div];
     float *lut_s = reinterpret_cast<float *>(smem);   // [128]
     float *ls_s = lut_s + kM * kCodes;                // [L]
@@ -667,6 +669,39 @@ constexpr int kTtHalf = kD / 2;             // elements per staged half
 constexpr int kTtStride = kTtHalf + 4;      // floats per staged half centroid (16-byte aligned rows that miss each other's banks)
 constexpr int kXcdCount = 8;
 
+// A stream's centroids on their way through the registers of a workgroup of 1024 threads: both
+// halves are requested at once, 8 loads of 16 bytes per thread and half; load u of a half is float4
+// (tid + 1024 u) of it, which is part i % 16 of list i / 16.  (No branch: what lies past the last
+// list is loaded from the last list's end and never used.  Named values rather than arrays, which
+// the compiler would keep in scratch memory here.)
+struct CentroidHalves {
+    static constexpr int kParts = kTtHalf / 4;  // float4 per half centroid
+    static_assert(kTtLists * kParts == 8 * kSelThreads, "written out for 8 loads per thread and half");
+    float4 a0, a1, a2, a3, a4, a5, a6, a7, b0, b1, b2, b3, b4, b5, b6, b7;
+
+    __device__ __forceinline__ void request(const float4 *c4, int L, int tid) {
+        const int last4 = L * (kD / 4) - 1;
+        auto at = [&](int half, int u) __attribute__((always_inline)) {
+            const int i = tid + u * kSelThreads;
+            return c4[min((i / kParts) * (kD / 4) + half * kParts + i % kParts, last4)];
+        };
+        a0 = at(0, 0); a1 = at(0, 1); a2 = at(0, 2); a3 = at(0, 3); a4 = at(0, 4); a5 = at(0, 5); a6 = at(0, 6); a7 = at(0, 7);
+        b0 = at(1, 0); b1 = at(1, 1); b2 = at(1, 2); b3 = at(1, 3); b4 = at(1, 4); b5 = at(1, 5); b6 = at(1, 6); b7 = at(1, 7);
+    }
+    // this thread's part of one half into cs[kTtLists][kTtStride]; a barrier must follow before the rows are read
+    __device__ __forceinline__ void stage(int half, float *cs, int tid) const {
+        auto put = [&](int u, const float4 &v) __attribute__((always_inline)) {
+            const int i = tid + u * kSelThreads;
+            *reinterpret_cast<float4 *>(cs + (size_t)(i / kParts) * kTtStride + (i % kParts) * 4) = v;
+        };
+        if (half == 0) {
+            put(0, a0); put(1, a1); put(2, a2); put(3, a3); put(4, a4); put(5, a5); put(6, a6); put(7, a7);
+        } else {
+            put(0, b0); put(1, b1); put(2, b2); put(3, b3); put(4, b4); put(5, b5); put(6, b6); put(7, b7);
+        }
+    }
+};
+
 struct TablesArgs {
     const char *q;             // [B, H * G, 128]
     const float *coarse;       // [BH, L, 128]
@@ -676,7 +711,83 @@ struct TablesArgs {
     uint32_t *zero_base;       // scratch that the step's later kernels accumulate into
     size_t zero_words;
     int streams;
+    int thresh_wgs;            // workgroups of the query rows; one more per stream follows in a step that appends
+    AppendFinish append;       // count != NULL: the step appends (nearest is not used: the workgroup finds it itself)
+    int32_t *n_after;          // [B] out: keys per sequence after the append
 };
+
+// The workgroup of stream bh in a step that appends: the sequence's new key (if it has one) is
+// normalised, the nearest of the stream's centroids is found by the chains of the table kernel's
+// list blocks (same order, same bits; the centroids pass through LDS as for the list scores), and
+// append_finish encodes and stores the key.  The new key counts are published for the kernels
+// that follow.  cs: LDS for kTtLists x kTtStride floats; kx: 128 floats.
+__device__ inline void append_role(const TablesArgs &p, const int bh, float *cs, float *kx) {
+    __shared__ unsigned long long near_s[kSelWaves];
+    const AppendFinish &f = p.append;
+    const EncodeArgs &enc = f.enc;
+    const int tid = threadIdx.x, lane = tid % kWave;
+    const int b = bh / enc.H, h = bh % enc.H;
+    const bool appending = append_wanted(enc, f.count, b);
+    if (h == 0 && tid == 0) p.n_after[b] = enc.n_idx[b] + (appending ? 1 : 0);
+    if (!appending) return;
+    // the new key sits at retrieval-local index n_idx[b], the end of the stored keys; every wave
+    // loads elements lane and lane + 64 (the first wave uses them), then the centroids
+    const size_t kesz = f.kv_dtype == PQHSA_F32 ? 4 : 2;
+    const char *krow = enc.kv.k_base + row_offset(enc.kv, b, h, (int64_t)enc.sink + enc.n_idx[b]) * (int64_t)kesz;
+    const float ka = load1_any(f.kv_dtype, krow, lane), kb = load1_any(f.kv_dtype, krow, lane + kWave);
+    __builtin_amdgcn_sched_barrier(0);
+    const int L = enc.L;
+    CentroidHalves ch;
+    ch.request(reinterpret_cast<const float4 *>(enc.coarse + (size_t)bh * L * kD), L, tid);
+    if (tid < kWave) {  // the key's norm: one chain over d in order, as in the encode kernels
+        float ss = 0.0f;
+#pragma unroll
+        for (int d = 0; d < kWave; ++d) {
+            const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ka), d));
+            ss = __builtin_fmaf(x, x, ss);
+        }
+#pragma unroll
+        for (int d = 0; d < kWave; ++d) {
+            const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(kb), d));
+            ss = __builtin_fmaf(x, x, ss);
+        }
+        const float nrm = sqrtf(ss);
+        const float kn = nrm < enc.eps ? enc.eps : nrm;
+        kx[lane] = ka / kn;
+        kx[lane + kWave] = kb / kn;
+    }
+    // squared distance to list l by lane l % 64 of wave l / 64
+    const int l = tid;
+    float d2 = 0.0f;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        ch.stage(half, cs, tid);
+        __syncthreads();  // (the first one also publishes the normalised key)
+        if (l < L) {
+            const float *c = cs + (size_t)l * kTtStride;
+            const float *x4 = kx + half * kTtHalf;
+#pragma unroll 4
+            for (int d4 = 0; d4 < CentroidHalves::kParts; ++d4) {
+                const float4 cc = *reinterpret_cast<const float4 *>(c + 4 * d4);
+                const float4 xx = *reinterpret_cast<const float4 *>(x4 + 4 * d4);
+                float t = xx.x - cc.x; d2 = __builtin_fmaf(t, t, d2);
+                t = xx.y - cc.y; d2 = __builtin_fmaf(t, t, d2);
+                t = xx.z - cc.z; d2 = __builtin_fmaf(t, t, d2);
+                t = xx.w - cc.w; d2 = __builtin_fmaf(t, t, d2);
+            }
+        }
+        __syncthreads();
+    }
+    // its bit pattern orders like the value (>= 0) and the list id breaks ties low
+    unsigned long long key = l < L ? ((unsigned long long)__builtin_bit_cast(uint32_t, d2) << 32) | (uint32_t)l : ~0ull;
+    key = wave_min_u64(key, kWave);
+    if (lane == 0) near_s[tid / kWave] = key;
+    __syncthreads();
+    unsigned long long best = near_s[0];
+#pragma unroll
+    for (int w = 1; w < kSelWaves; ++w) best = near_s[w] < best ? near_s[w] : best;
+    append_finish(f, bh, true, best);
+}
 
 template <int DT, int R>
 __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p, SampleArgs a) {
@@ -685,6 +796,10 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
     __shared__ __align__(16) float qrow[kD];
     __shared__ float qn_s;
     const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= p.thresh_wgs) {
+        append_role(p, (int)blockIdx.x - p.thresh_wgs, reinterpret_cast<float *>(smem), qrow);
+        return;
+    }
     const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
     const int g = slot % a.GP;
     const int bh = (slot / a.GP) * kXcdCount + xcd;
@@ -711,22 +826,8 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
     float *cs = reinterpret_cast<float *>(smem) + ((kM * kCodes + L + 3) & ~3);  // [kTtLists][kTtStride], past the tables
 
     auto tables = [&](float *lut_s, float *ls_s, auto request, auto early) __attribute__((always_inline)) -> float {
-        // both halves of the centroids are requested at once, 8 loads of 16 bytes per thread and half:
-        // load u of a half is float4 (tid + 1024 u) of it, which is part i % 16 of list i / 16
-        // (no branch: what lies past the last list is loaded from the last list's end and never used;
-        // named values rather than arrays, which the compiler would keep in scratch memory here)
-        const float4 *c4 = reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD);
-        constexpr int kParts = kTtHalf / 4;  // float4 per half centroid
-        static_assert(kTtLists * kParts == 8 * kSelThreads, "the halves below are written out for 8 loads per thread");
-        const int last4 = L * (kD / 4) - 1;
-        auto centroid4 = [&](int half, int u) __attribute__((always_inline)) {
-            const int i = tid + u * kSelThreads;
-            return c4[min((i / kParts) * (kD / 4) + half * kParts + i % kParts, last4)];
-        };
-        const float4 a0 = centroid4(0, 0), a1 = centroid4(0, 1), a2 = centroid4(0, 2), a3 = centroid4(0, 3);
-        const float4 a4 = centroid4(0, 4), a5 = centroid4(0, 5), a6 = centroid4(0, 6), a7 = centroid4(0, 7);
-        const float4 b0 = centroid4(1, 0), b1 = centroid4(1, 1), b2 = centroid4(1, 2), b3 = centroid4(1, 3);
-        const float4 b4 = centroid4(1, 4), b5 = centroid4(1, 5), b6 = centroid4(1, 6), b7 = centroid4(1, 7);
+        CentroidHalves ch;
+        ch.request(reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD), L, tid);
         __builtin_amdgcn_sched_barrier(0);
         request();  // (the sampled keys behind the centroids: they are not needed before the tables stand)
 
@@ -782,14 +883,8 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
         // list scores: list l by lane l % 64 of wave l / 64
         const int l = tid;
         float score = 0.0f;
-        auto stage = [&](int u, const float4 &v) __attribute__((always_inline)) {
-            const int i = tid + u * kSelThreads;
-            *reinterpret_cast<float4 *>(cs + (size_t)(i / kParts) * kTtStride + (i % kParts) * 4) = v;
-        };
-        auto run_half = [&](int half, const float4 &v0, const float4 &v1, const float4 &v2, const float4 &v3,
-                            const float4 &v4, const float4 &v5, const float4 &v6, const float4 &v7) __attribute__((always_inline)) {
-            stage(0, v0); stage(1, v1); stage(2, v2); stage(3, v3);
-            stage(4, v4); stage(5, v5); stage(6, v6); stage(7, v7);
+        auto run_half = [&](int half) __attribute__((always_inline)) {
+            ch.stage(half, cs, tid);
             if (half == 0) {
 #pragma unroll
                 for (int j = 0; j < kSub / 4; ++j) w[j] = w4[j];  // (every thread: no branch between the loads in flight)
@@ -800,7 +895,7 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
                 const float *c = cs + (size_t)l * kTtStride;
                 const float *qq4 = qrow + half * kTtHalf;
 #pragma unroll 4
-                for (int d4 = 0; d4 < kParts; ++d4) {
+                for (int d4 = 0; d4 < CentroidHalves::kParts; ++d4) {
                     const float4 cc = *reinterpret_cast<const float4 *>(c + 4 * d4);
                     const float4 qq = *reinterpret_cast<const float4 *>(qq4 + 4 * d4);
                     score = __builtin_fmaf(qq.x, cc.x, score);
@@ -811,8 +906,8 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
             }
             __syncthreads();
         };
-        run_half(0, a0, a1, a2, a3, a4, a5, a6, a7);  // (its first barrier also publishes the normalised row)
-        run_half(1, b0, b1, b2, b3, b4, b5, b6, b7);
+        run_half(0);  // (its first barrier also publishes the normalised row)
+        run_half(1);
         const float qn = qn_s;
         if (l < L) {
             ls_s[l] = score;
@@ -1096,19 +1191,23 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
     return check_launch("sample_thresh");
 }
 
-// Whether the tables and the threshold estimate of a step share one launch: no append, every
-// row's workgroup on a compute unit of its own (it fills one), and sample and lists within what
-// the kernel is compiled for.
-bool tables_thresh_fits(int streams, int GP, int L, int64_t s_cap) {
+// Whether the tables and the threshold estimate of a step share one launch: every row's workgroup
+// (and, in a step that appends, one more per stream) on a compute unit of its own (it fills one),
+// and sample and lists within what the kernel is compiled for.
+bool tables_thresh_fits(int streams, int GP, int L, int64_t s_cap, bool appending) {
     const int rounds = (streams + kXcdCount - 1) / kXcdCount;
-    return rounds * kXcdCount * GP <= 256 && L <= kTtLists && s_cap <= 8 * kSelThreads;
+    return rounds * kXcdCount * GP + (appending ? streams : 0) <= 256 && L <= kTtLists && s_cap <= 8 * kSelThreads;
 }
 
 int launch_tables_thresh(TablesArgs p, int q_dtype, SampleArgs a, hipStream_t stream) {
-    PQHSA_REQUIRE(tables_thresh_fits(p.streams, a.GP, a.L, a.s_cap), "tables_thresh: shape outside the kernel's range");
+    const bool appending = p.append.count != nullptr;
+    PQHSA_REQUIRE(tables_thresh_fits(p.streams, a.GP, a.L, a.s_cap, appending), "tables_thresh: shape outside the kernel's range");
     PQHSA_REQUIRE(p.q && p.coarse && p.codebooks && p.qnorm && p.lut && p.list_scores, "tables_thresh: NULL argument");
+    PQHSA_REQUIRE(!appending || (p.n_after && p.append.enc.L == a.L && p.append.enc.coarse == p.coarse),
+                  "tables_thresh: append arguments do not match the index");
     const int rounds = (p.streams + kXcdCount - 1) / kXcdCount;
-    dim3 grid(rounds * kXcdCount * a.GP), block(kSelThreads);
+    p.thresh_wgs = rounds * kXcdCount * a.GP;
+    dim3 grid(p.thresh_wgs + (appending ? p.streams : 0)), block(kSelThreads);
     const size_t lds = (size_t)((kM * kCodes + a.L + 3) & ~3) * 4 + (size_t)kTtLists * kTtStride * 4;
     const bool small = a.s_cap <= 4 * kSelThreads;
 #define PQHSA_TT(DT_, R_)                                                                           \
@@ -1637,18 +1736,25 @@ int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnor
     return launch_sample_thresh(sa, index->batch * index->kv_heads, stream);
 }
 
-bool decode_tables_thresh_fits(const pqhsa_index *index, int G) {
-    return tables_thresh_fits(index->batch * index->kv_heads, padded_groups(G), index->num_lists, index->s_cap);
+bool decode_tables_thresh_fits(const pqhsa_index *index, int G, bool appending) {
+    return tables_thresh_fits(index->batch * index->kv_heads, padded_groups(G), index->num_lists, index->s_cap, appending);
 }
 
-// the tables of every query row and its threshold in one launch (a step without an append whose
-// shape decode_tables_thresh_fits accepts); clears zero_words words at zero_base as lut_build does
+// the tables of every query row and its threshold in one launch (a step whose shape
+// decode_tables_thresh_fits accepts); clears zero_words words at zero_base as lut_build does.
+// `index` holds the key counts from before the step's append (if any), n_after receives the new ones.
 int decode_tables_thresholds(const void *q, int q_dtype, const pqhsa_index *index, int G, int GP, float eps, float *qnorm,
                              float *lut, float *list_scores, uint32_t *zero_base, size_t zero_words, float scale,
                              const pqhsa_select *select, uint32_t *thr_key, int32_t *k_row, float *ref_val,
-                             hipStream_t stream) {
-    const SampleArgs sa = decode_sample_args(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val);
+                             const AppendFinish *append, int32_t *n_after, hipStream_t stream) {
+    SampleArgs sa = decode_sample_args(index, G, GP, qnorm, lut, list_scores, scale, select, thr_key, k_row, ref_val);
     TablesArgs p = {};
+    if (append) {
+        sa.append = *append;
+        sa.counts_before_append = 1;
+        p.append = *append;
+        p.n_after = n_after;
+    }
     p.q = static_cast<const char *>(q); p.coarse = index->coarse; p.codebooks = index->codebooks; p.eps = eps;
     p.qnorm = qnorm; p.lut = lut; p.list_scores = list_scores; p.zero_base = zero_base; p.zero_words = zero_words;
     p.streams = index->batch * index->kv_heads;

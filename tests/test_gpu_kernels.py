@@ -882,7 +882,12 @@ def test_ragged_batch_tile_hint_changes_no_result(lens, heads):
     # 64 streams x 13 table blocks: the table-building launch gives a block two tiles of lists, and the
     # appended key's nearest list is found over the tiles' answers (a sample of the streams is checked)
     dict(steps=2, lens=[862, 852, 847, 842, 872, 882, 843, 854], heads=8, groups=2, lists=768, every=9),
-], ids=["small", "many_streams"])
+    # the same steps with the tables and the threshold estimate as two launches (the appended key's
+    # nearest list is then found by the table kernel's list blocks, as for "many_streams")
+    dict(steps=5, lens=[1805, 1505], heads=2, groups=4, lists=32, every=1, apart=True),
+    # streams that do not fill a round of eight, a padded group, lists that end inside a staged half
+    dict(steps=3, lens=[1405, 1205, 1100], heads=3, groups=7, lists=300, every=2),
+], ids=["small", "many_streams", "small_two_launches", "ragged_groups"])
 def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
     the launch that builds the tables, attends over the grown index, and leaves the new count in
@@ -905,7 +910,9 @@ def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     one = torch.ones(p.B, dtype=torch.int32, device=dev)
     seq = torch.tensor(lens0, dtype=torch.int32, device=dev)
     call = ops.DecodeCall(q, out, kv, idx, p.G, seq, sink=p.sink, full_max=p.sink + p.local, fraction=frac, topk=0,
-                          scale=SCALE, workspace=ws, append_count=one)
+                          scale=SCALE, workspace=ws, append_count=one, separate_tables=shape.get("apart", False))
+    want_launches = 5 if shape.get("apart") or shape["lists"] > 512 else 4
+    assert ops.decode_step_launches(idx, p.G, ws, appending=True, separate_tables=shape.get("apart", False)) == want_launches
     for t in range(1, steps + 1):
         seq.add_(1)
         call.n_max = max(n0) + t
