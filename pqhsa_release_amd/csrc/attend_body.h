@@ -189,8 +189,8 @@ __device__ inline void fold_row_if_last(const AttendArgs &a, AttendLds &lds, siz
             m = peek(part + tid * kPartWidth);
             ms0 = peek(part + tid * kPartWidth + 2);
         }
-        m = wave_max(m);
-        ms0 = wave_sum(ms0);
+        m = wave_max_all(m);    // (every lane of the first wave is here: no LDS traffic)
+        ms0 = wave_total(ms0);
         if (tid == 0) { head_s[0] = m; head_s[1] = ms0; }
     }
     __syncthreads();

@@ -243,6 +243,19 @@ __device__ inline uint32_t wave_max_u32(uint32_t v) {
     return max(max(r0, r1), max(r2, r3));
 }
 
+// largest value of the wave, returned in every lane
+__device__ inline float wave_max_all(float f) {
+    int v = __float_as_int(f);
+    auto mx = [](int x, int y) { return __float_as_int(fmaxf(__int_as_float(x), __int_as_float(y))); };
+    v = mx(v, dpp_move<kDppXor1>(v));
+    v = mx(v, dpp_move<kDppXor2>(v));
+    v = mx(v, dpp_move<kDppHalfMirror>(v));
+    v = mx(v, dpp_move<kDppMirror>(v));
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(v, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(v, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(v, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(v, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 // sum over the 16 lanes of a row group (one DPP row), returned in each of them
 __device__ inline float group_sum16(float v) {
     v += __int_as_float(dpp_move<kDppXor1>(__float_as_int(v)));

@@ -1559,9 +1559,9 @@ __global__ __launch_bounds__(kSelThreads) void decode_small_kernel(SmallArgs a) 
     __syncthreads();
     if (tid < kWave) {  // one group per lane: row maximum
         float m = red_m[tid];
-        m = wave_max(m);
+        m = wave_max_all(m);
         float ms = tid < kBgParts ? ms_s[tid] : 0.0f;
-        ms = wave_sum(ms);
+        ms = wave_total(ms);
         if (tid == 0) { fin_s[0] = m; fin_s[1] = ms; }
     }
     __syncthreads();
