@@ -538,7 +538,6 @@ __device__ inline void sample_thresh_body(const SampleArgs &a, const int g, cons
         }
     };
     int n = a.n_arr[bh / a.n_div];
-    if (a.counts_before_append && append_wanted(a.append.enc, a.append.count, bh / a.n_div)) ++n;
     const int ns = a.ns_arr[bh / a.n_div];
     float *lut_s = reinterpret_cast<float *>(smem);   // [128]
     float *ls_s = lut_s + kM * kCodes;                // [L]
@@ -546,6 +545,8 @@ __device__ inline void sample_thresh_body(const SampleArgs &a, const int g, cons
     int k = 0;
     double want_d = 0.0;
     auto resolve = [&]() __attribute__((always_inline)) {
+        // (asked here, not where n is loaded: the test's loads would stand before every other request)
+        if (a.counts_before_append && append_wanted(a.append.enc, a.append.count, bh / a.n_div)) ++n;
         // (the device-side count may have moved past what the host sized k_cap for: stay inside it)
         k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
         // expected sampled keys among the top max(k, 1), plus the margin
