@@ -57,6 +57,9 @@ __global__ __launch_bounds__(kScanThreads, GP <= 4 ? 4 : GP == 8 ? 3 : 2) void s
     } else if (a.tile_major) {
         tile = blockIdx.y;
         bh = (int)((blockIdx.x + blockIdx.y) % gridDim.x);
+        // (many tiles of such a launch lie past the end of their stream: they leave before they ask
+        // for anything but the count, so that their slots go to tiles with work at once)
+        if ((int64_t)tile * a.tile_windows * kWaveKeys >= min(a.n_arr[bh / a.n_div], (int)a.n_cap)) return;
     } else {
         tile = blockIdx.x;
         bh = blockIdx.y;

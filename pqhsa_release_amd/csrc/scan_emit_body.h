@@ -63,80 +63,78 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
         int4 pw;
     };
     const size_t base = (size_t)bh * a.n_cap;
-    // window w = stored keys [256 w, 256 w + 256); loads stay inside the arrays whatever the key count
-    auto fetch = [&](int w) {
+    // window w = stored keys [256 w, 256 w + 256).  No branch: a window past the end of the arrays
+    // (only the first request of a workgroup can ask for one, before it knows the key count) is
+    // read from their last four slots and never used.
+    auto fetch = [&](int w) __attribute__((always_inline)) {
         KeyWords k;
         const int64_t i = (int64_t)w * kWaveKeys + lane * kKeysPerThread;
-        k.cw = make_uint4(0, 0, 0, 0); k.lw = make_uint2(0, 0); k.nw = make_float4(0, 0, 0, 0);
+        const int64_t at = min(i, a.n_cap - kKeysPerThread);
+        k.cw = *reinterpret_cast<const uint4 *>(a.codes + base + at);
+        k.lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + at);
+        k.nw = *reinterpret_cast<const float4 *>(a.norms + base + at);
         k.pw = make_int4((int)i, (int)i + 1, (int)i + 2, (int)i + 3);
-        if (i < a.n_cap) {
-            k.cw = *reinterpret_cast<const uint4 *>(a.codes + base + i);
-            k.lw = *reinterpret_cast<const uint2 *>(a.list_ids + base + i);
-            k.nw = *reinterpret_cast<const float4 *>(a.norms + base + i);
-            if (a.pos && !packed) k.pw = *reinterpret_cast<const int4 *>(a.pos + base + i);
-        }
+        if (a.pos && !packed) k.pw = *reinterpret_cast<const int4 *>(a.pos + base + at);  // (uniform)
         return k;
     };
     // the workgroup's tile of windows; wave w takes windows w, w + waves, ... of it
     const int tile_end = (tile + 1) * a.tile_windows;
     int win = tile * a.tile_windows + wave;
-    // A tile past the end of its stream has nothing to do.  In a tile-major launch there are many:
-    // they leave before they ask for anything but the count, so that their slots go to tiles with
-    // work at once.  Otherwise the first window is requested before the count is
-    // looked at, and a tile with work never waits for the count alone.
-    const int n = min(a.n_arr[bh / a.n_div], (int)a.n_cap);
-    const bool idle = (int64_t)tile * a.tile_windows * kWaveKeys >= n;
-    if (a.tile_major && idle) return;  // (uniform over the workgroup)
+    // Everything the workgroup needs before its first window is scored -- the window, the tables,
+    // the rows' thresholds and norms, the key count -- is requested at once: one round trip to
+    // memory, and a tile with work never waits for the count alone.  (A tile past the end of its
+    // stream has nothing to do; the launches that hold many of those let them leave before they
+    // get here, scan_emit_kernel.)
     KeyWords cur = fetch(win);
 
+    // all table loads are requested before the first is stored (no branch: a thread without a
+    // word of its own loads the last one, and does not store it)
+    constexpr int kLutVec = kM * kCodes * GP / 4;
+    constexpr int kLutPer = (kLutVec + TH - 1) / TH;
+    float4 lut_r[kLutPer];
+    const float4 *lut_src = reinterpret_cast<const float4 *>(a.lut + (size_t)bh * kM * kCodes * GP);
+#pragma unroll
+    for (int u = 0; u < kLutPer; ++u) lut_r[u] = lut_src[min(tid + u * TH, kLutVec - 1)];
+    constexpr int kLsPer = GP >= 4 ? 2 : 0;  // (narrower groups copy their list scores word by word below)
+    const float4 *ls4 = reinterpret_cast<const float4 *>(a.list_scores + (size_t)bh * L * GP);
+    const int ls_vec = L * GP / 4;
+    float4 ls_r[kLsPer > 0 ? kLsPer : 1];
+#pragma unroll
+    for (int u = 0; u < kLsPer; ++u) ls_r[u] = ls4[min(tid + u * TH, ls_vec - 1)];
     float qn[GP];
-    {
-        // all table loads are requested before the first is stored
-        constexpr int kLutVec = kM * kCodes * GP / 4;
-        constexpr int kLutPer = (kLutVec + TH - 1) / TH;
-        float4 lut_r[kLutPer];
-        const float4 *src = reinterpret_cast<const float4 *>(a.lut + (size_t)bh * kM * kCodes * GP);
+    uint32_t thr_k[GP];
+    float ref_v[GP];
 #pragma unroll
-        for (int u = 0; u < kLutPer; ++u) {
-            const int i = tid + u * TH;
-            lut_r[u] = i < kLutVec ? src[i] : make_float4(0, 0, 0, 0);
-        }
-        if constexpr (GP >= 4) {
-            const float4 *ls = reinterpret_cast<const float4 *>(a.list_scores + (size_t)bh * L * GP);
-            const int nvec = L * GP / 4;
-            float4 ls_r[2];
+    for (int g = 0; g < GP; ++g) {
+        qn[g] = a.qnorm[(size_t)bh * GP + g];
+        thr_k[g] = a.thr_key ? a.thr_key[(size_t)bh * GP + g] : 0xffffffffu;  // no thresholds: no candidates
+        ref_v[g] = a.ref_val[(size_t)bh * GP + g];
+    }
+    const int n = min(a.n_arr[bh / a.n_div], (int)a.n_cap);
+    // (no branch between the requests and the stores below: behind one, the compiler would move
+    // each load down to its first use and they would go out one after the other; a tile with
+    // nothing to do therefore leaves after the tables are staged, not before)
+    if constexpr (GP >= 4) {
+        // (a thread without a word of its own stores the last word again, the value it loaded: no
+        // branch around a store either, or the compiler moves the load into it)
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int i = tid + u * TH;
-                ls_r[u] = i < nvec ? ls[i] : make_float4(0, 0, 0, 0);
-            }
-            if (idle) return;  // (uniform over the workgroup)
+        for (int u = 0; u < kLsPer; ++u) reinterpret_cast<float4 *>(ls_s)[min(tid + u * TH, ls_vec - 1)] = ls_r[u];
+        for (int i = tid + kLsPer * TH; i < ls_vec; i += TH) reinterpret_cast<float4 *>(ls_s)[i] = ls4[i];
+    } else {
+        const float *ls = a.list_scores + (size_t)bh * L * GP;
+        for (int i = tid; i < L * GP; i += TH) ls_s[i] = ls[i];
+    }
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int i = tid + u * TH;
-                if (i < nvec) reinterpret_cast<float4 *>(ls_s)[i] = ls_r[u];
-            }
-            for (int i = tid + 2 * TH; i < nvec; i += TH) reinterpret_cast<float4 *>(ls_s)[i] = ls[i];
+    for (int u = 0; u < kLutPer; ++u) {
+        const int i = min(tid + u * TH, kLutVec - 1);
+        if constexpr (GP >= 4) {  // word i holds rows 4q .. 4q+3 of entry e: two pair sub-tables
+            const int e = i / (GP / 4), q = i % (GP / 4);
+            float2 *pair = reinterpret_cast<float2 *>(lut_s);
+            pair[(2 * q) * (kM * kCodes) + e] = make_float2(lut_r[u].x, lut_r[u].y);
+            pair[(2 * q + 1) * (kM * kCodes) + e] = make_float2(lut_r[u].z, lut_r[u].w);
         } else {
-            if (idle) return;  // (uniform over the workgroup)
-            const float *ls = a.list_scores + (size_t)bh * L * GP;
-            for (int i = tid; i < L * GP; i += TH) ls_s[i] = ls[i];
+            reinterpret_cast<float4 *>(lut_s)[i] = lut_r[u];
         }
-#pragma unroll
-        for (int u = 0; u < kLutPer; ++u) {
-            const int i = tid + u * TH;
-            if (i >= kLutVec) continue;
-            if constexpr (GP >= 4) {  // word i holds rows 4q .. 4q+3 of entry e: two pair sub-tables
-                const int e = i / (GP / 4), q = i % (GP / 4);
-                float2 *pair = reinterpret_cast<float2 *>(lut_s);
-                pair[(2 * q) * (kM * kCodes) + e] = make_float2(lut_r[u].x, lut_r[u].y);
-                pair[(2 * q + 1) * (kM * kCodes) + e] = make_float2(lut_r[u].z, lut_r[u].w);
-            } else {
-                reinterpret_cast<float4 *>(lut_s)[i] = lut_r[u];
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < GP; ++g) qn[g] = a.qnorm[(size_t)bh * GP + g];
     }
     // A key is a candidate when its logit, as a float, reaches the threshold: the same order as on
     // the 32-bit keys (-0 and +0 compare equal, as their keys do).  Threshold key 0 keeps every key,
@@ -148,8 +146,8 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
     for (int i = tid; i < L * GP; i += TH) mass_s[i] = 0.0f;
 #pragma unroll
     for (int g = 0; g < GP; ++g) {
-        const uint32_t tk = a.thr_key ? a.thr_key[(size_t)bh * GP + g] : 0xffffffffu;  // no thresholds: no candidates
-        const float rv = a.ref_val[(size_t)bh * GP + g];
+        const uint32_t tk = thr_k[g];
+        const float rv = ref_v[g];
         // keys below that of the lowest finite float are not keys of ordered floats: such a
         // threshold keeps every key of the index (its logits are finite)
         thr_f[g] = tk < 0x00800000u ? -3.402823466e38f : key_to_float(tk);
@@ -158,6 +156,7 @@ __device__ inline void scan_emit_body(const ScanArgs &a, const int tile, const i
     }
     __syncthreads();
     PQHSA_SCAN_MARK(trace_wg, 1);
+    if ((int64_t)tile * a.tile_windows * kWaveKeys >= n) return;  // (uniform over the workgroup)
 
     const int nwin = min((n + kWaveKeys - 1) / kWaveKeys, tile_end);
     while (win < nwin) {  // wave-uniform
