@@ -268,12 +268,11 @@ __device__ inline void attend_body(const AttendArgs &a, const int split, const i
     const int start_g = min(split * chunk_g, total_g);
     const int32_t *tk = a.topk_idx + orow * a.k_cap;
     int32_t spec[kSpec];
+    // (no branch around a load anywhere before the first rows are requested: behind one, the loads
+    // go out one after the other; an entry outside the chunk is read from the row's nearest end)
 #pragma unroll
-    for (int u = 0; u < kSpec; ++u) {
-        const int i = tid + u * kAttThreads;
-        const int r = start_g + i;
-        spec[u] = (i < chunk_g && r >= F_g && r < total_g) ? load_shared<FUSED>(tk + (r - F_g)) : 0;
-    }
+    for (int u = 0; u < kSpec; ++u)
+        spec[u] = load_shared<FUSED>(tk + max(0, min(start_g + tid + u * kAttThreads - F_g, (int)a.k_cap - 1)));
     const int len = a.seq_lens[b];
     const int n = a.n_idx[b];
     const int sink_end = min(a.sink, len);
@@ -305,13 +304,12 @@ __device__ inline void attend_body(const AttendArgs &a, const int split, const i
     auto bg_fetch = [&](int first) {
 #pragma unroll
         for (int u = 0; u < kBgU; ++u) {
+            // (a list past the slice is read as the last list of the index, with weight 0)
             const int l = first + bl + u * kBgRows;
-            bv[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            bw0[u] = 0.0f;
-            if (l < l_hi) {
-                bv[u] = *reinterpret_cast<const float4 *>(vb + (size_t)l * kD + bd);
-                if (m0) bw0[u] = load_shared<FUSED>(m0 + (size_t)l * a.mass_l);
-            }
+            const int lc = min(l, a.L - 1);
+            bv[u] = *reinterpret_cast<const float4 *>(vb + (size_t)lc * kD + bd);
+            bw0[u] = m0 ? load_shared<FUSED>(m0 + (size_t)lc * a.mass_l) : 0.0f;  // (uniform)
+            if (l >= l_hi) bw0[u] = 0.0f;
         }
     };
     bg_fetch(l_lo);
@@ -320,20 +318,29 @@ __device__ inline void attend_body(const AttendArgs &a, const int split, const i
     int64_t *off_s = reinterpret_cast<int64_t *>(smem);  // [chunk] element offsets of the rows
     {
         const bool guessed = F == F_g && total == total_g;  // then the chunk is where the guess put it
-        auto resolve = [&](int i, int32_t ahead, bool have) {
+        // position of chunk row i in the sequence: sink, window, or a selected key
+        auto position = [&](int i, int32_t selected) {
             const int r = start + i;
-            int64_t pos;
-            if (r < sink_end) pos = r;
-            else if (r < F) pos = local_start + (r - sink_end);
-            else pos = sink_end + (have ? ahead : load_shared<FUSED>(tk + (r - F)));
+            const int64_t pos = r < sink_end ? r : r < F ? local_start + (r - sink_end) : sink_end + selected;
             // (a selected index is a stored key of the sequence; whatever the array holds, the row stays inside it)
-            pos = max((int64_t)0, min(pos, (int64_t)len - 1));
-            off_s[i] = row_offset(a.kv, b, h, pos);
+            return max((int64_t)0, min(pos, (int64_t)len - 1));
         };
+        if (!guessed) {  // (uniform, rare: the indices are read again from where the chunk really lies)
+#pragma unroll
+            for (int u = 0; u < kSpec; ++u)
+                spec[u] = load_shared<FUSED>(tk + max(0, min(start + tid + u * kAttThreads - F, (int)a.k_cap - 1)));
+        }
+        // the block-table look-ups of this thread's rows go out together (every thread takes them,
+        // a thread past the chunk for a row that exists; only rows of the chunk are stored)
+        int64_t pos[kSpec], off[kSpec];
+#pragma unroll
+        for (int u = 0; u < kSpec; ++u) pos[u] = position(tid + u * kAttThreads, spec[u]);
+        row_offsets<kSpec>(a.kv, b, h, pos, off);
 #pragma unroll
         for (int u = 0; u < kSpec; ++u)
-            if (tid + u * kAttThreads < cnt) resolve(tid + u * kAttThreads, spec[u], guessed);
-        for (int i = tid + kSpec * kAttThreads; i < cnt; i += kAttThreads) resolve(i, 0, false);
+            if (tid + u * kAttThreads < cnt) off_s[tid + u * kAttThreads] = off[u];
+        for (int i = tid + kSpec * kAttThreads; i < cnt; i += kAttThreads)
+            off_s[i] = row_offset(a.kv, b, h, position(i, start + i >= F ? load_shared<FUSED>(tk + (start + i - F)) : 0));
     }
     __syncthreads();
 

@@ -113,6 +113,25 @@ __device__ inline int64_t row_offset(const KvView &v, int b, int h, int64_t pos)
     return (int64_t)b * v.stride_seq + (int64_t)h * v.stride_head + pos * v.stride_tok;
 }
 
+// element offsets of N rows of one stream; in a paged cache the N block-table look-ups go out together
+template <int N>
+__device__ inline void row_offsets(const KvView &v, int b, int h, const int64_t (&pos)[N], int64_t (&off)[N]) {
+    if (v.paged) {
+        int64_t row[N], phys[N];
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const int64_t blk = pos[u] / v.block_size;
+            row[u] = pos[u] - blk * v.block_size;
+            phys[u] = v.block_table[(int64_t)b * v.max_blocks + blk];
+        }
+#pragma unroll
+        for (int u = 0; u < N; ++u) off[u] = phys[u] * v.stride_block + row[u] * v.stride_tok + (int64_t)h * v.stride_head;
+    } else {
+#pragma unroll
+        for (int u = 0; u < N; ++u) off[u] = (int64_t)b * v.stride_seq + (int64_t)h * v.stride_head + pos[u] * v.stride_tok;
+    }
+}
+
 // ---- typed 8-element row slices ---------------------------------------------------------
 // Load elements [8*j, 8*j + 8) of a 128-element row as floats.
 template <int DT>
