@@ -452,8 +452,10 @@ int pqhsa_gather_probe(const pqhsa_kv_view *kv, int32_t B, int32_t H, const int3
  * read back only at collect time (the sync-free event log of the reference,
  * benchmarks/cuda_event_log.py:49-88).  pqhsa_profile_enable creates events for up to
  * max_steps decode steps; pqhsa_profile_collect synchronises the recorded events, writes the
- * average milliseconds of the 5 kernels (lut_build, sample_thresh, scan_emit, select_final,
- * attend) and the number of steps seen, and turns profiling off.
+ * average milliseconds of the 5 slots (lut_build, sample_thresh, scan_emit, select_final,
+ * attend; a step that builds tables and thresholds in one launch books it under the first slot
+ * and leaves the second with the cost of recording an event, see pqhsa_decode_step_launches)
+ * and the number of steps seen, and turns profiling off.
  * pqhsa_profile_only(kernel), called after enable, restricts the log to the two events around
  * one kernel (-1: all), so that a timed run carries two event records per step instead of
  * six; the other entries of kernel_ms are then 0.  pqhsa_profile_every(stride), also after
