@@ -1147,6 +1147,8 @@ TABLES_CASES = [
     dict(lens=[17000, 17500], heads=4, groups=4, lists=512, dtype=torch.bfloat16),
     dict(lens=[20000], heads=1, groups=16, lists=16, dtype=torch.bfloat16),
     dict(lens=[2000, 700, 60, 1500], heads=2, groups=2, lists=40, dtype=torch.float32),   # (one sequence without indexed keys)
+    # room for 170 000 keys per sequence: a sample of more than 4 096 keys per stream, eight per thread
+    dict(lens=[20000, 12000], heads=1, groups=4, lists=128, dtype=torch.bfloat16, spare=150000),
 ]
 
 
@@ -1159,7 +1161,9 @@ def test_tables_and_thresholds_in_one_launch_match_the_two_launches(case):
     dev = _cuda()
     p = Problem(lens=case["lens"], heads=case["heads"], groups=case["groups"], lists=case["lists"],
                 dtype=case["dtype"], seed=131)
-    idx = p.device_index(dev)
+    idx = p.device_index(dev, spare=case.get("spare", 64))
+    if "spare" in case:
+        assert 4096 < idx.s_cap <= 8192
     kv = ops.kv_contiguous(*p.dense_kv())
     ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.03, 0))
     assert ops.decode_step_launches(idx, p.G, ws, general_path=True) == 4
