@@ -27,7 +27,15 @@
  *                        pq_hsa/attention/sparse_attention.py:646 (logit = raw * scale)
  *   pqo_topk             pq_hsa/attention/sparse_attention.py:661-666 (torch.topk), ties at the
  *                        k boundary broken by lowest index
- *   pqo_attend           pq_hsa/attention/sparse_attention.py:887-1013 (centroid, no-details)
+ *   pqo_attend           pq_hsa/attention/sparse_attention.py:887-1013 (centroid, no-details).
+ *                        One deliberate difference in form: the reference sums exp(approximate
+ *                        logit) over ALL indexed keys and takes the selected keys' terms back
+ *                        (:954-967, denom = full + retrieval - old_exact + exact); here the selected
+ *                        keys are left out of the background sums instead.  Equal in exact
+ *                        arithmetic and on every golden vector; they part only where a selected
+ *                        key's approximate logit lies tens of nats above every exact logit
+ *                        (weights of 1 added and taken back beside terms of 1e-15), where the
+ *                        subtraction loses the digits and this form keeps them.
  *   pqo_paged_gather     benchmarks/vllm_backend/paged_kv_fa.py:95-126, 129-156
  */
 #include <math.h>
@@ -192,7 +200,8 @@ int pqo_attend(const float *q, int G, int D, int Dv, const float *K, const float
     if (len < local_start || Dv > PQO_MAX_D) return -1;
     float *fl = (float *)malloc(sizeof(float) * (size_t)(F + k + 1));
     double *mass = (double *)malloc(sizeof(double) * (size_t)L);
-    if (!fl || !mass) return -2;
+    unsigned char *chosen = (unsigned char *)malloc((size_t)(n > 0 ? n : 1));
+    if (!fl || !mass || !chosen) return -2;
     float *xl = fl + F;
     for (int g = 0; g < G; ++g) {
         const float *qg = q + (int64_t)g * D;
@@ -204,7 +213,11 @@ int pqo_attend(const float *q, int G, int D, int Dv, const float *K, const float
             fl[f] = dot_fixed(K + pos * D, qg, D) * scale;
             if (fl[f] > m) m = fl[f];
         }
-        for (int64_t i = 0; i < n; ++i) if (a[i] > m) m = a[i];
+        /* (the reference point is the largest term that is present: exact logits and the
+         * approximate logits of the keys that were not selected) */
+        memset(chosen, 0, (size_t)(n > 0 ? n : 1));
+        for (int t = 0; t < k; ++t) chosen[tk[t]] = 1;
+        for (int64_t i = 0; i < n; ++i) if (!chosen[i] && a[i] > m) m = a[i];
         for (int t = 0; t < k; ++t) {
             xl[t] = dot_fixed(K + ((int64_t)sink_end + tk[t]) * D, qg, D) * scale;
             if (xl[t] > m) m = xl[t];
@@ -219,16 +232,18 @@ int pqo_attend(const float *q, int G, int D, int Dv, const float *K, const float
             den += e;
             for (int d = 0; d < Dv; ++d) acc[d] += e * V[pos * Dv + d];
         }
+        /* the background holds the keys that were NOT selected; a selected key's approximate logit
+         * is left out rather than added and taken back, so that a selected key whose approximate
+         * logit lies far above every exact one (its weight would be 1 against 1e-15) costs no digits */
         for (int64_t i = 0; i < n; ++i) {
+            if (chosen[i]) continue;
             double e = exp((double)a[i] - (double)m);
             den += e;
             mass[list_ids[i]] += e;
         }
         for (int t = 0; t < k; ++t) {
-            double old = exp((double)a[tk[t]] - (double)m);
             double e = exp((double)xl[t] - (double)m);
-            den += e - old;
-            mass[list_ids[tk[t]]] -= old;
+            den += e;
             int64_t pos = (int64_t)sink_end + tk[t];
             for (int d = 0; d < Dv; ++d) acc[d] += e * V[pos * Dv + d];
         }
@@ -239,6 +254,7 @@ int pqo_attend(const float *q, int G, int D, int Dv, const float *K, const float
     }
     free(fl);
     free(mass);
+    free(chosen);
     return 0;
 }
 

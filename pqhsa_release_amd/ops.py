@@ -652,13 +652,18 @@ class DecodeCall:
         if rc:
             _lib.check(rc, "pqhsa_decode_step")
 
-    def capture(self) -> "torch.cuda.CUDAGraph":
+    def capture(self, warm: bool = True) -> "torch.cuda.CUDAGraph":
         """Record the step's kernels into a HIP graph (the graphed steady state of the reference's
         sidecar, benchmarks e2e:6052-6235).  The step clears its scratch with kernels, so the
         graph holds no memset nodes.  A replay runs on the tensors' current contents (new queries
-        are copied into ``q``, counts live in device memory); ``n_max``, ``full_max`` and the
-        launch shapes are those of the capture, so the index must not outgrow them."""
-        self.run()                      # once outside: kernel attributes are set before capture
+        are copied into ``q``, counts and sequence lengths live in device memory); ``n_max``,
+        ``full_max`` and the launch shapes are those of the capture, so the index must not outgrow
+        them: a step that appends is captured with ``n_max`` (and the workspace's ``k_cap``) at the
+        length the sequences will grow to.  ``warm`` runs the step once before the capture, so that
+        the kernels are loaded and their attributes set; a caller whose step appends has run one
+        itself (the warm-up would append a key) and passes ``warm=False``."""
+        if warm:
+            self.run()                  # once outside: kernel attributes are set before capture
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -887,7 +887,10 @@ def test_ragged_batch_tile_hint_changes_no_result(lens, heads):
     dict(steps=5, lens=[1805, 1505], heads=2, groups=4, lists=32, every=1, apart=True),
     # streams that do not fill a round of eight, a padded group, lists that end inside a staged half
     dict(steps=3, lens=[1405, 1205, 1100], heads=3, groups=7, lists=300, every=2),
-], ids=["small", "many_streams", "small_two_launches", "ragged_groups"])
+    # the steps after the first replayed from ONE HIP graph, captured with the launch shapes of the
+    # final length: sequence lengths, key counts and the new keys are all read from device memory
+    dict(steps=5, lens=[1805, 1505], heads=2, groups=4, lists=32, every=1, graph=True),
+], ids=["small", "many_streams", "small_two_launches", "ragged_groups", "graph_replay"])
 def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
     the launch that builds the tables, attends over the grown index, and leaves the new count in
@@ -915,8 +918,19 @@ def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     assert ops.decode_step_launches(idx, p.G, ws, appending=True, separate_tables=shape.get("apart", False)) == want_launches
     for t in range(1, steps + 1):
         seq.add_(1)
-        call.n_max = max(n0) + t
-        call.run()
+        if shape.get("graph"):
+            if t == 1:
+                call.n_max = max(n0) + steps     # the launch shapes of every later step
+                call.run()                       # (eager: loads the kernels; its append is step 1)
+            else:
+                if t == 2:
+                    call.capture(warm=False)     # records a step, runs nothing
+                out.fill_(float("nan"))
+                ws.topk_idx.fill_(-1)
+                call.replay()
+        else:
+            call.n_max = max(n0) + t
+            call.run()
         idx.note_appended([1] * p.B)
         torch.cuda.synchronize()
         assert idx.n_idx.cpu().tolist() == [n + t for n in n0]          # the step advanced the device-side counts

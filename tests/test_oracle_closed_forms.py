@@ -181,6 +181,42 @@ def test_centroid_background_closed_form(which):
     np.testing.assert_allclose(out, expected, rtol=2e-4, atol=2e-5)
 
 
+def test_attend_keeps_its_digits_when_a_selected_key_is_overrated():
+    """The C oracle's attention where the approximate logit of a selected key lies tens of nats
+    above every exact logit (key norms of several hundred make such rows): its weight relative to
+    the largest term present is 1 against exact terms of 1e-15, so a form that adds every
+    approximate weight and takes the selected ones back loses the digits.  The oracle leaves the
+    selected keys out instead; checked against a float64 softmax over exactly the terms present."""
+    rng = np.random.default_rng(5)
+    n, sink, local, dim, lists = 200, 4, 8, 128, 6
+    length = sink + n + local
+    keys = rng.standard_normal((length, dim)).astype(np.float32)
+    values = rng.standard_normal((length, dim)).astype(np.float32)
+    q = rng.standard_normal((2, dim)).astype(np.float32)
+    scale = 1.0
+    list_ids = rng.integers(0, lists, n).astype(np.uint16)
+    vbar = rng.standard_normal((lists, dim)).astype(np.float32)
+    exact = (keys[sink : sink + n].astype(np.float64) @ q.astype(np.float64).T).T * scale
+    logits = (exact + rng.standard_normal((2, n))).astype(np.float32)      # approximate logits: exact + noise ...
+    k = 20
+    topk = np.stack([np.argsort(-logits[g], kind="stable")[:k] for g in range(2)]).astype(np.int32)
+    logits[0, topk[0, 0]] += 40.0                                           # ... and one selected key overrated by 40 nats
+    logits[1, topk[1, :3]] += np.float32(60.0)
+    out = fixed.attend(q, keys, values, sink, logits, topk, list_ids, vbar, scale)
+    for g in range(2):
+        full = list(range(sink)) + list(range(sink + n, length))
+        pos = full + [sink + int(i) for i in topk[g]]
+        le = (keys[pos].astype(np.float64) @ q[g].astype(np.float64)) * scale
+        rest = np.ones(n, bool)
+        rest[topk[g]] = False
+        lb = logits[g].astype(np.float64)[rest]
+        m = max(le.max(), lb.max())
+        we, wb = np.exp(le - m), np.exp(lb - m)
+        mass = np.bincount(list_ids[rest].astype(np.int64), weights=wb, minlength=lists)
+        want = (we @ values[pos].astype(np.float64) + mass @ vbar.astype(np.float64)) / (we.sum() + mass.sum())
+        np.testing.assert_allclose(out[g], want, rtol=1e-5, atol=1e-6)
+
+
 def test_value_centroids_are_segment_means():
     g = torch.Generator().manual_seed(40)
     values = torch.randn(90, 16, generator=g)
