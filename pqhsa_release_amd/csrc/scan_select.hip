@@ -680,14 +680,19 @@ struct CentroidHalves {
     static_assert(kTtLists * kParts == 8 * kSelThreads, "written out for 8 loads per thread and half");
     float4 a0, a1, a2, a3, a4, a5, a6, a7, b0, b1, b2, b3, b4, b5, b6, b7;
 
-    __device__ __forceinline__ void request(const float4 *c4, int L, int tid) {
+    // `half`: 0 or 1, or -1 for both
+    __device__ __forceinline__ void request(const float4 *c4, int L, int tid, int half = -1) {
         const int last4 = L * (kD / 4) - 1;
-        auto at = [&](int half, int u) __attribute__((always_inline)) {
+        auto at = [&](int hf, int u) __attribute__((always_inline)) {
             const int i = tid + u * kSelThreads;
-            return c4[min((i / kParts) * (kD / 4) + half * kParts + i % kParts, last4)];
+            return c4[min((i / kParts) * (kD / 4) + hf * kParts + i % kParts, last4)];
         };
-        a0 = at(0, 0); a1 = at(0, 1); a2 = at(0, 2); a3 = at(0, 3); a4 = at(0, 4); a5 = at(0, 5); a6 = at(0, 6); a7 = at(0, 7);
-        b0 = at(1, 0); b1 = at(1, 1); b2 = at(1, 2); b3 = at(1, 3); b4 = at(1, 4); b5 = at(1, 5); b6 = at(1, 6); b7 = at(1, 7);
+        if (half != 1) {
+            a0 = at(0, 0); a1 = at(0, 1); a2 = at(0, 2); a3 = at(0, 3); a4 = at(0, 4); a5 = at(0, 5); a6 = at(0, 6); a7 = at(0, 7);
+        }
+        if (half != 0) {
+            b0 = at(1, 0); b1 = at(1, 1); b2 = at(1, 2); b3 = at(1, 3); b4 = at(1, 4); b5 = at(1, 5); b6 = at(1, 6); b7 = at(1, 7);
+        }
     }
     // this thread's part of one half into cs[kTtLists][kTtStride]; a barrier must follow before the rows are read
     __device__ __forceinline__ void stage(int half, float *cs, int tid) const {
@@ -828,9 +833,9 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
 
     auto tables = [&](float *lut_s, float *ls_s, auto request, auto early) __attribute__((always_inline)) -> float {
         CentroidHalves ch;
-        ch.request(reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD), L, tid);
+        const float4 *c4 = reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD);
+        ch.request(c4, L, tid, 0);  // (the first halves of all waves before any second half: they are needed first)
         __builtin_amdgcn_sched_barrier(0);
-        request();  // (the sampled keys behind the centroids: they are not needed before the tables stand)
 
         // the row's norm by the first wave alone, while the others wait for their centroids: one
         // chain over d in order, as in lut_build_kernel, every lane running it on the elements read
@@ -857,11 +862,15 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
             }
         }
         PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 5);
-        early();  // (the caller's arithmetic on the stream's key counts, while the centroids travel)
+        ch.request(c4, L, tid, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        request();  // (the sampled keys behind the centroids: they are not needed before the tables stand)
+        early();    // (the caller's arithmetic on the stream's key counts, while the centroids travel)
         clear_scratch();
-        // PQ table: entry (m, c) by thread m * 16 + c of the workgroup's last two waves, after the
-        // list chains (the codebook entry is requested once the first half has left its registers:
-        // requested with the centroids, it would only stand in their way)
+        // PQ table: entry (m, c) by thread m * 16 + c of the workgroup's last two waves, beside the
+        // second half's list chains, which keep only the first eight waves busy (the codebook entry
+        // is requested once the first half has left its registers: requested with the centroids, it
+        // would only stand in their way)
         const bool lut_thread = tid >= kSelThreads - kM * kCodes;
         const int e = lut_thread ? tid - (kSelThreads - kM * kCodes) : 0;
         float4 w[kSub / 4];
@@ -892,6 +901,7 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
             }
             __syncthreads();
             if (half == 0) PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 6);
+            if (half == 1 && lut_thread) pq_table();  // (the last two waves, beside the first eight's chains)
             if (l < L && live) {  // the chain runs over d in order, four elements per LDS read
                 const float *c = cs + (size_t)l * kTtStride;
                 const float *qq4 = qrow + half * kTtHalf;
@@ -915,8 +925,7 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
             p.list_scores[((size_t)bh * L + l) * GP + g] = score;
         }
         PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 7);
-        if (lut_thread) pq_table();  // (the caller has a barrier before the tables' first use)
-        return qn;
+        return qn;  // (the caller has a barrier before the tables' first use)
     };
     sample_thresh_body<R, 4>(a, g, bh, t, smem, blockIdx.x, tables);  // (short batches: the centroids fill the registers)
 }
