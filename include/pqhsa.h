@@ -274,6 +274,27 @@ int pqhsa_lut_scan_mass(const pqhsa_index *index, int32_t G, int32_t n_max, cons
                         float *list_mass, void *stream);
 
 /*
+ * Block statistics of the scan, stand-alone, and their fold: for every query row and every block
+ * of block_keys consecutive STORED keys of its stream (the order of index->codes: list-sorted
+ * once the index is laid out),
+ *   block_max[bh, g, c]    = max over the block's keys of logit            (-inf for an empty block)
+ *   block_expsum[bh, g, c] = sum over the block's keys of exp(logit - block_max[bh, g, c])   (0 ...)
+ * both f32 [BH, G, blocks] with blocks * block_keys >= n_max; no logit is written.  The maxima are
+ * the scan's logits bit for bit, the sums are fp32 sums in no fixed order.
+ * pqhsa_block_reduce folds [rows, blocks] statistics into one pair per row,
+ *   row_max[r] = max_c block_max[r, c],  exp_sum[r] = sum_c block_expsum[r, c] * exp(block_max[r, c] - row_max[r]),
+ * so that row_max + log(exp_sum) is the row's log-sum-exp over all indexed keys (a row without
+ * keys gives -inf and 0).  Counterparts of the block outputs of the reference's pq_scan_only
+ * (pq_hsa/kernels/cuda/pq_fused_h20.cu:2426-2491, written at :324, :389, :461-462) and of its
+ * pq_block_reduce (pq_hsa/kernels/cuda/pq_fused_h20.cu:3094-3145).
+ */
+int pqhsa_lut_scan_stats(const pqhsa_index *index, int32_t G, int32_t n_max, const float *qnorm,
+                         const float *lut, const float *list_scores, float scale, int32_t block_keys,
+                         int32_t blocks, float *block_max, float *block_expsum, void *stream);
+int pqhsa_block_reduce(const float *block_max, const float *block_expsum, int32_t rows, int32_t blocks,
+                       float *row_max, float *exp_sum, void *stream);
+
+/*
  * Exact top-k of each row of a logit matrix [rows, stride] by radix selection on the fp32
  * bit pattern (no sort); ties at the k boundary go to the lowest index; the k winners are
  * written (in no particular order) with their logits.  n[r] and k[r] are per-row device

@@ -133,6 +133,9 @@ SIGNATURES = {
                                              c_void_p]),
     "pqhsa_lut_scan_mass": (ctypes.c_int, [_P(Index), c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
                                            c_void_p, c_void_p]),
+    "pqhsa_lut_scan_stats": (ctypes.c_int, [_P(Index), c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_float, c_int32,
+                                            c_int32, c_void_p, c_void_p, c_void_p]),
+    "pqhsa_block_reduce": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "pqhsa_decode_step_launches": (c_int32, [_P(Index), c_int32, c_int32, _P(Select), c_int32]),
     "pqhsa_gather_probe": (ctypes.c_int, [_P(KvView), c_int32, c_int32, c_void_p, c_int64, c_void_p, c_void_p]),
 }

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libpqhsa.so")
-SOURCES = ["api.hip", "lut_build.hip", "scan_select.hip", "scan_emit.hip", "attend.hip", "encode.hip", "encode_prefilter.hip", "nearest.hip", "decode.hip", "probe.hip", "fused.hip"]
+SOURCES = ["api.hip", "lut_build.hip", "scan_select.hip", "scan_emit.hip", "scan_stats.hip", "attend.hip", "encode.hip", "encode_prefilter.hip", "nearest.hip", "decode.hip", "probe.hip", "fused.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

@@ -471,6 +471,44 @@ def lut_scan_mass(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scal
     return mass
 
 
+def lut_scan_stats(index: DeviceIndex, groups: int, qnorm, lut, list_scores, scale: float, block_keys: int = 4096):
+    """Block statistics of the scan without writing logits (``pqhsa_lut_scan_stats``): ``(block_max,
+    block_expsum)``, both float32 ``[BH, G, blocks]`` over blocks of ``block_keys`` consecutive stored
+    keys; an empty block holds ``-inf`` and 0."""
+    lib = _lib.load()
+    if block_keys < 1:
+        raise ValueError("block_keys must be positive")
+    bh = index.batch * index.kv_heads
+    n_max = int(index.n_max)
+    blocks = max(1, -(-n_max // block_keys))
+    bmax = torch.empty(bh, groups, blocks, dtype=torch.float32, device=index.device)
+    bexp = torch.empty_like(bmax)
+    rc = lib.pqhsa_lut_scan_stats(index.ref(), groups, n_max, qnorm.data_ptr(), lut.data_ptr(), list_scores.data_ptr(),
+                                  float(scale), int(block_keys), blocks, bmax.data_ptr(), bexp.data_ptr(), _stream())
+    _lib.check(rc, "pqhsa_lut_scan_stats")
+    return bmax, bexp
+
+
+def block_reduce(block_max: torch.Tensor, block_expsum: torch.Tensor):
+    """Fold block statistics ``[..., blocks]`` into ``(row_max, exp_sum)`` of shape ``[...]``
+    (``pqhsa_block_reduce``): ``row_max + log(exp_sum)`` is the row's log-sum-exp."""
+    lib = _lib.load()
+    _need_cuda(block_max)
+    _need_cuda(block_expsum)
+    if block_max.shape != block_expsum.shape or block_max.ndim < 1 or block_max.shape[-1] < 1:
+        raise ValueError("block_max and block_expsum must have the same shape [..., blocks >= 1]")
+    if block_max.dtype != torch.float32 or block_expsum.dtype != torch.float32:
+        raise ValueError("block statistics must be float32")
+    bm, be = block_max.contiguous(), block_expsum.contiguous()
+    blocks = bm.shape[-1]
+    rows = bm.numel() // blocks
+    row_max = torch.empty(bm.shape[:-1], dtype=torch.float32, device=bm.device)
+    exp_sum = torch.empty_like(row_max)
+    rc = lib.pqhsa_block_reduce(bm.data_ptr(), be.data_ptr(), rows, blocks, row_max.data_ptr(), exp_sum.data_ptr(), _stream())
+    _lib.check(rc, "pqhsa_block_reduce")
+    return row_max, exp_sum
+
+
 def topk_radix(logits: torch.Tensor, n, k):
     """Exact top-k of each row of ``logits [rows, stride]``; ``n``/``k`` per row.  Returns
     (indices int32 [rows, k_cap], values f32 [rows, k_cap]), the selected keys in no particular order."""

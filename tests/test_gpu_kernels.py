@@ -424,6 +424,66 @@ def test_stand_alone_scan_list_mass_matches_the_logits():
         assert (got[bh, :, p.G:] == 0).all()                          # padded rows of the group carry nothing
 
 
+@pytest.mark.parametrize("lens,groups,lists,block_keys,finalize", [
+    ([5000, 2300], 3, 32, 1024, True),      # ragged: the short stream's last blocks are empty
+    ([3001], 4, 64, 700, True),             # blocks that are no multiple of the workgroup, a ragged last one
+    ([1800, 1800], 1, 16, 4096, False),     # one block per row, index in arrival order
+    ([2600], 7, 40, 256, True),             # padded group
+])
+def test_stand_alone_scan_block_statistics_and_their_fold(lens, groups, lists, block_keys, finalize):
+    """pqhsa_lut_scan_stats + pqhsa_block_reduce: per block of stored keys the largest logit (the
+    oracle's, bit for bit) and the sum of exp(logit - maximum) (against float64 sums over the
+    oracle's logits, 1e-5); folded, the row's maximum and its log-sum-exp over all indexed keys."""
+    dev = _cuda()
+    p = Problem(lens=lens, heads=2, groups=groups, lists=lists, seed=83)
+    idx = p.device_index(dev, finalize=finalize)
+    qnorm, lut, ls = ops.lut_build(p.q_tensor(), idx, p.G)
+    bmax, bexp = ops.lut_scan_stats(idx, p.G, qnorm, lut, ls, SCALE, block_keys=block_keys)
+    row_max, exp_sum = ops.block_reduce(bmax, bexp)
+    torch.cuda.synchronize()
+    blocks = -(-int(idx.n_max) // block_keys)
+    assert tuple(bmax.shape) == (p.B * p.H, p.G, blocks)
+    got_m, got_e = bmax.cpu().numpy(), bexp.cpu().numpy()
+    got_rm, got_es = row_max.cpu().numpy(), exp_sum.cpu().numpy()
+    pos = idx.pos.cpu().numpy()
+    for (b, h) in p.index:
+        bh, n = b * p.H + h, p.n(b)
+        _, _, logits = p.oracle_step(b, h, 0.02)                      # [G, n] by retrieval-local index
+        stored = logits[:, pos[bh, :n]]                               # ... and in the order of the stored keys
+        for c in range(blocks):
+            part = stored[:, c * block_keys : min(n, (c + 1) * block_keys)]
+            if part.shape[1] == 0:
+                assert (got_m[bh, :, c] == -np.inf).all() and (got_e[bh, :, c] == 0).all()
+                continue
+            top = part.max(axis=1)
+            assert np.array_equal(got_m[bh, :, c], top)
+            np.testing.assert_allclose(got_e[bh, :, c], np.exp(part.astype(np.float64) - top[:, None]).sum(axis=1), rtol=1e-5)
+        top = stored.max(axis=1)
+        assert np.array_equal(got_rm[bh], top)
+        lse = top + np.log(np.exp(stored.astype(np.float64) - top[:, None]).sum(axis=1))
+        np.testing.assert_allclose(got_rm[bh] + np.log(got_es[bh].astype(np.float64)), lse, rtol=0, atol=2e-5)
+
+
+def test_block_reduce_of_rows_without_keys_and_of_many_blocks():
+    dev = _cuda()
+    rng = np.random.default_rng(5)
+    bm = rng.standard_normal((6, 1000)).astype(np.float32) * 20
+    be = (rng.random((6, 1000)) * 256 + 1).astype(np.float32)
+    bm[1], be[1] = -np.inf, 0.0                                       # a row without keys
+    bm[2, 3:], be[2, 3:] = -np.inf, 0.0                               # three blocks with keys
+    bm[3, :] = bm[3, 0]                                               # equal maxima
+    row_max, exp_sum = ops.block_reduce(torch.from_numpy(bm).to(dev), torch.from_numpy(be).to(dev))
+    torch.cuda.synchronize()
+    rm, es = row_max.cpu().numpy(), exp_sum.cpu().numpy()
+    want_m = bm.max(axis=1)
+    assert np.array_equal(rm, want_m)
+    assert rm[1] == -np.inf and es[1] == 0.0
+    with np.errstate(invalid="ignore"):
+        w = np.where(np.isfinite(bm), be.astype(np.float64) * np.exp(bm.astype(np.float64) - want_m[:, None]), 0.0)
+    keep = [0, 2, 3, 4, 5]
+    np.testing.assert_allclose(es[keep], w.sum(axis=1)[keep], rtol=1e-5)
+
+
 def test_decode_step_all_selected_equals_dense_attention():
     dev = _cuda()
     p = Problem(lens=[600], heads=1, groups=2, lists=16, seed=17)
