@@ -14,7 +14,8 @@ The marks (slot numbers as printed):
           for the table block), 4 end
   sample  0 start, 1 tables and first sampled keys loaded, 2 sampled keys scored, 3 smallest and
           largest key known, 4 threshold found (end); where the launch also builds the tables (no
-          lut launch then): 5 query row normalised, 6 first 256 centroids staged, 7 list scores done
+          lut launch then): 5 query row normalised, 6 first half of every centroid staged, 7 list scores and
+          PQ table done
   scan    0 start, 1 tables staged, 2 last window scored, 3 candidates and per-list sums flushed (end)
   select  0 start, 1 candidates requested and LDS cleared, 2 histogram of the keys built, 3 k-th key
           found and ties ranked, 4 output slots assigned, 5 winners and losers' weights written, 6 end
