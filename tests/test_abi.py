@@ -161,3 +161,28 @@ def test_integration_document_stub_matches_the_library_structs():
         assert ctypes.sizeof(g) == ctypes.sizeof(w)
         assert (g is w) or (hasattr(g, "_type_") and hasattr(w, "_type_") and
                             [f[0] for f in getattr(g._type_, "_fields_", [])] == [f[0] for f in getattr(w._type_, "_fields_", [])])
+
+
+def test_stand_alone_scan_statistics_reject_bad_arguments_before_any_gpu_work():
+    """pqhsa_lut_scan_stats and pqhsa_block_reduce check their arguments before the first HIP call:
+    the error code and message come back on a machine without a GPU too."""
+    import ctypes
+
+    lib = _lib.load()
+    idx = _lib.Index()
+    idx.batch, idx.kv_heads, idx.num_lists, idx.n_cap = 1, 1, 16, 1024
+    p = 4096  # stands for device pointers that a rejected call never follows
+
+    def stats(G=4, n_max=1000, block_keys=512, blocks=2, qnorm=p):
+        return lib.pqhsa_lut_scan_stats(ctypes.byref(idx), G, n_max, qnorm, p, p, 1.0, block_keys, blocks, p, p, None)
+
+    assert stats(qnorm=None) == -1 and b"NULL" in lib.pqhsa_last_error()
+    assert stats(G=17) == -1 and b"G=17" in lib.pqhsa_last_error()
+    assert stats(n_max=2000) == -1 and b"n_max=2000" in lib.pqhsa_last_error()
+    assert stats(blocks=1) == -1 and b"do not cover" in lib.pqhsa_last_error()
+    assert stats(block_keys=0) == -1
+    idx.num_lists = 4096                     # 4096 lists x 16 padded rows of list scores: more than a compute unit's LDS
+    assert stats(G=16) == -1 and b"LDS" in lib.pqhsa_last_error()
+    assert lib.pqhsa_block_reduce(None, p, 4, 8, p, p, None) == -1 and b"NULL" in lib.pqhsa_last_error()
+    assert lib.pqhsa_block_reduce(p, p, 4, 0, p, p, None) == -1 and b"blocks=0" in lib.pqhsa_last_error()
+    assert lib.pqhsa_block_reduce(p, p, 0, 8, p, p, None) == 0          # no rows: nothing to do
