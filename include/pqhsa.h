@@ -134,11 +134,13 @@ typedef struct pqhsa_select {
  * that is faster at every measured shape, because rows of a group already meet in the L2 and the
  * classification pass and the extra partial records cost more than the saved fetches. */
 #define PQHSA_SELECT_SHARE_ROWS 4
-/* A step of the general path that appends nothing, with at most 256 query rows (batches padded to
- * a multiple of 8 streams), at most 512 lists and at most 8 192 sampled keys per stream, builds
- * each query row's lookup tables and its threshold estimate in ONE launch (four launches per step
- * instead of five; same tables, thresholds and results to the bit).  This flag keeps the two as
- * separate launches, as steps of every other shape have them. */
+/* A step of the general path with at most 512 lists and at most 8 192 sampled keys per stream
+ * builds each query row's lookup tables and its threshold estimate in ONE launch (four launches
+ * per step instead of five; same tables, thresholds and results to the bit) when that launch fits
+ * the chip at once: one workgroup per query row of the padded group, or per two rows, for every
+ * stream (streams padded to a multiple of 8), plus one per stream in a step that appends, at most
+ * 256 in all (up to 512 query rows in groups of four).  This flag keeps the two as separate
+ * launches, as steps of every other shape have them. */
 #define PQHSA_SELECT_SEPARATE_TABLES 8
 
 const char *pqhsa_version(void);

@@ -626,6 +626,167 @@ __device__ inline void sample_thresh_body(const SampleArgs &a, const int g, cons
     }
 }
 
+// LDS of a workgroup that estimates the thresholds of two query rows at once
+struct ThreshPairLds {
+    __align__(16) uint32_t red[2][kSelWaves];
+    uint32_t span[2][2 * kSelWaves];
+    __align__(16) uint32_t hist[2][kSelBins];
+    uint32_t found[2][2];
+};
+
+// sample_thresh_body for rows g0 and g0 + 1 of stream bh together: the sampled keys are fetched once
+// and scored against both rows' tables, and the two estimates share every barrier (smallest and
+// largest key of both rows in one exchange, two histograms, a wave each for the walk from the top).
+// `tables(lut2, ls2, request, early)` leaves the two rows' tables in LDS with the rows side by side
+// (entry e of row r at lut2[2 e + r], list l at ls2[2 l + r]: one 8-byte read serves both rows), and
+// the rows' query norms in qn_pair[0..1].
+template <int R, int kBatch, class Tables>
+__device__ inline void sample_thresh_pair_body(const SampleArgs &a, const int g0, const int bh, ThreshPairLds &tl,
+                                               unsigned char *smem, const float *qn_pair,
+                                               [[maybe_unused]] const size_t trace_wg, Tables tables) {
+    const int tid = threadIdx.x;
+    const size_t row = (size_t)bh * a.GP + g0;
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 0);
+    const size_t base = (size_t)bh * a.s_cap;
+    uint32_t code[kBatch], lid[kBatch];
+    float kn[kBatch];
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int64_t p = min((int64_t)(r0 + r) * kSelThreads + tid, a.s_cap - 1);
+            code[r] = a.codes[base + p];
+            lid[r] = a.list_ids[base + p];
+            kn[r] = a.norms[base + p];
+        }
+    };
+    int n = a.n_arr[bh / a.n_div];
+    const int ns = a.ns_arr[bh / a.n_div];
+    float2 *lut2 = reinterpret_cast<float2 *>(smem);  // [128]
+    float2 *ls2 = lut2 + kM * kCodes;                 // [L]
+    int k = 0;
+    double want_d = 0.0;
+    auto resolve = [&]() __attribute__((always_inline)) {
+        if (a.counts_before_append && append_wanted(a.append.enc, a.append.count, bh / a.n_div)) ++n;
+        k = min(resolve_k(n, a.fraction, a.topk), a.k_cap);
+        const double ks = (double)max(k, 1) * (double)ns / (double)max(n, 1);
+        const double x = 0.5 * (kMarginSigmas + sqrt(kMarginSigmas * kMarginSigmas + 4.0 * ks));
+        want_d = ceil(x * x) + 1.0;
+    };
+    tables(lut2, ls2, [&]() __attribute__((always_inline)) { fetch(0); }, resolve);
+    const bool real[2] = {g0 < a.G, g0 + 1 < a.G};
+    auto leave = [&](int r, uint32_t thr, uint32_t hi, int kk, float ref) {
+        a.thr_key[row + r] = thr;
+        if (a.hi_key) a.hi_key[row + r] = hi;
+        a.k_row[row + r] = kk;
+        a.ref_val[row + r] = ref;
+    };
+    if (!real[0] || ns <= 0 || want_d >= (double)ns) {
+        // rows of the padding, or a sample too small to say anything (every key is a candidate then)
+        if (tid < 2) {
+            if (real[tid]) leave(tid, 0u, 0u, k, -INFINITY);
+            else leave(tid, 0xffffffffu, 0u, 0, -INFINITY);
+        }
+        return;
+    }
+    const uint32_t want = (uint32_t)want_d;
+    for (int i = tid; i < kSelBins; i += kSelThreads) tl.hist[0][i] = tl.hist[1][i] = 0u;
+    __syncthreads();
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 1);
+    const float qn0 = qn_pair[0], qn1 = qn_pair[1];
+    uint32_t key0[R], key1[R];
+#pragma unroll
+    for (int r0 = 0; r0 < R; r0 += kBatch) {
+        if (r0 > 0) fetch(r0);
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int p = (r0 + r) * kSelThreads + tid;
+            if (lid[r] >= (uint32_t)a.L) lid[r] = 0u;
+            // (each row's sum in the oracle's order, as score_one forms it)
+            float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+            for (int m = 0; m < kM; ++m) {
+                const float2 e = lut2[m * kCodes + ((code[r] >> (4 * m)) & 15u)];
+                s0 = s0 + e.x;
+                s1 = s1 + e.y;
+            }
+            const float2 l2 = ls2[lid[r]];
+            s0 = (((s0 + l2.x) * qn0) * kn[r]) * a.scale;
+            s1 = (((s1 + l2.y) * qn1) * kn[r]) * a.scale;
+            key0[r0 + r] = p < ns ? max(order_key(s0), 1u) : 0u;
+            key1[r0 + r] = p < ns ? max(order_key(s1), 1u) : 0u;
+        }
+    }
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 2);
+    // smallest and largest key of each row: one exchange for both
+    uint32_t hi[2] = {0u, 0u}, lo[2] = {0xffffffffu, 0xffffffffu};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        hi[0] = max(hi[0], key0[r]);
+        lo[0] = min(lo[0], key0[r] != 0u ? key0[r] : 0xffffffffu);
+        hi[1] = max(hi[1], key1[r]);
+        lo[1] = min(lo[1], key1[r] != 0u ? key1[r] : 0xffffffffu);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        hi[j] = wave_max_u32(hi[j]);
+        lo[j] = ~wave_max_u32(~lo[j]);
+    }
+    if ((tid & (kWave - 1)) == 0) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            tl.span[j][tid / kWave] = hi[j];
+            tl.span[j][kSelWaves + tid / kWave] = lo[j];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int w = 0; w < kSelWaves; ++w) {
+            hi[j] = max(hi[j], tl.span[j][w]);
+            lo[j] = min(lo[j], tl.span[j][kSelWaves + w]);
+        }
+    }
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 3);
+    // the histogram window of each row, as in sample_thresh_body
+    constexpr uint32_t kWindow = 1u << 25;
+    uint32_t wbase[2];
+    int shift[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        wbase[j] = hi[j] > kWindow ? max(hi[j] - kWindow, lo[j]) : lo[j];
+        const uint32_t range = hi[j] >= wbase[j] ? hi[j] - wbase[j] : 0u;
+        shift[j] = range < (uint32_t)kSelBins ? 0 : (31 - __clz(range)) - 9;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (key0[r] != 0u && key0[r] >= wbase[0]) atomicAdd(&tl.hist[0][(key0[r] - wbase[0]) >> shift[0]], 1u);
+        if (key1[r] != 0u && key1[r] >= wbase[1]) atomicAdd(&tl.hist[1][(key1[r] - wbase[1]) >> shift[1]], 1u);
+    }
+    if (tid < 2) tl.found[tid][0] = 0xffffffffu;
+    __syncthreads();
+    if (tid < 2 * kWave) find_from_top_1024(tl.hist[tid / kWave], want, &tl.found[tid / kWave][0], &tl.found[tid / kWave][1]);
+    __syncthreads();
+    uint32_t t[2];
+    int step = 0;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {  // (uniform over the workgroup)
+        const uint32_t bin = tl.found[j][0];
+        if (bin < (uint32_t)kSelBins && tl.hist[j][bin] <= max(want / 8u, 16u)) {
+            t[j] = wbase[j] + (bin << shift[j]);
+        } else {
+            bool exact;
+            t[j] = j == 0 ? bisect_regs<R>(key0, want, want / 8u, tl.red, step, exact)
+                          : bisect_regs<R>(key1, want, want / 8u, tl.red, step, exact);
+        }
+    }
+    PQHSA_TRACE_MARK(trace_sample, trace_wg, 4);
+    if (tid < 2) {
+        if (real[tid]) leave(tid, t[tid], hi[tid], k, t[tid] == 0u ? -INFINITY : key_to_float(t[tid]));
+        else leave(tid, 0xffffffffu, 0u, 0, -INFINITY);
+    }
+}
+
 // the row's tables as an earlier launch left them in memory
 struct TablesFromMemory {
     const SampleArgs &a;
@@ -931,6 +1092,144 @@ __global__ __launch_bounds__(kSelThreads) void tables_thresh_kernel(TablesArgs p
 }
 
 
+// The same for batches of 257 to 512 query rows: a workgroup takes TWO rows of a stream (rows 2 j and
+// 2 j + 1 of the padded group), so that every workgroup still has a compute unit of its own.  The
+// stream's centroids pass through its LDS once, every staged element feeds both rows' chains (the
+// same chains, the same bits), the first two waves normalise a row each, the last four compute the
+// two PQ tables; the two threshold estimates run together (sample_thresh_pair_body).
+template <int DT, int R>
+__global__ __launch_bounds__(kSelThreads) void tables_thresh_pair_kernel(TablesArgs p, SampleArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ ThreshPairLds t;
+    __shared__ __align__(16) float qrow[2][kD];
+    __shared__ float qn_s[2];
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= p.thresh_wgs) {
+        append_role(p, (int)blockIdx.x - p.thresh_wgs, reinterpret_cast<float *>(smem), qrow[0]);
+        return;
+    }
+    const int L = a.L, GP = a.GP, pairs = GP / 2;
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int g0 = 2 * (slot % pairs);
+    const int bh = (slot / pairs) * kXcdCount + xcd;
+    const bool idle = bh >= p.streams;  // (the grid is whole rounds of the 8 XCDs)
+    const bool live0 = !idle && g0 < a.G, live1 = !idle && g0 + 1 < a.G;
+    // a wave loads elements lane and lane + 64 of the row it would normalise (even waves the first
+    // row, odd waves the second; of a row that exists when its own does not: no branch to wait in)
+    const int lane = tid % kWave, mine = (tid / kWave) & 1;
+    const bool live_mine = mine ? live1 : live0;
+    const size_t q_row = live_mine ? (size_t)bh * a.G + g0 + mine : 0;
+    const char *q_ptr = p.q + q_row * kD * (DT == PQHSA_F32 ? 4 : 2);
+    float qa = load1<DT>(q_ptr, lane), qb = load1<DT>(q_ptr, lane + kWave);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!live_mine) qa = qb = 0.0f;
+    auto clear_scratch = [&]() __attribute__((always_inline)) {
+        const size_t nthreads = (size_t)gridDim.x * kSelThreads;
+        for (size_t i = (size_t)blockIdx.x * kSelThreads + tid; i < p.zero_words; i += nthreads) p.zero_base[i] = 0u;
+    };
+    if (idle) {
+        clear_scratch();
+        return;
+    }
+    const int tbl = (kM * kCodes + L + 3) & ~3;  // floats of one row's tables
+    float *cs = reinterpret_cast<float *>(smem) + 2 * tbl;  // [kTtLists][kTtStride], past both rows' tables
+
+    auto tables = [&](float2 *lut2, float2 *ls2, auto request, auto early) __attribute__((always_inline)) {
+        CentroidHalves ch;
+        const float4 *c4 = reinterpret_cast<const float4 *>(p.coarse + (size_t)bh * L * kD);
+        ch.request(c4, L, tid, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (tid < 2 * kWave) {  // the rows' norms, a wave each: one chain over d in order
+            float ss = 0.0f;
+#pragma unroll
+            for (int d = 0; d < kWave; ++d) {
+                const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qa), d));
+                ss = __builtin_fmaf(x, x, ss);
+            }
+#pragma unroll
+            for (int d = 0; d < kWave; ++d) {
+                const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(qb), d));
+                ss = __builtin_fmaf(x, x, ss);
+            }
+            const float nrm = sqrtf(ss);
+            const float qn0 = nrm < p.eps ? p.eps : nrm;
+            qrow[mine][lane] = qa / qn0;
+            qrow[mine][lane + kWave] = qb / qn0;
+            if (lane == 0) {
+                qn_s[mine] = qn0;
+                p.qnorm[(size_t)bh * GP + g0 + mine] = live_mine ? qn0 : 0.0f;
+            }
+        }
+        PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 5);
+        ch.request(c4, L, tid, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        request();
+        early();
+        clear_scratch();
+        // PQ tables: entry (m, c) of row r by thread r * 128 + m * 16 + c of the last four waves
+        constexpr int kLutThreads = 2 * kM * kCodes;
+        const bool lut_thread = tid >= kSelThreads - kLutThreads;
+        const int lt = lut_thread ? tid - (kSelThreads - kLutThreads) : 0;
+        const int e = lt % (kM * kCodes), er = lt / (kM * kCodes);
+        float4 w[kSub / 4];
+        const float4 *w4 = reinterpret_cast<const float4 *>(p.codebooks + ((size_t)bh * kM * kCodes + e) * kSub);
+        auto pq_table = [&]() __attribute__((always_inline)) {
+            const float *qm = qrow[er] + (e / kCodes) * kSub;
+            float acc = 0.0f;
+            if (er ? live1 : live0) {
+#pragma unroll
+                for (int j = 0; j < kSub / 4; ++j) {
+                    acc = __builtin_fmaf(qm[4 * j], w[j].x, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 1], w[j].y, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 2], w[j].z, acc);
+                    acc = __builtin_fmaf(qm[4 * j + 3], w[j].w, acc);
+                }
+            }
+            reinterpret_cast<float *>(lut2)[2 * e + er] = acc;
+            p.lut[((size_t)bh * kM * kCodes + e) * GP + g0 + er] = acc;
+        };
+        // list scores: list l by lane l % 64 of wave l / 64, both rows from one read of the centroid
+        const int l = tid;
+        float score0 = 0.0f, score1 = 0.0f;
+        auto run_half = [&](int half) __attribute__((always_inline)) {
+            ch.stage(half, cs, tid);
+            if (half == 0) {
+#pragma unroll
+                for (int j = 0; j < kSub / 4; ++j) w[j] = w4[j];
+            }
+            __syncthreads();
+            if (half == 0) PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 6);
+            if (half == 1 && lut_thread) pq_table();
+            if (l < L) {  // (a row that does not exist has a row of zeros: its scores are zero)
+                const float *c = cs + (size_t)l * kTtStride;
+                const float *qa4 = qrow[0] + half * kTtHalf, *qb4 = qrow[1] + half * kTtHalf;
+#pragma unroll 2
+                for (int d4 = 0; d4 < CentroidHalves::kParts; ++d4) {
+                    const float4 cc = *reinterpret_cast<const float4 *>(c + 4 * d4);
+                    const float4 x = *reinterpret_cast<const float4 *>(qa4 + 4 * d4);
+                    const float4 y = *reinterpret_cast<const float4 *>(qb4 + 4 * d4);
+                    score0 = __builtin_fmaf(x.x, cc.x, score0); score1 = __builtin_fmaf(y.x, cc.x, score1);
+                    score0 = __builtin_fmaf(x.y, cc.y, score0); score1 = __builtin_fmaf(y.y, cc.y, score1);
+                    score0 = __builtin_fmaf(x.z, cc.z, score0); score1 = __builtin_fmaf(y.z, cc.z, score1);
+                    score0 = __builtin_fmaf(x.w, cc.w, score0); score1 = __builtin_fmaf(y.w, cc.w, score1);
+                }
+            }
+            __syncthreads();
+        };
+        run_half(0);  // (its first barrier also publishes the normalised rows)
+        run_half(1);
+        if (l < L) {
+            ls2[l] = make_float2(score0, score1);
+            // (rows g0 and g0 + 1 of the padded group lie side by side in memory as well)
+            *reinterpret_cast<float2 *>(p.list_scores + ((size_t)bh * L + l) * GP + g0) = make_float2(score0, score1);
+        }
+        PQHSA_TRACE_MARK(trace_sample, blockIdx.x, 7);
+        // (the caller has a barrier before the tables' and the norms' first use)
+    };
+    sample_thresh_pair_body<R, 4>(a, g0, bh, t, smem, qn_s, blockIdx.x, tables);
+}
+
+
 // RS > 0: the host expects at most RS * 1024 candidates per row, and the kernel requests that many
 // candidate slots before it knows the count, together with the count itself (one round trip to
 // memory instead of two); slots past the count hold leftovers of earlier steps and are masked.
@@ -1204,29 +1503,40 @@ int launch_sample_thresh(SampleArgs a, int streams, hipStream_t stream) {
 // Whether the tables and the threshold estimate of a step share one launch: every row's workgroup
 // (and, in a step that appends, one more per stream) on a compute unit of its own (it fills one),
 // and sample and lists within what the kernel is compiled for.
-bool tables_thresh_fits(int streams, int GP, int L, int64_t s_cap, bool appending) {
-    const int rounds = (streams + kXcdCount - 1) / kXcdCount;
-    return rounds * kXcdCount * GP + (appending ? streams : 0) <= 256 && L <= kTtLists && s_cap <= 8 * kSelThreads;
+// Returns the query rows per workgroup (1, or 2 where every row with a workgroup of its own would not
+// fit the chip at once), or 0 when the shape takes the two separate launches.
+int tables_thresh_fits(int streams, int GP, int L, int64_t s_cap, bool appending) {
+    if (L > kTtLists || s_cap > 8 * kSelThreads) return 0;
+    const int rounds = (streams + kXcdCount - 1) / kXcdCount, extra = appending ? streams : 0;
+    if (rounds * kXcdCount * GP + extra <= 256) return 1;
+    if (GP >= 2 && rounds * kXcdCount * (GP / 2) + extra <= 256) return 2;
+    return 0;
 }
 
 int launch_tables_thresh(TablesArgs p, int q_dtype, SampleArgs a, hipStream_t stream) {
     const bool appending = p.append.count != nullptr;
-    PQHSA_REQUIRE(tables_thresh_fits(p.streams, a.GP, a.L, a.s_cap, appending), "tables_thresh: shape outside the kernel's range");
+    const int rows_per_wg = tables_thresh_fits(p.streams, a.GP, a.L, a.s_cap, appending);
+    PQHSA_REQUIRE(rows_per_wg != 0, "tables_thresh: shape outside the kernel's range");
     PQHSA_REQUIRE(p.q && p.coarse && p.codebooks && p.qnorm && p.lut && p.list_scores, "tables_thresh: NULL argument");
     PQHSA_REQUIRE(!appending || (p.n_after && p.append.enc.L == a.L && p.append.enc.coarse == p.coarse),
                   "tables_thresh: append arguments do not match the index");
     const int rounds = (p.streams + kXcdCount - 1) / kXcdCount;
-    p.thresh_wgs = rounds * kXcdCount * a.GP;
+    p.thresh_wgs = rounds * kXcdCount * a.GP / rows_per_wg;
     dim3 grid(p.thresh_wgs + (appending ? p.streams : 0)), block(kSelThreads);
-    const size_t lds = (size_t)((kM * kCodes + a.L + 3) & ~3) * 4 + (size_t)kTtLists * kTtStride * 4;
+    const size_t lds = (size_t)rows_per_wg * ((kM * kCodes + a.L + 3) & ~3) * 4 + (size_t)kTtLists * kTtStride * 4;
     const bool small = a.s_cap <= 4 * kSelThreads;
-#define PQHSA_TT(DT_, R_)                                                                           \
+#define PQHSA_TT(KERNEL_, DT_, R_)                                                                  \
     do {                                                                                            \
-        const int rc = raise_lds_limit((const void *)tables_thresh_kernel<DT_, R_>, lds, "tables_thresh"); \
+        const int rc = raise_lds_limit((const void *)KERNEL_<DT_, R_>, lds, "tables_thresh");       \
         if (rc) return rc;                                                                          \
-        hipLaunchKernelGGL((tables_thresh_kernel<DT_, R_>), grid, block, lds, stream, p, a);        \
+        hipLaunchKernelGGL((KERNEL_<DT_, R_>), grid, block, lds, stream, p, a);                     \
     } while (0)
-    PQHSA_DISPATCH_DTYPE(q_dtype, if (small) PQHSA_TT(DT, 4); else PQHSA_TT(DT, 8));
+    if (rows_per_wg == 1) {
+        PQHSA_DISPATCH_DTYPE(q_dtype, if (small) PQHSA_TT(tables_thresh_kernel, DT, 4); else PQHSA_TT(tables_thresh_kernel, DT, 8));
+    } else {
+        PQHSA_DISPATCH_DTYPE(q_dtype, if (small) PQHSA_TT(tables_thresh_pair_kernel, DT, 4);
+                             else PQHSA_TT(tables_thresh_pair_kernel, DT, 8));
+    }
 #undef PQHSA_TT
     return check_launch("tables_thresh");
 }
@@ -1747,7 +2057,7 @@ int decode_thresholds(const pqhsa_index *index, int G, int GP, const float *qnor
 }
 
 bool decode_tables_thresh_fits(const pqhsa_index *index, int G, bool appending) {
-    return tables_thresh_fits(index->batch * index->kv_heads, padded_groups(G), index->num_lists, index->s_cap, appending);
+    return 0 != tables_thresh_fits(index->batch * index->kv_heads, padded_groups(G), index->num_lists, index->s_cap, appending);
 }
 
 // the tables of every query row and its threshold in one launch (a step whose shape

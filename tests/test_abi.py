@@ -58,7 +58,9 @@ def test_launch_count_follows_the_short_context_rule():
     assert launches(4, 16385) == 4            # more keys than a workgroup holds in registers
     assert launches(4, 8192, appending=1) == 4
     assert launches(16, 8192) == 1 and launches(16, 8192) == launches(16, 1)
-    index.batch = 3                           # 3 * 8 * 16 query rows > 256
+    index.batch = 3                           # 3 * 8 * 16 query rows > 256: two rows per workgroup
+    assert launches(16, 8192) == 4
+    index.batch = 5                           # 5 * 8 * 16 / 2 workgroups > 256
     assert launches(16, 8192) == 5
     index.batch = 1
     sel.flags = _lib.SELECT_GENERAL_PATH
@@ -66,20 +68,22 @@ def test_launch_count_follows_the_short_context_rule():
     sel.flags, sel.k_cap = 0, 2049
     assert launches(4, 8192) == 4
     # tables and threshold estimate in one launch: unless the caller keeps them apart, for steps
-    # whose query rows (streams padded to a multiple of 8; one more workgroup per stream in a step
-    # that appends) each get a compute unit, with at most 512 lists and 8 192 sampled keys per stream
+    # whose query rows, or pairs of them (streams padded to a multiple of 8; one more workgroup per
+    # stream in a step that appends), each get a compute unit, with at most 512 lists and 8 192
+    # sampled keys per stream
     sel.flags = _lib.SELECT_SEPARATE_TABLES
     assert launches(4, 8192) == 5
     sel.flags = 0
-    index.batch = 9                           # 72 streams x 4 rows > 256
+    index.batch = 9                           # 72 streams x 4 rows > 256: two rows per workgroup
+    assert launches(4, 20000) == 4
+    index.batch = 16                          # 128 streams x 2 pairs = 256
+    assert launches(4, 20000) == 4 and launches(4, 20000, appending=1) == 5   # (one more workgroup per stream)
+    index.batch = 17
     assert launches(4, 20000) == 5
-    index.batch = 7                           # 56 streams x 4 rows
-    assert launches(4, 20000) == 4 and launches(4, 20000, appending=1) == 5   # (one more workgroup per stream: 224 + 56)
-    index.batch = 6
-    assert launches(4, 20000, appending=1) == 4
-    index.batch = 7
-    index.batch, index.kv_heads = 7, 9        # 63 streams, padded to 64: 256 rows
-    assert launches(4, 20000) == 4 and launches(5, 20000) == 5
+    index.batch = 7                           # 56 streams x 4 rows; with the appending workgroups 224 + 56: pairs
+    assert launches(4, 20000) == 4 and launches(4, 20000, appending=1) == 4
+    index.batch, index.kv_heads = 7, 9        # 63 streams, padded to 64: 256 rows, or 256 pairs of a group of 5 (padded to 8)
+    assert launches(4, 20000) == 4 and launches(5, 20000) == 4 and launches(9, 20000) == 5
     index.batch, index.kv_heads = 1, 8
     index.num_lists = 513
     assert launches(4, 20000) == 5

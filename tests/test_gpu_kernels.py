@@ -950,7 +950,9 @@ def test_ragged_batch_tile_hint_changes_no_result(lens, heads):
     # the steps after the first replayed from ONE HIP graph, captured with the launch shapes of the
     # final length: sequence lengths, key counts and the new keys are all read from device memory
     dict(steps=5, lens=[1805, 1505], heads=2, groups=4, lists=32, every=1, graph=True),
-], ids=["small", "many_streams", "small_two_launches", "ragged_groups", "graph_replay"])
+    # more than 256 query rows: two rows of a stream per workgroup, and the appending workgroups beside them
+    dict(steps=2, lens=[862, 852, 847, 842, 872, 882, 843, 854, 866], heads=8, groups=4, lists=64, every=7),
+], ids=["small", "many_streams", "small_two_launches", "ragged_groups", "graph_replay", "row_pairs"])
 def test_fused_append_decode_steps_match_oracle_and_separate_append(shape):
     """pqhsa_append_decode_step over several steps: each step encodes the sequence's next key in
     the launch that builds the tables, attends over the grown index, and leaves the new count in
@@ -1088,8 +1090,9 @@ def test_decode_step_random_shapes_match_oracle(seed):
 
 def test_decode_step_batch_of_more_than_256_query_rows():
     """288 query rows (9 sequences x 8 KV heads x 4): the selection kernel then runs in the form
-    that shares a compute unit between two workgroups, and the short-context kernel does not
-    apply.  A sample of the streams against the oracle, all rows for sane counts."""
+    that shares a compute unit between two workgroups, the launch that builds the tables and
+    estimates the thresholds gives a workgroup two rows of a stream, and the short-context kernel
+    does not apply.  A sample of the streams against the oracle, all rows for sane counts."""
     dev = _cuda()
     lens = [2400, 1300, 1900, 2100, 900, 1700, 2300, 1100, 1500]
     p = Problem(lens=lens, heads=8, groups=4, lists=32, dtype=torch.bfloat16, seed=83)
@@ -1101,7 +1104,7 @@ def test_decode_step_batch_of_more_than_256_query_rows():
     ops.decode_step(q, out, kv, idx, p.G, p.seq_lens(), sink=p.sink, full_max=p.sink + p.local, fraction=0.04,
                     topk=0, scale=SCALE, workspace=ws)
     torch.cuda.synchronize()
-    assert ops.decode_step_launches(idx, p.G, ws) == 5
+    assert ops.decode_step_launches(idx, p.G, ws) == 4
     tidx = ws.topk_idx.cpu().numpy().reshape(p.B, p.H, p.G, -1)
     cnt = ws.topk_cnt.cpu().numpy().reshape(p.B, p.H, p.G)
     o = out.cpu().numpy().reshape(p.B, p.H, p.G, DIM)
@@ -1223,6 +1226,11 @@ TABLES_CASES = [
     dict(lens=[2000, 700, 60, 1500], heads=2, groups=2, lists=40, dtype=torch.float32),   # (one sequence without indexed keys)
     # room for 170 000 keys per sequence: a sample of more than 4 096 keys per stream, eight per thread
     dict(lens=[20000, 12000], heads=1, groups=4, lists=128, dtype=torch.bfloat16, spare=150000),
+    # more than 256 query rows: a workgroup takes two rows of a stream (whole groups, a group padded
+    # from 7 to 8 rows whose last pair holds one row, a group of 3 whose last pair holds one)
+    dict(lens=[2500, 1800, 2100, 900, 2300, 1500, 2600, 1200, 2000], heads=8, groups=4, lists=64, dtype=torch.bfloat16),
+    dict(lens=[2400, 1700, 2900, 1300, 2000], heads=8, groups=7, lists=300, dtype=torch.float32),
+    dict(lens=[2500, 1800, 2100, 900, 2300, 1500, 2600, 1200, 2000], heads=8, groups=3, lists=512, dtype=torch.float16),
 ]
 
 
