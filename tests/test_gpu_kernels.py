@@ -585,6 +585,30 @@ def _check_step(p, idx, kv, ws, fraction, tol=1e-4, general_path=True):
     return runs
 
 
+@pytest.mark.parametrize("lens,heads", [([5000], 2), ([1500, 1300, 1700, 1200, 1600, 1400, 1100, 1800, 1250], 8)],
+                         ids=["workgroup_per_row", "workgroup_per_row_pair"])
+def test_threshold_estimate_on_heavily_tied_logits(lens, heads):
+    """An index whose stored keys repeat five (code, list, norm) triples: a row's sampled logits take
+    five values only, the histogram of the threshold estimate cannot separate them, and its
+    bit-by-bit search takes over -- in both forms of the launch, a workgroup per query row and a
+    workgroup per pair of rows (288 rows).  The selection is still the exact top-k, ties to the
+    lowest index, and the candidates are whole groups of equal logits."""
+    dev = _cuda()
+    p = Problem(lens=lens, heads=heads, groups=4, lists=32, seed=67)
+    for ix in p.index.values():
+        pick = np.arange(ix["codes"].shape[0]) % 5
+        for name in ("codes", "list_ids", "norms"):
+            ix[name] = ix[name][pick].copy()
+    idx = p.device_index(dev)
+    kv = ops.kv_contiguous(*p.dense_kv())
+    ws = ops.DecodeWorkspace(idx, p.G, ops.resolve_topk(p.n_max, 0.05, 0))
+    assert ops.decode_step_launches(idx, p.G, ws, general_path=True) == 4
+    assert _check_step(p, idx, kv, ws, 0.05) >= 2                 # (tables and thresholds in one launch, and apart)
+    counts = ws.candidate_counts().cpu().numpy().reshape(p.B, p.H, -1)[:, :, : p.G]
+    for b in range(p.B):
+        assert (counts[b] >= p.n(b) // 5).all()                   # at least the whole group of the best logit
+
+
 def test_decode_step_rescans_rows_when_the_sampled_threshold_keeps_too_few():
     """A sample made of the stream's best-scoring keys puts the threshold far too high: every row
     keeps fewer than k candidates, is re-scored in full by its selection workgroup, and the
