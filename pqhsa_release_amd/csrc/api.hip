@@ -56,15 +56,33 @@ static int g_prof_only = -1;  // >= 0: only this kernel is bracketed by events
 static int g_prof_every = 1;  // one decode step in this many is logged
 static int g_prof_seen = 0;   // decode steps since the log was enabled
 
-void profile_mark(int slot, hipStream_t stream) {
+// `stamped`: the launcher of the one bracketed kernel gives (or gave) the slot's event to the launch
+// itself (profile_kernel_stamps): nothing is recorded here, only the steps are counted.
+void profile_mark(int slot, hipStream_t stream, bool stamped) {
     if (!g_prof_on || g_prof_step >= g_prof_steps) return;
     const bool logged = g_prof_seen % g_prof_every == 0;
-    if (logged && (g_prof_only < 0 || slot == g_prof_only || slot == g_prof_only + 1))
+    if (logged && !stamped && (g_prof_only < 0 || slot == g_prof_only || slot == g_prof_only + 1))
         (void)hipEventRecord(g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot], stream);
     if (slot == kProfKernels) {
         if (logged) ++g_prof_step;
         ++g_prof_seen;
     }
+}
+
+// When kernel `slot` is the only one bracketed and this step is logged: the two events of its
+// slot, for a launch that stamps them with the kernel's own start and end (hipExtLaunchKernelGGL)
+// instead of event records before and after it, which add a marker of their own to the stream on
+// either side.  The caller then passes `stamped` to the slot's two profile_mark calls.
+bool profile_kernel_stamps(int slot, hipEvent_t *start, hipEvent_t *stop) {
+    if (!g_prof_on || g_prof_step >= g_prof_steps || g_prof_only != slot || g_prof_seen % g_prof_every != 0) return false;
+    static const bool brackets = [] {
+        const char *e = getenv("PQHSA_PROFILE_BRACKETS");
+        return e && e[0] == '1';
+    }();
+    if (brackets) return false;
+    *start = g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot];
+    *stop = g_events[(size_t)g_prof_step * (kProfKernels + 1) + slot + 1];
+    return true;
 }
 
 }  // namespace pqhsa

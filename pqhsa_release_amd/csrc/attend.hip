@@ -13,6 +13,8 @@
 // output row (fold_row_if_last): the step needs no further launch.
 #include <cfloat>
 
+#include <hip/hip_ext.h>
+
 #include "common.h"
 
 namespace pqhsa {
@@ -172,6 +174,10 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
         if (mark) profile_mark(kProfKernels, stream);
         return check_launch("attend_shared");
     }
+    // (when the event log brackets this kernel alone, the launch itself stamps the slot's two events
+    // with the kernel's start and end; decode_scan_select has left the slot's first event alone)
+    hipEvent_t stamp_start = nullptr, stamp_stop = nullptr;
+    const bool stamped = mark && profile_kernel_stamps(kProfAttend, &stamp_start, &stamp_stop);
 #define PQHSA_ATT(KD, QD)                                                                              \
     {                                                                                                  \
         auto kern = attend_partial_kernel<KD, QD>;                                                     \
@@ -183,7 +189,8 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
                 return PQHSA_ELAUNCH;                                                                  \
             }                                                                                          \
         }                                                                                              \
-        hipLaunchKernelGGL(kern, grid, dim3(kAttThreads), lds, stream, a);                             \
+        if (stamped) hipExtLaunchKernelGGL(kern, grid, dim3(kAttThreads), (uint32_t)lds, stream, stamp_start, stamp_stop, 0, a); \
+        else hipLaunchKernelGGL(kern, grid, dim3(kAttThreads), lds, stream, a);                        \
     }
     if (kv_dtype == PQHSA_BF16 && q_dtype == PQHSA_BF16) PQHSA_ATT(PQHSA_BF16, PQHSA_BF16)
     else if (kv_dtype == PQHSA_F32 && q_dtype == PQHSA_F32) PQHSA_ATT(PQHSA_F32, PQHSA_F32)
@@ -195,7 +202,7 @@ int launch_attend(AttendArgs a, int q_dtype, int kv_dtype, int BH, int rows_max,
         return PQHSA_EINVAL;
     }
 #undef PQHSA_ATT
-    if (mark) profile_mark(kProfKernels, stream);
+    if (mark) profile_mark(kProfKernels, stream, stamped);
     return check_launch("attend");
 }
 

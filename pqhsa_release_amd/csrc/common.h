@@ -23,7 +23,8 @@ void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 int launch_fill_zero(void *p, size_t bytes, hipStream_t stream);  // clears with a kernel (graph-capturable)
 // Records the next profiling event on `stream` when profiling is enabled (no-op otherwise).
-void profile_mark(int slot, hipStream_t stream);
+void profile_mark(int slot, hipStream_t stream, bool stamped = false);
+bool profile_kernel_stamps(int slot, hipEvent_t *start, hipEvent_t *stop);
 enum { kProfLut = 0, kProfSample, kProfEmit, kProfSelect, kProfAttend, kProfKernels };
 
 #define PQHSA_REQUIRE(cond, ...)            \

@@ -24,6 +24,8 @@ namespace pqhsa {
 PQHSA_TRACE_DECL(trace_scan)
 }
 #define PQHSA_SCAN_MARK(wg, slot) PQHSA_TRACE_MARK(trace_scan, wg, slot)
+#include <hip/hip_ext.h>
+
 #include "scan_emit_body.h"
 
 namespace pqhsa {
@@ -72,7 +74,9 @@ constexpr int kPackedSeqs = 64;
 
 
 // n_mean: the mean key count per stream when the caller knows it (0: every stream is taken to hold n_max)
-int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream) {
+// stamp_start / stamp_stop: events that take the kernel's own start and end (both or neither)
+int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream,
+                     hipEvent_t stamp_start, hipEvent_t stamp_stop) {
     if (streams == 0 || n_max <= 0) return PQHSA_OK;
     PQHSA_REQUIRE(a.mass, "scan_emit: no list-mass output");
     a.stage_cap = emit_stage_cap(GP);
@@ -120,7 +124,8 @@ int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_m
                 return PQHSA_ELAUNCH;                                                                       \
             }                                                                                               \
         }                                                                                                   \
-        hipLaunchKernelGGL(kern, grid, dim3(kScanThreads), lds, stream, a);                                 \
+        if (stamp_start) hipExtLaunchKernelGGL(kern, grid, dim3(kScanThreads), (uint32_t)lds, stream, stamp_start, stamp_stop, 0, a); \
+        else hipLaunchKernelGGL(kern, grid, dim3(kScanThreads), lds, stream, a);                            \
     }
 #define PQHSA_EMIT_CASE(gp)                                                                                 \
     case gp:                                                                                                \
@@ -170,5 +175,5 @@ extern "C" int pqhsa_lut_scan_mass(const pqhsa_index *index, int32_t G, int32_t 
     a.codes = index->codes; a.list_ids = index->list_ids; a.norms = index->norms; a.pos = nullptr;
     a.n_cap = index->n_cap; a.n_arr = index->n_idx;
     a.thr_key = nullptr; a.ref_val = ref; a.mass = list_mass;
-    return launch_scan_emit(a, GP, streams, n_max, 0, stream);
+    return launch_scan_emit(a, GP, streams, n_max, 0, stream, nullptr, nullptr);
 }

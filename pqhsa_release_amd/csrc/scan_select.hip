@@ -2021,7 +2021,8 @@ int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
     return rc;
 }
 
-int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream);
+int launch_scan_emit(ScanArgs a, int GP, int streams, int64_t n_max, int64_t n_mean, hipStream_t stream,
+                     hipEvent_t stamp_start, hipEvent_t stamp_stop);
 
 // what the threshold estimate aims at for the longest row, plus its tolerance and a margin
 int64_t decode_expected_candidates(const pqhsa_index *index, int64_t n_max, const pqhsa_select *select) {
@@ -2118,13 +2119,16 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
                                                   ref_val, append, stream);
     if (rc) return rc;
     uint32_t *hi_key = thr_key + (size_t)streams * GP;
-    profile_mark(kProfEmit, stream);
+    // (when the event log brackets the scan alone, the launch itself stamps the slot's two events)
+    hipEvent_t scan_start = nullptr, scan_stop = nullptr;
+    const bool scan_stamped = profile_kernel_stamps(kProfEmit, &scan_start, &scan_stop);
+    profile_mark(kProfEmit, stream, scan_stamped);
     // 2. the full scan
     const ScanArgs a = decode_scan_args(index, G, qnorm, lut, list_scores, scale, emit_count, thr_key, ref_val, pairs, aux,
                                         emit_cap, mass);
-    rc = launch_scan_emit(a, GP, streams, n_max, select->n_mean, stream);
+    rc = launch_scan_emit(a, GP, streams, n_max, select->n_mean, stream, scan_start, scan_stop);
     if (rc) return rc;
-    profile_mark(kProfSelect, stream);
+    profile_mark(kProfSelect, stream, scan_stamped);
     // 3. exact selection among the candidates
     SelectArgs s = {};
     s.pairs = static_cast<uint2 *>(pairs); s.raw_keys = 1; s.aux = a.packed_records ? nullptr : aux; s.packed = a.packed_records;
@@ -2138,7 +2142,9 @@ int decode_scan_select(const pqhsa_index *index, int G, int GP, int64_t n_max, c
     s.share_map = share_map; s.share_stride = share_stride;
     s.expected_candidates = decode_expected_candidates(index, n_max, select);
     rc = launch_select_final(s, streams, stream);
-    profile_mark(kProfAttend, stream);
+    // (the attention launch that follows stamps its own events in that case: see launch_attend)
+    hipEvent_t att_start, att_stop;
+    profile_mark(kProfAttend, stream, share_map == nullptr && profile_kernel_stamps(kProfAttend, &att_start, &att_stop));
     return rc;
 }
 
