@@ -807,7 +807,8 @@ def main():
         g = run.gather_ceiling()
         result["roofline"]["random_row_ceiling_GBps"] = g["GBps"]
         result["roofline"]["random_row_probe"] = g
-        att_us = result["kernels"]["attend"]["us"]
+        # (the attention's time from the timed region where it is the dominant kernel, else from the survey)
+        att_us = run.dominant_us if run.dominant == "attend" else result["kernels"]["attend"]["us"]
         if att_us > 0:   # the rows alone (the attention kernel's figure also counts the list means)
             result["roofline"]["attend_frac_of_random_row_ceiling"] = round(
                 (ab["exact"] + ab["full"]) / 1e3 / att_us / g["GBps"], 4)
