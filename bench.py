@@ -714,7 +714,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--layers", type=int, default=3, help="distinct resident layers rotated through (defeats cache reuse)")
-    ap.add_argument("--event-every", type=int, default=8,
+    ap.add_argument("--event-every", type=int, default=10,
                     help="in the timed region the dominant kernel is bracketed by HIP events on one step in this many")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
