@@ -85,6 +85,16 @@ bool profile_kernel_stamps(int slot, hipEvent_t *start, hipEvent_t *stop) {
     return true;
 }
 
+LaunchStamps g_launch_stamps;
+
+// profile_kernel_stamps for a launcher that takes the events from g_launch_stamps: true when set
+bool profile_stamp_next_launch(int slot) {
+    LaunchStamps s;
+    if (!profile_kernel_stamps(slot, &s.start, &s.stop)) return false;
+    g_launch_stamps = s;
+    return true;
+}
+
 }  // namespace pqhsa
 
 extern "C" int pqhsa_profile_enable(int32_t max_steps) {

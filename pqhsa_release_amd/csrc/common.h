@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
@@ -25,6 +26,24 @@ int launch_fill_zero(void *p, size_t bytes, hipStream_t stream);  // clears with
 // Records the next profiling event on `stream` when profiling is enabled (no-op otherwise).
 void profile_mark(int slot, hipStream_t stream, bool stamped = false);
 bool profile_kernel_stamps(int slot, hipEvent_t *start, hipEvent_t *stop);
+// The two events of profile_kernel_stamps on their way to a launcher that takes no events of its
+// own: set by the launcher's caller right before the call and cleared right after it; the one
+// launch made through PQHSA_LAUNCH in between takes them.
+struct LaunchStamps {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+extern LaunchStamps g_launch_stamps;
+bool profile_stamp_next_launch(int slot);
+#define PQHSA_LAUNCH(kern, grid, block, lds, stream, ...)                                                          \
+    do {                                                                                                           \
+        if (::pqhsa::g_launch_stamps.start) {                                                                      \
+            hipExtLaunchKernelGGL(kern, grid, block, (uint32_t)(lds), stream, ::pqhsa::g_launch_stamps.start,      \
+                                  ::pqhsa::g_launch_stamps.stop, 0, __VA_ARGS__);                                  \
+            ::pqhsa::g_launch_stamps = ::pqhsa::LaunchStamps();                                                    \
+        } else {                                                                                                   \
+            hipLaunchKernelGGL(kern, grid, block, lds, stream, __VA_ARGS__);                                       \
+        }                                                                                                          \
+    } while (0)
 enum { kProfLut = 0, kProfSample, kProfEmit, kProfSelect, kProfAttend, kProfKernels };
 
 #define PQHSA_REQUIRE(cond, ...)            \

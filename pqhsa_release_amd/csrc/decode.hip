@@ -219,13 +219,16 @@ static int decode_step_impl(const void *q, int32_t q_dtype, void *out, const pqh
     }
     const pqhsa_index *index_in = index;
     index = &after;
-    profile_mark(kProfLut, stream);
     const bool merged = pqhsa_decode_step_launches(index_in, G, n_max, select, append_count != nullptr) == PQHSA_PROFILE_KERNELS - 1;
+    // (one launch, and the log brackets its slot alone: the launch stamps the slot's two events itself)
+    const bool tables_stamped = merged && profile_stamp_next_launch(kProfLut);
+    profile_mark(kProfLut, stream, tables_stamped);
     if (merged) {  // (the event log books the launch under the table slot)
         rc = decode_tables_thresholds(q, q_dtype, index_in, G, GP, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words, scale,
                                       select, c.thr_key, c.k_row, c.ref_val, append_count ? &ap : nullptr, c.n_after, stream);
+        g_launch_stamps = LaunchStamps();
         if (rc) return rc;
-        profile_mark(kProfSample, stream);
+        profile_mark(kProfSample, stream, tables_stamped);
     } else {
         rc = launch_lut_build(q, q_dtype, index_in, G, eps, c.qnorm, c.lut, c.ls, c.emit_count, c.zero_words,
                               append_count ? &ap : nullptr, c.n_after, c.nearest, stream);

@@ -1529,7 +1529,7 @@ int launch_tables_thresh(TablesArgs p, int q_dtype, SampleArgs a, hipStream_t st
     do {                                                                                            \
         const int rc = raise_lds_limit((const void *)KERNEL_<DT_, R_>, lds, "tables_thresh");       \
         if (rc) return rc;                                                                          \
-        hipLaunchKernelGGL((KERNEL_<DT_, R_>), grid, block, lds, stream, p, a);                     \
+        PQHSA_LAUNCH((KERNEL_<DT_, R_>), grid, block, lds, stream, p, a);                           \
     } while (0)
     if (rows_per_wg == 1) {
         PQHSA_DISPATCH_DTYPE(q_dtype, if (small) PQHSA_TT(tables_thresh_kernel, DT, 4); else PQHSA_TT(tables_thresh_kernel, DT, 8));
@@ -1970,7 +1970,7 @@ static int launch_decode_small_kdt(const SmallArgs &a, int streams, int64_t n_ma
             }                                                                                                    \
             if (dev >= 0 && dev < 64) raised[dev] = lds;                                                         \
         }                                                                                                        \
-        hipLaunchKernelGGL(kern, grid, block, lds, stream, a);                                                   \
+        PQHSA_LAUNCH(kern, grid, block, lds, stream, a);                                                         \
     }
     if (n_max <= 8 * kSelThreads) PQHSA_SMALL(8)
     else PQHSA_SMALL(16)
@@ -2015,9 +2015,12 @@ int decode_small(const void *q, int q_dtype, void *out, const pqhsa_kv_view *kv,
     profile_mark(kProfSample, stream);
     profile_mark(kProfEmit, stream);
     profile_mark(kProfSelect, stream);
-    profile_mark(kProfAttend, stream);
+    // (when the log brackets that slot alone, the launch stamps its two events itself)
+    const bool stamped = profile_stamp_next_launch(kProfAttend);
+    profile_mark(kProfAttend, stream, stamped);
     const int rc = launch_decode_small(a, kv->dtype, index->batch * index->kv_heads, n_max, stream);
-    profile_mark(kProfKernels, stream);
+    g_launch_stamps = LaunchStamps();
+    profile_mark(kProfKernels, stream, stamped);
     return rc;
 }
 
