@@ -481,9 +481,9 @@ int pqhsa_gather_probe(const pqhsa_kv_view *kv, int32_t B, int32_t H, const int3
  * and the number of steps seen, and turns profiling off.
  * pqhsa_profile_only(kernel), called after enable, restricts the log to the two events around
  * one kernel (-1: all), so that a timed run carries two event records per step instead of
- * six; the other entries of kernel_ms are then 0.  For the candidate scan and the attention of
- * the general path those two events are not recorded before and after the launch but handed to
- * the launch itself, which stamps them with the kernel's own start and end (no marker of their
+ * six; the other entries of kernel_ms are then 0.  For the candidate scan, the attention, the
+ * launch that builds tables and thresholds together and the short-context launch those two events
+ * are not recorded before and after the launch but handed to the launch itself, which stamps them with the kernel's own start and end (no marker of their
  * own on the stream; the figure a profiler's kernel trace reports); the environment variable
  * PQHSA_PROFILE_BRACKETS=1 keeps the records around the launch.  pqhsa_profile_every(stride), also after
  * enable, logs one decode step in `stride` (the first, then every stride-th): a timed run then
