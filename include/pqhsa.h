@@ -117,11 +117,12 @@ typedef struct pqhsa_select {
 
 /* pqhsa_decode_step serves short contexts (at most 16 384 indexed keys per sequence, at most 256
  * query rows in the batch, no append in the step) with one kernel, one workgroup per query row;
- * the results are the same.  This flag keeps such a step on the general five-kernel path. */
+ * the results are the same.  This flag keeps such a step on the general path of four or five
+ * launches. */
 #define PQHSA_SELECT_GENERAL_PATH 1
 /* On the general path, asks for the scan, the selection and the exact attention of a step as ONE
  * launch whose workgroups hand work to each other through counters in the workspace (three
- * launches per step instead of five; same results), for batches of sequences of about one length
+ * launches per step instead of four or five; same results), for batches of sequences of about one length
  * (n_mean within an eighth of n_max, or a single sequence) with a GQA group of 3 to 8 query rows;
  * other shapes ignore the flag.  Off by default: on MI355X the three separate launches are
  * faster (the one launch saves two launch gaps and loses more to device-scope memory traffic). */
